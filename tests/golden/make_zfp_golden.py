@@ -1,0 +1,118 @@
+#!/usr/bin/env python3
+"""Regenerates the ZFP golden fixtures in this directory.
+
+The generator is the stock zfp 0.5.5 command-line codec that ships with the
+build image (``/opt/conda/bin/zfp``, serial execution policy).  It is the same
+codec version the reference snapshots (CSWAP+/zfp/version.h:9-15) and is not
+part of the reference tree.  It is only needed to *re*generate; the tests read
+the committed ``zfp_golden.npz`` / ``zfp_digests.json``.
+
+    python tests/golden/make_zfp_golden.py
+
+Fixture contents
+  zfp_golden.npz   small fields: ``<name>/in`` fp32 (nz,ny,nx), and per rate
+                   ``<name>/r<rate>/stream`` (uint8) and ``<name>/r<rate>/dec``.
+  zfp_digests.json SHA-256 of input, stream and decoded output for the large
+                   seeded configurations (inputs are re-created from the seed).
+"""
+import hashlib
+import json
+import os
+import subprocess
+import sys
+import tempfile
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ZFP = os.environ.get("ZFP_CLI", "/opt/conda/bin/zfp")
+
+sys.path.insert(0, os.path.join(HERE, "..", ".."))
+from cswap_amd.workloads import config1_field, config3_fields  # noqa: E402
+
+
+def run_zfp(field: np.ndarray, rate: float):
+    nz, ny, nx = field.shape
+    with tempfile.TemporaryDirectory() as d:
+        fi, fz, fo = (os.path.join(d, n) for n in ("in.f32", "out.zfp", "out.f32"))
+        field.astype("<f4").tofile(fi)
+        subprocess.check_call([ZFP, "-q", "-f", "-3", str(nx), str(ny), str(nz), "-r", repr(rate),
+                               "-i", fi, "-z", fz, "-o", fo])
+        stream = np.fromfile(fz, dtype=np.uint8)
+        dec = np.fromfile(fo, dtype="<f4").reshape(field.shape)
+    return stream, dec
+
+
+def small_fields():
+    rng = np.random.default_rng(1234)
+    f = {}
+    f["rand_8x8x8"] = rng.standard_normal((8, 8, 8)).astype(np.float32)
+    f["one_block"] = rng.standard_normal((4, 4, 4)).astype(np.float32) * 100
+    f["partial_7x5x6"] = rng.standard_normal((7, 5, 6)).astype(np.float32)
+    f["rows_8x4x12"] = np.maximum(rng.standard_normal((8, 4, 12)), 0).astype(np.float32)
+    f["prelu_16x8x8"] = rng.standard_normal((16, 8, 8)).astype(np.float32)
+    f["prelu_16x8x8"] = np.where(f["prelu_16x8x8"] > 0, f["prelu_16x8x8"],
+                                 0.25 * f["prelu_16x8x8"]).astype(np.float32)
+    f["nx2_ny2_8x2x2"] = rng.standard_normal((8, 2, 2)).astype(np.float32)
+    f["odd_4x3x9"] = rng.standard_normal((4, 3, 9)).astype(np.float32)
+    f["single_1x1x1"] = np.array([[[3.25]]], dtype=np.float32)
+    f["line_5x1x3"] = rng.standard_normal((5, 1, 3)).astype(np.float32)
+    z = rng.standard_normal((8, 8, 8)).astype(np.float32)
+    z[0:4, 0:4, 0:4] = 0.0            # an all-zero block
+    z[4:8, 4:8, 4:8] = 7.5            # a constant block
+    z[0:4, 4:8, 0:4] = -0.0           # negative zeros only
+    f["zero_const_blocks"] = z
+    g = np.arange(12, dtype=np.float32)
+    zz, yy, xx = np.meshgrid(g, g, g, indexing="ij")
+    f["smooth_12"] = np.exp(-((xx - 5) ** 2 + (yy - 6) ** 2 + (zz - 4) ** 2) / 30).astype(np.float32)
+    w = rng.standard_normal((4, 8, 8)).astype(np.float32)
+    w *= np.float32(2.0) ** rng.integers(-40, 40, size=w.shape).astype(np.float32)
+    f["wide_range"] = w.astype(np.float32)
+    f["big_small"] = (rng.standard_normal((4, 4, 8)) * np.array([1e30, 1e-30] * 4)).astype(np.float32)
+    s = np.zeros((4, 4, 4), dtype=np.float32)
+    s[1, 2, 3] = -1.0
+    f["single_spike"] = s
+    f["softmax_like"] = (rng.random((4, 8, 16)) ** 8 / 16).astype(np.float32)
+    return f
+
+
+RATES_SMALL = [1, 2.5, 4, 4.5, 8, 9.75, 16, 20, 32]
+RATES_BIG = [4, 8, 16]
+
+
+def sha(a) -> str:
+    return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+
+
+def main():
+    out = {}
+    for name, fld in small_fields().items():
+        out[f"{name}/in"] = fld
+        for r in RATES_SMALL:
+            stream, dec = run_zfp(fld, r)
+            out[f"{name}/r{r}/stream"] = stream
+            out[f"{name}/r{r}/dec"] = dec
+    np.savez_compressed(os.path.join(HERE, "zfp_golden.npz"), **out)
+
+    dig = {}
+    big = {"config1_prelu_4096x32x32": config1_field()}
+    for nm, fld in config3_fields(batch=16).items():
+        big[f"config3_b16_{nm}"] = fld
+    for name, fld in big.items():
+        e = {"shape": list(fld.shape), "input_sha256": sha(fld), "rates": {}}
+        for r in RATES_BIG:
+            stream, dec = run_zfp(fld, r)
+            e["rates"][str(r)] = {
+                "stream_bytes": int(stream.size),
+                "stream_sha256": sha(stream),
+                "decoded_sha256": sha(dec),
+                "max_abs_err": float(np.max(np.abs(dec.astype(np.float64) - fld))),
+            }
+        dig[name] = e
+    with open(os.path.join(HERE, "zfp_digests.json"), "w") as fh:
+        json.dump(dig, fh, indent=1, sort_keys=True)
+    print("wrote", len(out), "arrays and", len(dig), "digest entries")
+
+
+if __name__ == "__main__":
+    main()
