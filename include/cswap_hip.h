@@ -1,0 +1,113 @@
+/*
+ * cswap_hip.h -- C ABI of libcswap_hip.so, the MI355X (gfx950) implementation of
+ * the compression path CSWAP+ puts in front of GPU<->CPU activation swapping.
+ *
+ * Every pointer named d_* is device memory, h_* is host memory.  Every call
+ * that launches work takes the HIP stream to launch on (a hipStream_t passed
+ * as void*; NULL = the default stream) and returns without synchronising.
+ * Return value: CSWAP_OK (0) or a negative CSWAP_E_* code; nothing throws and
+ * nothing is printed.  No entry point allocates device memory unless its
+ * comment says so.
+ *
+ * Each declaration cites the reference interface it stands in for
+ * (paths relative to the reference tree, CSWAP+/...).
+ */
+#ifndef CSWAP_HIP_H
+#define CSWAP_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CSWAP_OK            0
+#define CSWAP_E_ARG        -1  /* null pointer, zero size, size out of range */
+#define CSWAP_E_UNSUPPORTED -2 /* valid request this build does not implement */
+#define CSWAP_E_HIP        -3  /* a HIP runtime call failed (see cswap_last_hip_error) */
+#define CSWAP_E_NOMEM      -4  /* pool or caller-provided buffer too small */
+#define CSWAP_E_STATE      -5  /* call out of order (e.g. swap-in before swap-out) */
+
+typedef void* cswap_stream_t; /* hipStream_t */
+
+const char* cswap_strerror(int code);
+int         cswap_last_hip_error(void); /* hipError_t of the last CSWAP_E_HIP on this thread */
+int         cswap_abi_version(void);
+
+/* ------------------------------------------------------------------ ZFP -----
+ * Fixed-rate ZFP of a 3-D fp32 field a[nz][ny][nx] (x fastest).  Strides are in
+ * elements; 0 means the contiguous default (sx=1, sy=nx, sz=nx*ny), as in
+ * zfp/cuZFP.cu:372-375.  maxbits = bits per 4x4x4 block (64 * bits-per-value),
+ * 16 <= maxbits <= 4096; block b owns stream bits [b*maxbits, (b+1)*maxbits)
+ * (zfp/encode.cuh:229-230), blocks numbered x fastest (zfp/encode3.cuh:79-87).
+ */
+
+/* Stream size the reference reports: whole 64-bit words, rounded down
+ * (zfp/encode3.cuh:147, zfp/shared.h:73-84). */
+size_t cswap_zfp_stream_bytes(size_t nx, size_t ny, size_t nz, unsigned maxbits);
+/* Bytes the stream buffer must hold: whole words, rounded up.  Equal to the
+ * above whenever blocks*maxbits is a multiple of 64. */
+size_t cswap_zfp_stream_capacity(size_t nx, size_t ny, size_t nz, unsigned maxbits);
+
+/* Replaces cuZFP::encode<float> / encode3launch (zfp/encode3.cuh:117-199) as
+ * reached from cuda_compress (zfp/cuZFP.cu:364-436).  Writes every word of the
+ * stream (no prior memset needed). */
+int cswap_zfp_compress_f32(const float* d_in, size_t nx, size_t ny, size_t nz,
+                           ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
+                           uint64_t* d_stream, cswap_stream_t stream);
+
+/* Replaces cuZFP::decode3<float> (zfp/decode3.cuh:108-187) as reached from
+ * cuda_decompress (zfp/cuZFP.cu:440-532).  Writes every element of the field. */
+int cswap_zfp_decompress_f32(const uint64_t* d_stream, size_t nx, size_t ny, size_t nz,
+                             ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
+                             float* d_out, cswap_stream_t stream);
+
+/* ------------------------------------------------------------------ ZVC -----
+ * Zero-value compaction in the reference's format (zfp/compression.cu).  The
+ * tensor of n fp32 elements is cut into `process` chunks of
+ * E = ceil(n/process) elements (the reference uses process = 512*32,
+ * Execution.h:50-52); chunk i owns W = ceil(E/32) mask words starting at word
+ * i*W, bit k%32 of word k/32 set iff element E*i+k != 0, and its non-zeros
+ * start at d_values[d_begin[i]].  0 < n < 2^31, 0 < process <= 2^20.
+ */
+int    cswap_zvc_chunk_elems(int n, int process);   /* E */
+int    cswap_zvc_chunk_words(int n, int process);   /* W */
+int    cswap_zvc_active_chunks(int n, int process); /* chunks that hold data = ceil(n/E) */
+size_t cswap_zvc_mask_bytes(int n, int process);    /* W*process*4, Execution.h:88 */
+
+/* Replaces PreGPUcompression (zfp/compression.cu:134-165, launcher :334-341):
+ * d_count[i] = number of elements != 0 in chunk i, for the active chunks. */
+int cswap_zvc_count(const float* d_in, int n, int process, int* d_count, cswap_stream_t stream);
+
+/* Replaces PreAcc (zfp/compression.cu:9-19, launcher :342-350): in-place
+ * exclusive prefix sum over the first k entries; *d_nnz = total. */
+int cswap_zvc_scan(int* d_count, int k, int* d_nnz, cswap_stream_t stream);
+
+/* Replaces GPUcompression (zfp/compression.cu:168-239, launcher :351-365).
+ * d_values must hold nnz floats, d_mask cswap_zvc_mask_bytes(n,process).  Every
+ * mask word is written (words the reference leaves untouched are zeroed). */
+int cswap_zvc_compact(const float* d_in, int n, int process, const int* d_begin,
+                      float* d_values, uint32_t* d_mask, cswap_stream_t stream);
+
+/* Replaces GPUdecompression (zfp/compression.cu:241-318, launcher :367-374).
+ * Unlike the reference it writes all n outputs (zeros as +0.0) and needs no
+ * pre-zeroed destination. */
+int cswap_zvc_expand(const float* d_values, const uint32_t* d_mask, const int* d_begin,
+                     int n, int process, float* d_out, cswap_stream_t stream);
+
+/* count + scan + compact in one call with no host round trip (the reference
+ * copies nnz to the host between the steps, Execution.h:89-95).  d_values must
+ * hold n floats (worst case); *d_nnz receives the total. */
+int cswap_zvc_compress(const float* d_in, int n, int process, int* d_begin, int* d_nnz,
+                       float* d_values, uint32_t* d_mask, cswap_stream_t stream);
+
+/* ---------------------------------------------------------------- probe -----
+ * One fused read pass: *d_nnz = number of elements != 0 (the quantity the
+ * reference derives from PreGPUcompression + PreAcc, Execution.h:89-92). */
+int cswap_probe_nnz(const float* d_in, size_t n, unsigned long long* d_nnz, cswap_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CSWAP_HIP_H */

@@ -1,0 +1,131 @@
+"""GPU parity of zero-value compaction: bit-exact mask, packed values, chunk
+offsets and reconstruction against the CPU checker and numpy."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+P = 512 * 32
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return torch
+
+
+def run_gpu(torch, x, process=P):
+    from cswap_amd import api
+
+    t = torch.from_numpy(x).cuda()
+    values, mask, begin, nnz = api.zvc_compress(t, process)
+    out = torch.full_like(t, -1.0)                      # NOT pre-zeroed on purpose
+    api.GPUdecompression(values, out, mask, begin, process)
+    probe = api.probe_nnz(t)
+    torch.cuda.synchronize()
+    k = int(nnz.item())
+    return (values[:k].cpu().numpy(), mask.cpu().numpy().view(np.uint32), begin.cpu().numpy(), k,
+            out.cpu().numpy(), int(probe.item()))
+
+
+def check_against_oracle(x, got, process=P):
+    import oracle
+
+    vals, mask, begin, nnz = oracle.zvc_compress(x, process)
+    gv, gm, gb, gk, gout, gprobe = got
+    assert gk == nnz == gprobe == np.count_nonzero(x)
+    assert np.array_equal(gv.view(np.uint32), vals.view(np.uint32))
+    assert np.array_equal(gm, mask)
+    E, W, K = oracle.zvc_geometry(x.size, process)
+    assert np.array_equal(gb[:K], begin[:K])
+    want = np.where(x != 0, x, np.float32(0))
+    assert np.array_equal(gout.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("pct", [30, 50, 70, 90])
+def test_config2_sparsity_sweep(torch_cuda, pct):
+    from cswap_amd.workloads import config2_tensor
+
+    x = config2_tensor(pct).reshape(-1)
+    got = run_gpu(torch_cuda, x)
+    check_against_oracle(x, got)
+    assert np.array_equal(got[1].view(np.uint8), np.packbits(x != 0, bitorder="little"))
+
+
+@pytest.mark.parametrize("n", [1, 31, 33, 64, 1000, P - 1, P, P + 1, 1_000_003, P * 62 + 17, P * 64, P * 96 + 5])
+def test_ragged_sizes(torch_cuda, n):
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * (rng.random(n) < 0.4)).astype(np.float32)
+    print("n", n, flush=True)
+    check_against_oracle(x, run_gpu(torch_cuda, x))
+
+
+@pytest.mark.parametrize("process", [1, 7, 64, 4096])
+def test_other_chunk_counts(torch_cuda, process):
+    rng = np.random.default_rng(process)
+    x = np.maximum(rng.standard_normal(300_001), 0).astype(np.float32)
+    check_against_oracle(x, run_gpu(torch_cuda, x, process), process)
+
+
+def test_special_values_and_extremes(torch_cuda):
+    n = P * 64
+    x = np.zeros(n, dtype=np.float32)
+    x[[3, 10, 11, 12, 13, 70]] = [-0.0, np.nan, np.inf, -np.inf, 1e-45, -2.5]
+    got = run_gpu(torch_cuda, x)
+    assert got[3] == 5
+    assert np.array_equal(got[0].view(np.uint32), x[[10, 11, 12, 13, 70]].view(np.uint32))
+    want = x.copy(); want[3] = 0.0
+    assert np.array_equal(got[4].view(np.uint32), want.view(np.uint32))
+    check_against_oracle(np.zeros(n, np.float32), run_gpu(torch_cuda, np.zeros(n, np.float32)))
+    check_against_oracle(np.arange(1, n + 1, dtype=np.float32),
+                         run_gpu(torch_cuda, np.arange(1, n + 1, dtype=np.float32)))
+
+
+def test_reference_call_sequence(torch_cuda):
+    """The four launchers in the order CSWAP+/Execution.h:88-95 calls them, with a
+    host read of nnz in between, produce what the one-call path produces."""
+    torch = torch_cuda
+    from cswap_amd import api
+    from cswap_amd.workloads import config2_tensor
+
+    x = config2_tensor(70, shape=(32, 256, 16, 16)).reshape(-1)
+    t = torch.from_numpy(x).cuda()
+    n = t.numel()
+    E, W, K = api.zvc_geometry(n)
+    index_begin = torch.zeros(P, dtype=torch.int32, device="cuda")
+    num = torch.zeros(1, dtype=torch.int32, device="cuda")
+    api.PreGPUcompression(t, index_begin)
+    api.PreAcc(index_begin, K, num)
+    nnz = int(num.item())
+    values = torch.empty(nnz, dtype=torch.float32, device="cuda")
+    mask = torch.empty(W * P, dtype=torch.int32, device="cuda")
+    api.GPUcompression(t, values, index_begin, mask)
+    dest = torch.empty_like(t)
+    api.GPUdecompression(values, dest, mask, index_begin)
+    torch.cuda.synchronize()
+    assert torch.equal(dest, t)
+    assert nnz == np.count_nonzero(x)
+    assert np.array_equal(values.cpu().numpy(), x[x != 0])
+
+
+def test_full_size_round_trip(torch_cuda):
+    """256 MiB tensor: properties instead of the checker -- round trip, nnz,
+    monotone chunk offsets, mask popcount == nnz."""
+    torch = torch_cuda
+    from cswap_amd import api
+
+    g = torch.Generator(device="cuda"); g.manual_seed(1)
+    t = torch.relu(torch.randn(64 * 1024 * 1024, generator=g, device="cuda"))
+    values, mask, begin, nnz = api.zvc_compress(t)
+    out = torch.full_like(t, 3.0)
+    api.GPUdecompression(values, out, mask, begin)
+    torch.cuda.synchronize()
+    assert torch.equal(out, t)
+    k = int(nnz.item())
+    assert k == int((t != 0).sum().item()) == int(api.probe_nnz(t).item())
+    b = begin.cpu().numpy()
+    assert b[0] == 0 and np.all(np.diff(b) >= 0) and b[-1] <= k
+    m = mask.cpu().numpy().view(np.uint8)
+    assert int(np.unpackbits(m).sum()) == k
+    assert torch.equal(values[:k], t[t != 0])
