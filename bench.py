@@ -1,0 +1,245 @@
+#!/usr/bin/env python3
+"""Benchmark of the compression-before-swap hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one pass of the hot path over one synthetic batch: ZFP fixed-rate
+8 bits/value compress followed by decompress of the BERT-base attention
+probability tensor fp32 [32,12,512,512] (402,653,184 B; the >=256 MB tensor the
+throughput target is quoted on), already resident in HBM.  ``value`` is GB/s of
+uncompressed fp32 pushed through the compress+decompress pair:
+4*N bytes / (t_compress + t_decompress).
+
+The single JSON line also carries
+  roofline      HBM-roofline figures of the dominant (slower) ZFP kernel, from
+                HIP-event timing of that kernel inside the timed region
+  cpu_baseline  the CPU checker (a port of the reference algorithm) timed on a
+                bounded sample of the same tensor on this host
+  extra         the other kernels of the path (ZVC compact/expand, probe, other
+                rates, swap latency) -- reported, not the headline.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+
+def ev_ms(torch, fn, reps):
+    """Average duration of fn() in ms from HIP events on the current stream."""
+    a = torch.cuda.Event(enable_timing=True)
+    b = torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    b.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-extra", action="store_true", help="headline workload only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path is built and measured on ONE GPU; run with --gpus 1 "
+              "(DESIGN.md says how it would shard)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from cswap_amd import api
+    from cswap_amd.workloads import CONFIG5_SHAPES, config5_tensor_torch, field_dims
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    rate = 8
+    maxbits = 64 * rate
+    name = "attn_softmax"
+    x = config5_tensor_torch(name, dev, seed=0)
+    n = x.numel()
+    nx, ny, nz = field_dims(x.shape)
+    stream = torch.empty(api.zfp_stream_capacity(nx, ny, nz, maxbits), dtype=torch.uint8, device=dev)
+    out = torch.empty_like(x)
+
+    def step():
+        api.cuda_compress(x, maxbits, out=stream)
+        api.cuda_decompress(stream, x.shape, maxbits, out=out)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    # ---- timed region: exactly K steps, per-kernel HIP events inside it
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        evs[k][0].record()
+        api.cuda_compress(x, maxbits, out=stream)
+        evs[k][1].record()
+        api.cuda_decompress(stream, x.shape, maxbits, out=out)
+        evs[k][2].record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    enc_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
+    dec_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps
+    value = 4.0 * n / (ms_per_step * 1e-3) / 1e9
+
+    bytes_per_value = 4.0 + rate / 8.0          # read 4 B, write rate/8 B (or the reverse)
+    dom = "zfp_encode3_f32_kernel" if enc_ms >= dec_ms else "zfp_decode3_f32_kernel"
+    dom_ms = max(enc_ms, dec_ms)
+    achieved = bytes_per_value * n / (dom_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "algorithmic_bytes_per_launch": int(bytes_per_value * n),
+                "avg_launch_ms": round(dom_ms, 4),
+                "compress_ms": round(enc_ms, 4), "decompress_ms": round(dec_ms, 4),
+                "compress_frac": round(bytes_per_value * n / (enc_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                "decompress_frac": round(bytes_per_value * n / (dec_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(traffic_file):
+        try:
+            roofline["traffic"] = json.load(open(traffic_file)).get(dom)
+        except Exception:
+            pass
+
+    result = {
+        "metric": "compress+decompress GB/s (fp32 in), ZFP fixed-rate 8 bits/value, 1xMI355X",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32->i32/u64 bit planes", "data": "synthetic",
+        "config": {"workload": "config5 attention probabilities fp32 [32,12,512,512] = softmax(N(0,1)), "
+                               "zfp field nx=512 ny=512 nz=384, rate 8 (maxbits 512), compress then decompress",
+                   "bytes_in": 4 * n, "rate_bits_per_value": rate},
+        "roofline": roofline,
+    }
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(x, maxbits)
+    if not args.no_extra:
+        result["extra"] = extras(torch, api, dev)
+    print(json.dumps(result))
+
+
+def cpu_baseline(x, maxbits):
+    """The CPU checker (port of the reference algorithm) on a bounded sample:
+    the first 4 of the 32 batch entries (50 MB) of the same tensor."""
+    import numpy as np
+
+    import oracle
+
+    sample = x[:4].cpu().numpy().reshape(-1, x.shape[-2], x.shape[-1])
+    nbytes = sample.nbytes
+
+    def pair(omp):
+        best = None
+        for _ in range(3):
+            t0 = time.perf_counter()
+            s = oracle.zfp_encode3(sample, maxbits, omp=omp)
+            t1 = time.perf_counter()
+            oracle.zfp_decode3(s, sample.shape, maxbits, omp=omp)
+            t2 = time.perf_counter()
+            cur = (t2 - t0, t1 - t0, t2 - t1)
+            best = cur if best is None or cur[0] < best[0] else best
+        return best
+
+    ser = pair(False)
+    par = pair(True)
+    threads = oracle.lib(True).orc_threads()
+    return {"value": round(nbytes / ser[0] / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "first 4 of 32 batch entries (50.3 MB) of the same tensor, compress+decompress, best of 3",
+            "compress_GBs": round(nbytes / ser[1] / 1e9, 4), "decompress_GBs": round(nbytes / ser[2] / 1e9, 4),
+            "all_cores": {"value": round(nbytes / par[0] / 1e9, 4), "cores": threads}}
+
+
+def extras(torch, api, dev):
+    import numpy as np
+
+    from cswap_amd.workloads import config1_field, config2_tensor, field_dims
+
+    ex = {}
+    # ---- ZFP at other rates and on configuration 1
+    g = torch.Generator(device=dev); g.manual_seed(0)
+    big = torch.softmax(torch.randn((32, 12, 512, 512), generator=g, device=dev), dim=-1).contiguous()
+    c1 = torch.from_numpy(config1_field()).to(dev)
+    for label, t in (("attn_402MB", big), ("config1_16MB", c1)):
+        n = t.numel()
+        nx, ny, nz = field_dims(t.shape)
+        for rate in (4, 8, 16):
+            mb = 64 * rate
+            s = torch.empty(api.zfp_stream_capacity(nx, ny, nz, mb), dtype=torch.uint8, device=dev)
+            o = torch.empty_like(t)
+            api.cuda_compress(t, mb, out=s); api.cuda_decompress(s, t.shape, mb, out=o)
+            reps = 10 if n > 1 << 24 else 50
+            e = ev_ms(torch, lambda: api.cuda_compress(t, mb, out=s), reps)
+            d = ev_ms(torch, lambda: api.cuda_decompress(s, t.shape, mb, out=o), reps)
+            bpv = 4 + rate / 8
+            ex[f"zfp_{label}_r{rate}"] = {
+                "compress_ms": round(e, 4), "decompress_ms": round(d, 4),
+                "compress_GBs_fp32": round(4 * n / e / 1e6, 1), "decompress_GBs_fp32": round(4 * n / d / 1e6, 1),
+                "compress_hbm_frac": round(bpv * n / e / 1e6 / HBM_PEAK_GBS, 4),
+                "decompress_hbm_frac": round(bpv * n / d / 1e6 / HBM_PEAK_GBS, 4)}
+    del big
+
+    # ---- ZVC compact / expand / probe
+    def zvc_case(label, t):
+        n = t.numel()
+        values, mask, begin, nnz = api.zvc_compress(t)
+        o = torch.empty_like(t)
+        api.GPUdecompression(values, o, mask, begin)
+        torch.cuda.synchronize()
+        k = int(nnz.item())
+        dens = k / n
+        reps = 10 if n > 1 << 24 else 50
+        from cswap_amd._lib import lib
+        L = lib()
+        st = torch.cuda.current_stream().cuda_stream
+        full = ev_ms(torch, lambda: L.cswap_zvc_compress(t.data_ptr(), n, api.PROCESS, begin.data_ptr(),
+                                                         nnz.data_ptr(), values.data_ptr(), mask.data_ptr(), st), reps)
+        cnt = torch.zeros(api.PROCESS, dtype=torch.int32, device=dev)
+        count = ev_ms(torch, lambda: L.cswap_zvc_count(t.data_ptr(), n, api.PROCESS, cnt.data_ptr(), st), reps)
+        compact = ev_ms(torch, lambda: L.cswap_zvc_compact(t.data_ptr(), n, api.PROCESS, begin.data_ptr(),
+                                                           values.data_ptr(), mask.data_ptr(), st), reps)
+        expand = ev_ms(torch, lambda: api.GPUdecompression(values, o, mask, begin), reps)
+        pr = torch.zeros(1, dtype=torch.int64, device=dev)
+        probe = ev_ms(torch, lambda: api.probe_nnz(t, out=pr), reps)
+        bpv = 4 + 1 / 8 + 4 * dens
+        ex[f"zvc_{label}"] = {
+            "density": round(dens, 4), "ratio": round((4 * k + n / 8 + 4 * api.PROCESS) / (4 * n), 4),
+            "count_ms": round(count, 4), "compact_ms": round(compact, 4), "compress_total_ms": round(full, 4),
+            "expand_ms": round(expand, 4), "probe_ms": round(probe, 4),
+            "compact_GBs_fp32": round(4 * n / compact / 1e6, 1), "expand_GBs_fp32": round(4 * n / expand / 1e6, 1),
+            "compact_hbm_frac": round(bpv * n / compact / 1e6 / HBM_PEAK_GBS, 4),
+            "compress_total_hbm_frac": round(bpv * n / full / 1e6 / HBM_PEAK_GBS, 4),
+            "expand_hbm_frac": round(bpv * n / expand / 1e6 / HBM_PEAK_GBS, 4),
+            "probe_hbm_frac": round(4 * n / probe / 1e6 / HBM_PEAK_GBS, 4)}
+
+    for pct in (30, 50, 70, 90):
+        zvc_case(f"config2_s{pct}", torch.from_numpy(config2_tensor(pct)).to(dev))
+    g = torch.Generator(device=dev); g.manual_seed(1)
+    zvc_case("relu_256MiB", torch.relu(torch.randn(64 * 1024 * 1024, generator=g, device=dev)))
+
+    try:
+        from cswap_amd import swap
+        ex["swap"] = swap.bench_schedule(dev)
+    except ImportError:
+        pass
+    return ex
+
+
+if __name__ == "__main__":
+    main()
