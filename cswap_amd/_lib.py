@@ -23,6 +23,47 @@ _lib = None
 
 vp, sz, pd, u, i32 = C.c_void_p, C.c_size_t, C.c_ssize_t, C.c_uint, C.c_int
 
+
+class Costs(C.Structure):
+    _fields_ = [("bw_d2h_gbs", C.c_double), ("bw_h2d_gbs", C.c_double), ("copy_latency_us", C.c_double),
+                ("kernel_latency_us", C.c_double), ("zvc_compress_gbs", C.c_double),
+                ("zvc_expand_gbs", C.c_double), ("zfp_compress_gbs", C.c_double),
+                ("zfp_decompress_gbs", C.c_double), ("sparse_max_ratio", C.c_double), ("lossy_min_gain", C.c_double),
+                ("size_floor_bytes", C.c_size_t), ("allow_lossy", C.c_int), ("process", C.c_int)]
+
+
+class Choice(C.Structure):
+    _fields_ = [("policy", C.c_int), ("bytes_out", C.c_size_t), ("ratio", C.c_double),
+                ("t_none_us", C.c_double), ("t_sparse_us", C.c_double), ("t_zfp_us", C.c_double)]
+
+
+class EngineConfig(C.Structure):
+    _fields_ = [("pinned_pool_bytes", C.c_size_t), ("device_pool_bytes", C.c_size_t), ("process", C.c_int),
+                ("zfp_maxbits", C.c_uint), ("max_tickets", C.c_int), ("costs", Costs)]
+
+
+class TicketInfo(C.Structure):
+    _fields_ = [("policy", C.c_int), ("n", C.c_size_t), ("nnz", C.c_size_t), ("bytes_in", C.c_size_t),
+                ("bytes_out", C.c_size_t), ("state", C.c_int)]
+
+
+class ZfpBitstream(C.Structure):
+    _fields_ = [("bits", C.c_uint), ("buffer", C.c_uint64), ("ptr", C.c_void_p), ("begin", C.c_void_p),
+                ("end", C.c_void_p)]
+
+
+class ZfpStream(C.Structure):
+    _fields_ = [("minbits", C.c_uint), ("maxbits", C.c_uint), ("maxprec", C.c_uint), ("minexp", C.c_int),
+                ("stream", C.POINTER(ZfpBitstream)), ("exec_policy", C.c_int), ("omp_threads", C.c_uint),
+                ("omp_chunk", C.c_uint)]
+
+
+class ZfpField(C.Structure):
+    _fields_ = [("type", C.c_int), ("nx", C.c_size_t), ("ny", C.c_size_t), ("nz", C.c_size_t),
+                ("nw", C.c_size_t), ("sx", C.c_ssize_t), ("sy", C.c_ssize_t), ("sz", C.c_ssize_t),
+                ("sw", C.c_ssize_t), ("data", C.c_void_p)]
+
+
 _SIGNATURES = {
     "cswap_strerror": (C.c_char_p, [i32]),
     "cswap_last_hip_error": (i32, []),
@@ -41,6 +82,31 @@ _SIGNATURES = {
     "cswap_zvc_expand": (i32, [vp, vp, vp, i32, i32, vp, vp]),
     "cswap_zvc_compress": (i32, [vp, i32, i32, vp, vp, vp, vp, vp]),
     "cswap_probe_nnz": (i32, [vp, sz, vp, vp]),
+    "cswap_costs_default": (None, [C.POINTER(Costs)]),
+    "cswap_policy_bytes": (sz, [i32, sz, sz, u, i32, sz, sz, sz]),
+    "cswap_select": (i32, [sz, sz, u, C.POINTER(Costs), C.POINTER(Choice)]),
+    "cswap_engine_config_default": (None, [C.POINTER(EngineConfig)]),
+    "cswap_engine_create": (i32, [C.POINTER(vp), C.POINTER(EngineConfig)]),
+    "cswap_engine_destroy": (None, [vp]),
+    "cswap_swap_out": (i32, [vp, vp, sz, sz, sz, i32, vp, C.POINTER(i32)]),
+    "cswap_swap_wait": (i32, [vp, i32]),
+    "cswap_swap_in": (i32, [vp, i32, vp, vp]),
+    "cswap_swap_release": (i32, [vp, i32]),
+    "cswap_swap_info": (i32, [vp, i32, C.POINTER(TicketInfo)]),
+    "cswap_engine_calibrate": (i32, [vp, C.POINTER(Costs)]),
+    "cswap_engine_copy_stream": (vp, [vp]),
+    # the reference's own entry-point names (include/cswap_compat.h)
+    "PreGPUcompression": (None, [i32, i32, vp, vp, i32, i32, vp]),
+    "PreAcc": (None, [vp, i32, vp, i32, i32, vp]),
+    "GPUcompression": (None, [i32, i32, vp, vp, vp, vp, i32, i32, vp]),
+    "GPUdecompression": (None, [vp, vp, i32, i32, vp, vp, i32, i32]),
+    "cuda_compress": (sz, [C.POINTER(ZfpStream), C.POINTER(ZfpField)]),
+    "cuda_decompress": (None, [C.POINTER(ZfpStream), C.POINTER(ZfpField)]),
+    "setRatio": (None, [i32]),
+    "compress": (vp, [vp, C.c_longlong, C.POINTER(sz)]),
+    "decompress": (i32, [vp, C.c_longlong, vp]),
+    "cswap_set_allocator": (None, [vp, vp]),
+    "cswap_compat_set_field": (None, [sz, sz]),
 }
 
 

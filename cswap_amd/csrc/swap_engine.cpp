@@ -1,0 +1,528 @@
+// swap_engine.cpp -- compressed swap-out / swap-in through pinned host memory.
+//
+// Mirrors Execution::init_/pre/post of the reference (CSWAP+/Execution.h:46-133,
+// 217-310) and the backward-side swap-in it keeps in a patched autograd engine:
+//   swap_out  = pre  : (probe, select,) compress on the compute stream, then an
+//                      async device-to-host copy on a dedicated copy stream
+//   swap_wait = post : wait for that copy; the device tensor may then be freed
+//   swap_in          : async host-to-device copy on the copy stream, then
+//                      decompress on the compute stream
+// Differences by design: copies are ordered against kernels with events instead
+// of device-wide synchronisation (the reference's ZFP path runs on the default
+// stream between two cudaDeviceSynchronize calls, CSWAP+/zfp/cuZFP.cu:393-399);
+// pinned and staging memory come from pools created once (the reference calls
+// the pinned allocator per tensor, Execution.h:76,97-99,114); several tensors
+// can be in flight at once (the reference has one dataptr_/buffer per Execution,
+// Execution.h:432-441).
+#include <map>
+#include <mutex>
+#include <new>
+#include <vector>
+
+#include "common.h"
+
+namespace {
+
+using cswap::hip_fail;
+
+// First-fit free-list allocator over one region; offsets are 256-byte aligned.
+class Pool {
+ public:
+  void reset(size_t size)
+  {
+    free_.clear();
+    size_ = size;
+    if (size) free_[0] = size;
+  }
+  static size_t round(size_t b) { return (b + 255) & ~(size_t)255; }
+  bool alloc(size_t bytes, size_t* off)
+  {
+    bytes = round(bytes ? bytes : 1);
+    for (auto it = free_.begin(); it != free_.end(); ++it) {
+      if (it->second >= bytes) {
+        *off = it->first;
+        size_t rest = it->second - bytes;
+        size_t o = it->first;
+        free_.erase(it);
+        if (rest) free_[o + bytes] = rest;
+        return true;
+      }
+    }
+    return false;
+  }
+  void free(size_t off, size_t bytes)
+  {
+    bytes = round(bytes ? bytes : 1);
+    auto it = free_.emplace(off, bytes).first;
+    auto nx = std::next(it);
+    if (nx != free_.end() && it->first + it->second == nx->first) {
+      it->second += nx->second;
+      free_.erase(nx);
+    }
+    if (it != free_.begin()) {
+      auto pv = std::prev(it);
+      if (pv->first + pv->second == it->first) {
+        pv->second += it->second;
+        free_.erase(it);
+      }
+    }
+  }
+  // give back the tail of an allocation
+  void shrink(size_t off, size_t old_bytes, size_t new_bytes)
+  {
+    size_t o = round(old_bytes ? old_bytes : 1), n = round(new_bytes ? new_bytes : 1);
+    if (n < o) free(off + n, o - n);
+  }
+  size_t largest_free() const
+  {
+    size_t m = 0;
+    for (auto& kv : free_) m = kv.second > m ? kv.second : m;
+    return m;
+  }
+
+ private:
+  std::map<size_t, size_t> free_;
+  size_t size_ = 0;
+};
+
+enum TicketState { kFree = 0, kOutInFlight = 1, kOnHost = 2, kInInFlight = 3 };
+
+struct Ticket {
+  int state = kFree;
+  int policy = CSWAP_POLICY_NONE;
+  size_t n = 0, nnz = 0, nx = 0, ny = 0, nz = 0;
+  size_t bytes_out = 0;
+  size_t host_off = 0, host_bytes = 0;
+  size_t dev_off = 0, dev_bytes = 0;
+  bool dev_held = false;
+  hipEvent_t ev_ready = nullptr;  // compute stream: compressed data / destination ready
+  hipEvent_t ev_copy = nullptr;   // copy stream: transfer finished
+  hipEvent_t ev_done = nullptr;   // compute stream: decompression finished
+};
+
+}  // namespace
+
+struct cswap_engine {
+  std::mutex mu;
+  hipStream_t copy = nullptr;
+  char* h_base = nullptr;
+  char* d_base = nullptr;
+  Pool hpool, dpool;
+  std::vector<Ticket> tickets;
+  cswap_costs costs;
+  int process = 512 * 32;
+  unsigned maxbits = 512;
+  int* h_nnz = nullptr;  // pinned, 1 int
+  int* d_nnz = nullptr;
+  hipEvent_t ev_probe = nullptr;
+  int device = 0;
+};
+
+// layout of a ZVC payload: [begin: process ints][mask][values: nnz floats]
+static size_t zvc_header_bytes(int n, int process) { return 4 * (size_t)process + cswap_zvc_mask_bytes(n, process); }
+
+extern "C" void cswap_engine_config_default(cswap_engine_config* cfg)
+{
+  if (!cfg) return;
+  cfg->pinned_pool_bytes = (size_t)1 << 30;
+  cfg->device_pool_bytes = (size_t)1 << 30;
+  cfg->process = 512 * 32;
+  cfg->zfp_maxbits = 512;
+  cfg->max_tickets = 256;
+  cswap_costs_default(&cfg->costs);
+}
+
+extern "C" void cswap_engine_destroy(cswap_engine* e)
+{
+  if (!e) return;
+  if (e->copy) (void)hipStreamSynchronize(e->copy);
+  for (auto& t : e->tickets) {
+    if (t.ev_ready) (void)hipEventDestroy(t.ev_ready);
+    if (t.ev_copy) (void)hipEventDestroy(t.ev_copy);
+    if (t.ev_done) (void)hipEventDestroy(t.ev_done);
+  }
+  if (e->ev_probe) (void)hipEventDestroy(e->ev_probe);
+  if (e->h_nnz) (void)hipHostFree(e->h_nnz);
+  if (e->d_nnz) (void)hipFree(e->d_nnz);
+  if (e->h_base) (void)hipHostFree(e->h_base);
+  if (e->d_base) (void)hipFree(e->d_base);
+  if (e->copy) (void)hipStreamDestroy(e->copy);
+  delete e;
+}
+
+extern "C" int cswap_engine_create(cswap_engine** out, const cswap_engine_config* cfg_in)
+{
+  if (!out) return CSWAP_E_ARG;
+  cswap_engine_config cfg;
+  if (cfg_in) cfg = *cfg_in; else cswap_engine_config_default(&cfg);
+  if (!cfg.pinned_pool_bytes || !cfg.device_pool_bytes) return CSWAP_E_ARG;
+  if (cfg.process == 0) cfg.process = 512 * 32;
+  if (cfg.zfp_maxbits == 0) cfg.zfp_maxbits = 512;
+  if (cfg.max_tickets <= 0) cfg.max_tickets = 256;
+  if (cfg.process < 0 || cfg.process > (1 << 20) || cfg.zfp_maxbits < 16 || cfg.zfp_maxbits > 4096)
+    return CSWAP_E_ARG;
+  if (cfg.costs.bw_d2h_gbs <= 0 || cfg.costs.bw_h2d_gbs <= 0) cswap_costs_default(&cfg.costs);
+  cfg.costs.process = cfg.process;
+
+  cswap_engine* e = new (std::nothrow) cswap_engine;
+  if (!e) return CSWAP_E_NOMEM;
+  e->costs = cfg.costs;
+  e->process = cfg.process;
+  e->maxbits = cfg.zfp_maxbits;
+  int rc = CSWAP_OK;
+  auto fail = [&](hipError_t err) { rc = hip_fail(err); };
+  hipError_t err;
+  do {
+    if ((err = hipGetDevice(&e->device)) != hipSuccess) { fail(err); break; }
+    // default priority on purpose; non-blocking so it never serialises with the null stream
+    if ((err = hipStreamCreateWithFlags(&e->copy, hipStreamNonBlocking)) != hipSuccess) { fail(err); break; }
+    if ((err = hipHostMalloc((void**)&e->h_base, cfg.pinned_pool_bytes, hipHostMallocDefault)) != hipSuccess) { fail(err); break; }
+    if ((err = hipMalloc((void**)&e->d_base, cfg.device_pool_bytes)) != hipSuccess) { fail(err); break; }
+    if ((err = hipHostMalloc((void**)&e->h_nnz, 256, hipHostMallocDefault)) != hipSuccess) { fail(err); break; }
+    if ((err = hipMalloc((void**)&e->d_nnz, 256)) != hipSuccess) { fail(err); break; }
+    if ((err = hipEventCreateWithFlags(&e->ev_probe, hipEventDisableTiming)) != hipSuccess) { fail(err); break; }
+    e->hpool.reset(cfg.pinned_pool_bytes);
+    e->dpool.reset(cfg.device_pool_bytes);
+    e->tickets.resize((size_t)cfg.max_tickets);
+    for (auto& t : e->tickets) {
+      if ((err = hipEventCreateWithFlags(&t.ev_ready, hipEventDisableTiming)) != hipSuccess) break;
+      if ((err = hipEventCreateWithFlags(&t.ev_copy, hipEventDisableTiming)) != hipSuccess) break;
+      if ((err = hipEventCreateWithFlags(&t.ev_done, hipEventDisableTiming)) != hipSuccess) break;
+    }
+    if (err != hipSuccess) { fail(err); break; }
+  } while (0);
+  if (rc) { cswap_engine_destroy(e); return rc; }
+  *out = e;
+  return CSWAP_OK;
+}
+
+extern "C" cswap_stream_t cswap_engine_copy_stream(cswap_engine* e) { return e ? (cswap_stream_t)e->copy : nullptr; }
+
+static void drop_device(cswap_engine* e, Ticket& t)
+{
+  if (t.dev_held) {
+    e->dpool.free(t.dev_off, t.dev_bytes);
+    t.dev_held = false;
+  }
+}
+
+extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, size_t ny, size_t nz, int policy,
+                              cswap_stream_t compute_, int* ticket)
+{
+  if (!e || !d_in || !ticket || !nx || !ny || !nz) return CSWAP_E_ARG;
+  if (policy != CSWAP_POLICY_AUTO && policy != CSWAP_POLICY_NONE && policy != CSWAP_POLICY_SPARSE &&
+      policy != CSWAP_POLICY_ZFP)
+    return CSWAP_E_ARG;
+  hipStream_t compute = (hipStream_t)compute_;
+  std::lock_guard<std::mutex> lock(e->mu);
+  const size_t n = nx * ny * nz;
+  if (n / nz != nx * ny) return CSWAP_E_ARG;
+  const bool zvc_ok = n <= 0x7fffffffull;
+  if (policy == CSWAP_POLICY_SPARSE && !zvc_ok) return CSWAP_E_ARG;
+
+  int id = -1;
+  for (size_t i = 0; i < e->tickets.size(); i++)
+    if (e->tickets[i].state == kFree) { id = (int)i; break; }
+  if (id < 0) return CSWAP_E_NOMEM;
+  Ticket& t = e->tickets[(size_t)id];
+  t.policy = policy; t.n = n; t.nnz = 0; t.nx = nx; t.ny = ny; t.nz = nz;
+  t.dev_held = false;
+
+  int rc;
+  const bool want_probe = (policy == CSWAP_POLICY_AUTO && zvc_ok) || policy == CSWAP_POLICY_SPARSE;
+  if (want_probe) {
+    // Worst-case ZVC staging; the chunk counts go straight into its header so
+    // that a later compaction needs no second counting pass.
+    const size_t hdr = zvc_header_bytes((int)n, e->process);
+    const size_t worst = hdr + 4 * n;
+    size_t off;
+    if (e->dpool.alloc(worst, &off)) {
+      t.dev_off = off; t.dev_bytes = worst; t.dev_held = true;
+      int* d_begin = (int*)(e->d_base + off);
+      if ((rc = cswap_zvc_count(d_in, (int)n, e->process, d_begin, compute))) { drop_device(e, t); return rc; }
+      if ((rc = cswap_zvc_scan(d_begin, cswap_zvc_active_chunks((int)n, e->process), e->d_nnz, compute))) {
+        drop_device(e, t); return rc;
+      }
+      hipError_t err = hipMemcpyAsync(e->h_nnz, e->d_nnz, sizeof(int), hipMemcpyDeviceToHost, compute);
+      if (err == hipSuccess) err = hipEventRecord(e->ev_probe, compute);
+      if (err == hipSuccess) err = hipEventSynchronize(e->ev_probe);  // the one host round trip (Execution.h:92)
+      if (err != hipSuccess) { drop_device(e, t); return hip_fail(err); }
+      t.nnz = (size_t)*e->h_nnz;
+    } else if (policy == CSWAP_POLICY_SPARSE) {
+      return CSWAP_E_NOMEM;
+    } else {
+      t.nnz = n;  // no room to probe: treat as dense
+    }
+  } else {
+    t.nnz = n;
+  }
+
+  if (policy == CSWAP_POLICY_AUTO) {
+    cswap_choice ch;
+    cswap_costs c = e->costs;
+    if (!t.dev_held) c.sparse_max_ratio = 0.0;  // not probed: ZVC is not an option
+    if ((rc = cswap_select(n, t.nnz, e->maxbits, &c, &ch))) { drop_device(e, t); return rc; }
+    t.policy = ch.policy;
+  }
+
+  // ---- compress on the compute stream
+  const void* src = nullptr;
+  if (t.policy == CSWAP_POLICY_SPARSE) {
+    const size_t hdr = zvc_header_bytes((int)n, e->process);
+    char* base = e->d_base + t.dev_off;
+    int* d_begin = (int*)base;
+    uint32_t* d_mask = (uint32_t*)(base + 4 * (size_t)e->process);
+    float* d_values = (float*)(base + hdr);
+    if ((rc = cswap_zvc_compact(d_in, (int)n, e->process, d_begin, d_values, d_mask, compute))) {
+      drop_device(e, t); return rc;
+    }
+    t.bytes_out = hdr + 4 * t.nnz;
+    e->dpool.shrink(t.dev_off, t.dev_bytes, t.bytes_out);
+    t.dev_bytes = t.bytes_out;
+    src = base;
+  } else if (t.policy == CSWAP_POLICY_ZFP) {
+    t.bytes_out = cswap_zfp_stream_capacity(nx, ny, nz, e->maxbits);
+    if (t.dev_held) {
+      if (t.dev_bytes >= t.bytes_out) {
+        e->dpool.shrink(t.dev_off, t.dev_bytes, t.bytes_out);
+        t.dev_bytes = t.bytes_out;
+      } else {
+        drop_device(e, t);
+      }
+    }
+    if (!t.dev_held) {
+      size_t off;
+      if (!e->dpool.alloc(t.bytes_out, &off)) return CSWAP_E_NOMEM;
+      t.dev_off = off; t.dev_bytes = t.bytes_out; t.dev_held = true;
+    }
+    uint64_t* d_stream = (uint64_t*)(e->d_base + t.dev_off);
+    if ((rc = cswap_zfp_compress_f32(d_in, nx, ny, nz, 0, 0, 0, e->maxbits, d_stream, compute))) {
+      drop_device(e, t); return rc;
+    }
+    src = d_stream;
+  } else {
+    drop_device(e, t);
+    t.bytes_out = 4 * n;
+    src = d_in;
+  }
+
+  size_t hoff;
+  if (!e->hpool.alloc(t.bytes_out, &hoff)) { drop_device(e, t); return CSWAP_E_NOMEM; }
+  t.host_off = hoff; t.host_bytes = t.bytes_out;
+
+  // ---- copy on the copy stream, ordered after the compression by an event
+  hipError_t err = hipEventRecord(t.ev_ready, compute);
+  if (err == hipSuccess) err = hipStreamWaitEvent(e->copy, t.ev_ready, 0);
+  if (err == hipSuccess) err = hipMemcpyAsync(e->h_base + hoff, src, t.bytes_out, hipMemcpyDeviceToHost, e->copy);
+  if (err == hipSuccess) err = hipEventRecord(t.ev_copy, e->copy);
+  if (err != hipSuccess) {
+    (void)hipStreamSynchronize(e->copy);
+    drop_device(e, t);
+    e->hpool.free(t.host_off, t.host_bytes);
+    return hip_fail(err);
+  }
+  t.state = kOutInFlight;
+  *ticket = id;
+  return CSWAP_OK;
+}
+
+static Ticket* get_ticket(cswap_engine* e, int id)
+{
+  if (!e || id < 0 || (size_t)id >= e->tickets.size()) return nullptr;
+  return &e->tickets[(size_t)id];
+}
+
+extern "C" int cswap_swap_wait(cswap_engine* e, int ticket)
+{
+  if (!e) return CSWAP_E_ARG;
+  std::lock_guard<std::mutex> lock(e->mu);
+  Ticket* t = get_ticket(e, ticket);
+  if (!t) return CSWAP_E_ARG;
+  if (t->state == kOnHost) return CSWAP_OK;
+  if (t->state != kOutInFlight) return CSWAP_E_STATE;
+  CSWAP_HIP_TRY(hipEventSynchronize(t->ev_copy));
+  drop_device(e, *t);
+  t->state = kOnHost;
+  return CSWAP_OK;
+}
+
+extern "C" int cswap_swap_in(cswap_engine* e, int ticket, float* d_out, cswap_stream_t compute_)
+{
+  if (!e || !d_out) return CSWAP_E_ARG;
+  hipStream_t compute = (hipStream_t)compute_;
+  std::lock_guard<std::mutex> lock(e->mu);
+  Ticket* t = get_ticket(e, ticket);
+  if (!t) return CSWAP_E_ARG;
+  if (t->state == kOutInFlight) {  // swap-in right after swap-out: finish the outbound copy first
+    CSWAP_HIP_TRY(hipEventSynchronize(t->ev_copy));
+    drop_device(e, *t);
+    t->state = kOnHost;
+  }
+  if (t->state != kOnHost) return CSWAP_E_STATE;
+
+  void* dst = d_out;
+  if (t->policy != CSWAP_POLICY_NONE) {
+    size_t off;
+    if (!e->dpool.alloc(t->bytes_out, &off)) return CSWAP_E_NOMEM;
+    t->dev_off = off; t->dev_bytes = t->bytes_out; t->dev_held = true;
+    dst = e->d_base + off;
+  }
+  // the copy may not overtake earlier work of the compute stream on d_out
+  hipError_t err = hipEventRecord(t->ev_ready, compute);
+  if (err == hipSuccess) err = hipStreamWaitEvent(e->copy, t->ev_ready, 0);
+  if (err == hipSuccess) err = hipMemcpyAsync(dst, e->h_base + t->host_off, t->bytes_out, hipMemcpyHostToDevice, e->copy);
+  if (err == hipSuccess) err = hipEventRecord(t->ev_copy, e->copy);
+  if (err == hipSuccess) err = hipStreamWaitEvent(compute, t->ev_copy, 0);
+  if (err != hipSuccess) {
+    (void)hipStreamSynchronize(e->copy);
+    drop_device(e, *t);
+    return hip_fail(err);
+  }
+  int rc = CSWAP_OK;
+  if (t->policy == CSWAP_POLICY_SPARSE) {
+    const size_t hdr = zvc_header_bytes((int)t->n, e->process);
+    char* base = (char*)dst;
+    rc = cswap_zvc_expand((const float*)(base + hdr), (const uint32_t*)(base + 4 * (size_t)e->process),
+                          (const int*)base, (int)t->n, e->process, d_out, compute);
+  } else if (t->policy == CSWAP_POLICY_ZFP) {
+    rc = cswap_zfp_decompress_f32((const uint64_t*)dst, t->nx, t->ny, t->nz, 0, 0, 0, e->maxbits, d_out, compute);
+  }
+  err = hipEventRecord(t->ev_done, compute);
+  t->state = kInInFlight;
+  if (rc) return rc;
+  if (err != hipSuccess) return hip_fail(err);
+  return CSWAP_OK;
+}
+
+extern "C" int cswap_swap_release(cswap_engine* e, int ticket)
+{
+  if (!e) return CSWAP_E_ARG;
+  std::lock_guard<std::mutex> lock(e->mu);
+  Ticket* t = get_ticket(e, ticket);
+  if (!t) return CSWAP_E_ARG;
+  if (t->state == kFree) return CSWAP_E_STATE;
+  hipError_t err = hipSuccess;
+  if (t->state == kOutInFlight) err = hipEventSynchronize(t->ev_copy);
+  if (t->state == kInInFlight) err = hipEventSynchronize(t->ev_done);
+  drop_device(e, *t);
+  e->hpool.free(t->host_off, t->host_bytes);
+  t->state = kFree;
+  return err == hipSuccess ? CSWAP_OK : hip_fail(err);
+}
+
+extern "C" int cswap_swap_info(cswap_engine* e, int ticket, cswap_ticket_info* info)
+{
+  if (!e || !info) return CSWAP_E_ARG;
+  std::lock_guard<std::mutex> lock(e->mu);
+  Ticket* t = get_ticket(e, ticket);
+  if (!t) return CSWAP_E_ARG;
+  info->policy = t->policy;
+  info->n = t->n;
+  info->nnz = t->nnz;
+  info->bytes_in = 4 * t->n;
+  info->bytes_out = t->bytes_out;
+  info->state = t->state;
+  return CSWAP_OK;
+}
+
+// ----------------------------------------------------------------- calibration
+namespace {
+__global__ void fill_relu_like_kernel(float* p, size_t n)
+{
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += step) {
+    uint32_t h = (uint32_t)i * 2654435761u;
+    h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+    float v = (float)(h & 0xffff) * (1.0f / 65536.0f);
+    p[i] = (h & 0x10000) ? v : 0.0f;  // about half zeros
+  }
+}
+}  // namespace
+
+extern "C" int cswap_engine_calibrate(cswap_engine* e, cswap_costs* out_costs)
+{
+  if (!e) return CSWAP_E_ARG;
+  std::lock_guard<std::mutex> lock(e->mu);
+  // sample tensor: 64 MiB of fp32 (or what the pools allow), viewed as (64, 64, n/4096)
+  size_t n = (size_t)16 << 20;
+  int rc = CSWAP_OK;
+  float* d_x = nullptr;
+  float* d_y = nullptr;
+  char* d_tmp = nullptr;
+  hipEvent_t a = nullptr, b = nullptr;
+  hipStream_t s = e->copy;
+  size_t hoff = 0;
+  bool hheld = false;
+  auto ms = [&](auto&& fn, int reps, double* out) -> int {
+    hipError_t er = hipEventRecord(a, s);
+    for (int i = 0; i < reps && er == hipSuccess; i++) { int r = fn(); if (r) return r; }
+    if (er == hipSuccess) er = hipEventRecord(b, s);
+    if (er == hipSuccess) er = hipEventSynchronize(b);
+    float t = 0;
+    if (er == hipSuccess) er = hipEventElapsedTime(&t, a, b);
+    if (er != hipSuccess) return hip_fail(er);
+    *out = (double)t / reps;
+    return CSWAP_OK;
+  };
+  do {
+    size_t hfree = e->hpool.largest_free();
+    while (4 * n > hfree && n > (1 << 16)) n >>= 1;
+    if (4 * n > hfree) { rc = CSWAP_E_NOMEM; break; }
+    if (!e->hpool.alloc(4 * n, &hoff)) { rc = CSWAP_E_NOMEM; break; }
+    hheld = true;
+    const size_t hdr = zvc_header_bytes((int)n, e->process);
+    hipError_t er;
+    if ((er = hipMalloc((void**)&d_x, 4 * n)) != hipSuccess || (er = hipMalloc((void**)&d_y, 4 * n)) != hipSuccess ||
+        (er = hipMalloc((void**)&d_tmp, hdr + 4 * n)) != hipSuccess ||
+        (er = hipEventCreate(&a)) != hipSuccess || (er = hipEventCreate(&b)) != hipSuccess) {
+      rc = hip_fail(er); break;
+    }
+    hipLaunchKernelGGL(fill_relu_like_kernel, dim3(1024), dim3(256), 0, s, d_x, n);
+    char* h = e->h_base + hoff;
+    double t;
+    cswap_costs c = e->costs;
+    const double gb = 4.0 * (double)n / 1e9;
+    auto d2h = [&]() { hipError_t r = hipMemcpyAsync(h, d_x, 4 * n, hipMemcpyDeviceToHost, s); return r == hipSuccess ? 0 : hip_fail(r); };
+    auto h2d = [&]() { hipError_t r = hipMemcpyAsync(d_y, h, 4 * n, hipMemcpyHostToDevice, s); return r == hipSuccess ? 0 : hip_fail(r); };
+    if ((rc = ms(d2h, 1, &t))) break;  // warm-up
+    if ((rc = ms(d2h, 3, &t))) break;
+    c.bw_d2h_gbs = gb / (t * 1e-3);
+    if ((rc = ms(h2d, 1, &t))) break;
+    if ((rc = ms(h2d, 3, &t))) break;
+    c.bw_h2d_gbs = gb / (t * 1e-3);
+    auto small = [&]() { hipError_t r = hipMemcpyAsync(h, d_x, 256, hipMemcpyDeviceToHost, s); return r == hipSuccess ? 0 : hip_fail(r); };
+    if ((rc = ms(small, 20, &t))) break;
+    c.copy_latency_us = t * 1e3;
+    int* d_begin = (int*)d_tmp;
+    uint32_t* d_mask = (uint32_t*)(d_tmp + 4 * (size_t)e->process);
+    float* d_vals = (float*)(d_tmp + hdr);
+    auto zc = [&]() { return cswap_zvc_compress(d_x, (int)n, e->process, d_begin, e->d_nnz, d_vals, d_mask, s); };
+    auto ze = [&]() { return cswap_zvc_expand(d_vals, d_mask, d_begin, (int)n, e->process, d_y, s); };
+    if ((rc = ms(zc, 2, &t))) break;
+    if ((rc = ms(zc, 10, &t))) break;
+    c.zvc_compress_gbs = gb / (t * 1e-3);
+    if ((rc = ms(ze, 2, &t))) break;
+    if ((rc = ms(ze, 10, &t))) break;
+    c.zvc_expand_gbs = gb / (t * 1e-3);
+    const size_t fx = 64, fy = 64, fz = n / 4096;
+    auto fc = [&]() { return cswap_zfp_compress_f32(d_x, fx, fy, fz, 0, 0, 0, e->maxbits, (uint64_t*)d_tmp, s); };
+    auto fdc = [&]() { return cswap_zfp_decompress_f32((const uint64_t*)d_tmp, fx, fy, fz, 0, 0, 0, e->maxbits, d_y, s); };
+    if ((rc = ms(fc, 2, &t))) break;
+    if ((rc = ms(fc, 10, &t))) break;
+    c.zfp_compress_gbs = gb / (t * 1e-3);
+    if ((rc = ms(fdc, 2, &t))) break;
+    if ((rc = ms(fdc, 10, &t))) break;
+    c.zfp_decompress_gbs = gb / (t * 1e-3);
+    e->costs = c;
+  } while (0);
+  (void)hipStreamSynchronize(s);
+  if (hheld) e->hpool.free(hoff, 4 * n);
+  if (a) (void)hipEventDestroy(a);
+  if (b) (void)hipEventDestroy(b);
+  if (d_x) (void)hipFree(d_x);
+  if (d_y) (void)hipFree(d_y);
+  if (d_tmp) (void)hipFree(d_tmp);
+  if (!rc && out_costs) *out_costs = e->costs;
+  return rc;
+}

@@ -1,0 +1,153 @@
+"""Python face of the swap engine (C++: cswap_amd/csrc/swap_engine.cpp).
+
+``SwapEngine`` mirrors the reference's ``Execution`` object
+(CSWAP+/Execution.h:38-446): ``pre`` kicks compression + the asynchronous copy
+to pinned host memory for a tensor, ``post`` waits for that copy after the
+layer's compute was launched; ``swap_in`` is the backward-side mirror the
+reference keeps inside its patched autograd engine.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import time
+
+import torch
+
+from ._lib import Choice, Costs, EngineConfig, TicketInfo, check, lib
+from .workloads import field_dims
+
+AUTO, NONE, SPARSE, ZFP = -1, 2, 3, 6
+POLICY_NAME = {NONE: "none", SPARSE: "sparse", ZFP: "zfp"}
+
+
+def default_costs() -> Costs:
+    c = Costs()
+    lib().cswap_costs_default(C.byref(c))
+    return c
+
+
+def select(n: int, nnz: int, maxbits: int = 512, costs: Costs | None = None) -> Choice:
+    ch = Choice()
+    check(lib().cswap_select(n, nnz, maxbits, C.byref(costs) if costs is not None else None, C.byref(ch)),
+          "cswap_select")
+    return ch
+
+
+class SwapEngine:
+    def __init__(self, pinned_bytes: int = 1 << 30, device_bytes: int = 1 << 30, maxbits: int = 512,
+                 process: int = 512 * 32, max_tickets: int = 256, costs: Costs | None = None):
+        cfg = EngineConfig()
+        lib().cswap_engine_config_default(C.byref(cfg))
+        cfg.pinned_pool_bytes = pinned_bytes
+        cfg.device_pool_bytes = device_bytes
+        cfg.zfp_maxbits = maxbits
+        cfg.process = process
+        cfg.max_tickets = max_tickets
+        if costs is not None:
+            cfg.costs = costs
+        self._h = C.c_void_p()
+        check(lib().cswap_engine_create(C.byref(self._h), C.byref(cfg)), "cswap_engine_create")
+
+    def close(self):
+        if self._h:
+            lib().cswap_engine_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def calibrate(self) -> Costs:
+        c = Costs()
+        check(lib().cswap_engine_calibrate(self._h, C.byref(c)), "cswap_engine_calibrate")
+        return c
+
+    # Execution::pre
+    def pre(self, t: torch.Tensor, policy: int = AUTO) -> int:
+        if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()):
+            raise ValueError("expected a contiguous fp32 device tensor")
+        nx, ny, nz = field_dims(t.shape)
+        ticket = C.c_int(-1)
+        check(lib().cswap_swap_out(self._h, t.data_ptr(), nx, ny, nz, policy,
+                                   torch.cuda.current_stream().cuda_stream, C.byref(ticket)), "cswap_swap_out")
+        return ticket.value
+
+    # Execution::post
+    def post(self, ticket: int) -> None:
+        check(lib().cswap_swap_wait(self._h, ticket), "cswap_swap_wait")
+
+    def swap_in(self, ticket: int, out: torch.Tensor) -> torch.Tensor:
+        check(lib().cswap_swap_in(self._h, ticket, out.data_ptr(), torch.cuda.current_stream().cuda_stream),
+              "cswap_swap_in")
+        return out
+
+    def release(self, ticket: int) -> None:
+        check(lib().cswap_swap_release(self._h, ticket), "cswap_swap_release")
+
+    def info(self, ticket: int) -> TicketInfo:
+        i = TicketInfo()
+        check(lib().cswap_swap_info(self._h, ticket, C.byref(i)), "cswap_swap_info")
+        return i
+
+
+def _dummy_compute(a: torch.Tensor, b: torch.Tensor, reps: int) -> None:
+    """Stand-in for the layer's kernels that run while the copy is in flight."""
+    for _ in range(reps):
+        torch.mm(a, b)
+
+
+def bench_schedule(dev, batch: int = 128, seed: int = 0) -> dict:
+    """Configuration 4: walk the VGG-16 activation schedule; per tensor, swap out
+    (probe + select + compress + D2H on the copy stream, overlapped with a dummy
+    compute stream) and back in, against the raw (policy 2) swap."""
+    from .workloads import config4_schedule, config4_tensor
+
+    sched = config4_schedule(batch)
+    biggest = max(int(torch.tensor(e["shape"]).prod()) for e in sched) * 4
+    eng = SwapEngine(pinned_bytes=2 * biggest + (64 << 20), device_bytes=2 * biggest + (64 << 20))
+    costs = eng.calibrate()
+    a = torch.randn(2048, 2048, device=dev)
+    b = torch.randn(2048, 2048, device=dev)
+    rows = []
+    tot = {"auto": 0.0, "none": 0.0}
+    worst = 0.0
+    for e in sched:
+        x = torch.from_numpy(config4_tensor(e, seed)).to(dev)
+        out = torch.empty_like(x)
+        lat = {}
+        chosen = None
+        for label, pol in (("none", NONE), ("auto", AUTO)):
+            best = None
+            for _ in range(3):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                tk = eng.pre(x, pol)
+                _dummy_compute(a, b, 2)
+                eng.post(tk)
+                eng.swap_in(tk, out)
+                torch.cuda.synchronize()
+                t1 = time.perf_counter()
+                info = eng.info(tk)
+                eng.release(tk)
+                best = (t1 - t0) if best is None else min(best, t1 - t0)
+            lat[label] = best * 1e3
+            if label == "auto":
+                chosen = info
+        # dummy compute alone, to report how much of it the swap hides
+        torch.cuda.synchronize()
+        t0 = time.perf_counter(); _dummy_compute(a, b, 2); torch.cuda.synchronize()
+        comp_ms = (time.perf_counter() - t0) * 1e3
+        rows.append({"id": e["id"], "kind": e["kind"], "shape": list(e["shape"]), "MB": round(x.numel() * 4 / 1e6, 1),
+                     "policy": POLICY_NAME[chosen.policy], "ratio": round(chosen.bytes_out / chosen.bytes_in, 4),
+                     "none_ms": round(lat["none"], 3), "auto_ms": round(lat["auto"], 3),
+                     "compute_ms": round(comp_ms, 3)})
+        tot["auto"] += lat["auto"]; tot["none"] += lat["none"]
+        if chosen.policy != NONE:
+            worst = max(worst, lat["auto"] / lat["none"])
+        del x, out
+    eng.close()
+    return {"costs": {k: round(getattr(costs, k), 2) for k, _ in Costs._fields_ if k.endswith(("gbs", "us"))},
+            "total_none_ms": round(tot["none"], 2), "total_auto_ms": round(tot["auto"], 2),
+            "worst_compressed_over_raw": round(worst, 3), "tensors": rows}

@@ -107,6 +107,105 @@ int cswap_zvc_compress(const float* d_in, int n, int process, int* d_begin, int*
  * reference derives from PreGPUcompression + PreAcc, Execution.h:89-92). */
 int cswap_probe_nnz(const float* d_in, size_t n, unsigned long long* d_nnz, cswap_stream_t stream);
 
+/* -------------------------------------------------------------- selector -----
+ * Per-tensor choice between no compression, ZVC and fixed-rate ZFP.  The
+ * reference's selector (c10::GetPolicyMaker()->make_policy, call sites
+ * cp-vgg16.cpp:513 and vgg16-cifar10.cpp:481) is not in its tree; README.md:6
+ * describes it as weighing compression ratio, size and algorithm
+ * characteristics at run time.  This one minimises a modelled swap-out +
+ * swap-in latency:  t(option) = t_compress + bytes_out/bw_d2h + bytes_out/bw_h2d
+ * + t_decompress (+ fixed per-kernel and per-copy overheads), with kernel times
+ * = bytes_in / throughput.  Ties go to the lossless option; ZVC is only
+ * eligible when its size ratio is below sparse_max_ratio; tensors below
+ * size_floor_bytes are never compressed.  Lossless is preferred: when ZVC beats
+ * the raw swap, lossy ZFP replaces it only if it is modelled at least
+ * 1/lossy_min_gain times faster (the reference's hand-written policies give ZVC
+ * to ReLU outputs and ZFP to dense/pooled tensors, vgg16-cifar10.cpp:177-178,
+ * 393-397).
+ */
+typedef enum { CSWAP_POLICY_AUTO = -1, CSWAP_POLICY_NONE = 2, CSWAP_POLICY_SPARSE = 3,
+               CSWAP_POLICY_ZFP = 6 } cswap_policy; /* codes as in Execution.h:70,86,107 */
+
+typedef struct {
+  double bw_d2h_gbs, bw_h2d_gbs;         /* pinned host link, GB/s */
+  double copy_latency_us;                /* fixed cost of one async copy */
+  double kernel_latency_us;              /* fixed cost of one kernel */
+  double zvc_compress_gbs, zvc_expand_gbs; /* GB/s of fp32 in / out */
+  double zfp_compress_gbs, zfp_decompress_gbs;
+  double sparse_max_ratio;               /* ZVC eligible only below this size ratio */
+  double lossy_min_gain;                 /* ZFP replaces a winning ZVC only if t_zfp < gain * t_zvc */
+  size_t size_floor_bytes;               /* never compress smaller tensors */
+  int    allow_lossy;                    /* 0: ZFP is never chosen */
+  int    process;                        /* ZVC chunk count (512*32 in the reference) */
+} cswap_costs;
+
+typedef struct {
+  int    policy;            /* CSWAP_POLICY_NONE / SPARSE / ZFP */
+  size_t bytes_out;         /* bytes that cross the host link, one way */
+  double ratio;             /* bytes_out / (4*n) */
+  double t_none_us, t_sparse_us, t_zfp_us; /* modelled swap-out + swap-in latency */
+} cswap_choice;
+
+/* Defaults measured on one MI355X box (see cswap_calibrate to re-measure). */
+void cswap_costs_default(cswap_costs* c);
+/* Bytes a tensor of n elements with nnz non-zeros occupies under each policy. */
+size_t cswap_policy_bytes(int policy, size_t n, size_t nnz, unsigned maxbits, int process,
+                          size_t nx, size_t ny, size_t nz);
+/* Pure host function, no GPU work. */
+int cswap_select(size_t n, size_t nnz, unsigned maxbits, const cswap_costs* costs, cswap_choice* out);
+
+/* ----------------------------------------------------------- swap engine -----
+ * Mirror of Execution::init_/pre/post (Execution.h:46-133,217-310) and of the
+ * backward-side swap-in the reference keeps in its patched autograd
+ * (com_and_tran tags, Execution.h:262,280,299).  One engine owns a copy stream
+ * (default priority, non-blocking), a pinned host pool and a device staging
+ * pool, all allocated once in cswap_engine_create and freed in
+ * cswap_engine_destroy; the swap calls themselves do not allocate.
+ */
+typedef struct cswap_engine cswap_engine;
+
+typedef struct {
+  size_t pinned_pool_bytes;   /* host side: compressed tensors live here while swapped out */
+  size_t device_pool_bytes;   /* device staging for compressed data in flight */
+  int    process;             /* ZVC chunk count; 0 = 16384 */
+  unsigned zfp_maxbits;       /* bits per 4x4x4 block for policy ZFP; 0 = 512 (8 bits/value) */
+  int    max_tickets;         /* tensors that may be swapped out at once; 0 = 256 */
+  cswap_costs costs;          /* used by CSWAP_POLICY_AUTO; zero bw fields = defaults */
+} cswap_engine_config;
+
+typedef struct {
+  int    policy;              /* what was actually done */
+  size_t n, nnz;              /* elements; non-zeros (valid when probed) */
+  size_t bytes_in, bytes_out; /* 4*n; bytes that crossed the link */
+  int    state;               /* 0 free, 1 out in flight, 2 resident on host, 3 in in flight */
+} cswap_ticket_info;
+
+void cswap_engine_config_default(cswap_engine_config* cfg);
+int  cswap_engine_create(cswap_engine** out, const cswap_engine_config* cfg);
+void cswap_engine_destroy(cswap_engine* e);
+
+/* Execution::pre: compress d_in on `compute` (policy AUTO probes and selects
+ * first, which costs one small host round trip like Execution.h:92) and start
+ * the device-to-host copy on the engine's copy stream, ordered after the
+ * compression by an event.  The tensor is the field a[nz][ny][nx]. */
+int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, size_t ny, size_t nz, int policy,
+                   cswap_stream_t compute, int* ticket);
+/* Execution::post: block the host until the copy of `ticket` has finished;
+ * afterwards the caller may free or overwrite the device tensor. */
+int cswap_swap_wait(cswap_engine* e, int ticket);
+/* Backward side: copy back on the copy stream, then decompress into d_out on
+ * `compute` (ordered by an event).  Returns at once; the data is ready when
+ * `compute` reaches this point. */
+int cswap_swap_in(cswap_engine* e, int ticket, float* d_out, cswap_stream_t compute);
+/* Return the ticket's host (and any device) memory to the pools.  Waits for the
+ * work of the ticket that is still in flight. */
+int cswap_swap_release(cswap_engine* e, int ticket);
+int cswap_swap_info(cswap_engine* e, int ticket, cswap_ticket_info* info);
+/* Measure link bandwidth and kernel throughput on this box and store them in
+ * the engine's cost model (allocates temporaries; call once after create). */
+int cswap_engine_calibrate(cswap_engine* e, cswap_costs* out_costs);
+cswap_stream_t cswap_engine_copy_stream(cswap_engine* e);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,7 +23,7 @@ def declared_in_header():
 
 
 REFERENCE_NAMES = {"PreGPUcompression", "PreAcc", "GPUcompression", "GPUdecompression", "cuda_compress",
-                   "cuda_decompress", "compress", "setRatio"}
+                   "cuda_decompress", "compress", "decompress", "setRatio"}
 
 
 def test_library_exports_every_declared_symbol():

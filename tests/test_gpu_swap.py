@@ -1,0 +1,214 @@
+"""GPU tests of the swap engine (Execution::pre/post mirror + backward swap-in)
+and of the reference-named entry points."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return torch
+
+
+@pytest.fixture(scope="module")
+def engine(torch_cuda):
+    from cswap_amd import swap
+
+    e = swap.SwapEngine(pinned_bytes=512 << 20, device_bytes=512 << 20)
+    yield e
+    e.close()
+
+
+def relu_tensor(torch, shape, zeros, seed):
+    from cswap_amd.workloads import _ndtri
+
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal(shape, dtype=np.float32) - np.float32(_ndtri(zeros))
+    return torch.from_numpy(np.maximum(x, 0).astype(np.float32)).cuda()
+
+
+@pytest.mark.parametrize("policy_name", ["none", "sparse", "zfp"])
+def test_round_trip_equals_codec_round_trip(torch_cuda, engine, policy_name):
+    torch = torch_cuda
+    import oracle
+    from cswap_amd import swap
+
+    pol = {"none": swap.NONE, "sparse": swap.SPARSE, "zfp": swap.ZFP}[policy_name]
+    x = relu_tensor(torch, (16, 64, 32, 32), 0.6, 3)
+    out = torch.full_like(x, -5.0)
+    tk = engine.pre(x, pol)
+    engine.post(tk)
+    info = engine.info(tk)
+    assert info.policy == pol and info.state == 2
+    engine.swap_in(tk, out)
+    torch.cuda.synchronize()
+    engine.release(tk)
+    xn = x.cpu().numpy()
+    if pol == swap.ZFP:
+        f = xn.reshape(-1, 32, 32)
+        want = oracle.zfp_decode3(oracle.zfp_encode3(f, 512, omp=True), f.shape, 512, omp=True)
+        assert np.array_equal(out.cpu().numpy().reshape(f.shape).view(np.uint32), want.view(np.uint32))
+        assert info.bytes_out == xn.size
+    else:
+        assert torch.equal(out, x)
+        if pol == swap.SPARSE:
+            nnz = np.count_nonzero(xn)
+            assert info.nnz == nnz
+            assert info.bytes_out == 4 * nnz + xn.size // 8 + 4 * 16384
+
+
+def test_auto_policy_follows_selector(torch_cuda, engine):
+    torch = torch_cuda
+    from cswap_amd import swap
+
+    cases = [(relu_tensor(torch, (32, 64, 32, 32), 0.7, 1), swap.SPARSE),
+             (torch.randn((32, 64, 32, 32), device="cuda"), swap.ZFP),
+             (relu_tensor(torch, (1, 4, 8, 8), 0.7, 2), swap.NONE)]
+    for x, want in cases:
+        tk = engine.pre(x)
+        engine.post(tk)
+        info = engine.info(tk)
+        assert info.policy == want
+        assert info.policy == swap.select(x.numel(), info.nnz).policy
+        out = torch.empty_like(x)
+        engine.swap_in(tk, out)
+        torch.cuda.synchronize()
+        engine.release(tk)
+        if want != swap.ZFP:
+            assert torch.equal(out, x)
+        else:
+            assert float((out - x).abs().max()) < 0.5
+
+
+def test_many_in_flight_and_overlap_ordering(torch_cuda, engine):
+    """Several tensors out at once; compute keeps running on the compute stream
+    between pre and post; results come back intact in any order."""
+    torch = torch_cuda
+    from cswap_amd import swap
+
+    xs = [relu_tensor(torch, (8, 64, 32, 32), 0.5 + 0.05 * i, 10 + i) for i in range(6)]
+    a = torch.randn(1024, 1024, device="cuda")
+    tks = []
+    for i, x in enumerate(xs):
+        tks.append(engine.pre(x, [swap.SPARSE, swap.NONE, swap.AUTO][i % 3]))
+        a = a @ a * 1e-3          # layer compute while the copy is in flight
+    for tk in tks:
+        engine.post(tk)
+    keep = [x.clone() for x in xs]
+    for x in xs:
+        x.zero_()                 # device copies are gone
+    for i in reversed(range(len(xs))):
+        engine.swap_in(tks[i], xs[i])
+    torch.cuda.synchronize()
+    for tk in tks:
+        engine.release(tk)
+    for x, k in zip(xs, keep):
+        assert torch.equal(x, k)
+
+
+def test_state_machine_errors(torch_cuda, engine):
+    torch = torch_cuda
+    from cswap_amd._lib import lib
+
+    x = torch.randn(4096 * 64, device="cuda")
+    L = lib()
+    assert L.cswap_swap_wait(engine._h, 12345) == -1
+    assert L.cswap_swap_release(engine._h, 0) in (-5, 0)   # ticket 0 is free unless a test leaked it
+    tk = engine.pre(x.view(64, 64, 64), 2)
+    engine.post(tk)
+    engine.swap_in(tk, x)
+    assert L.cswap_swap_in(engine._h, tk, x.data_ptr(), None) == -5   # already in flight
+    torch.cuda.synchronize()
+    engine.release(tk)
+    assert L.cswap_swap_release(engine._h, tk) == -5
+    t2 = C.c_int(-1)
+    assert L.cswap_swap_out(engine._h, x.data_ptr(), 64, 64, 64, 99, None, C.byref(t2)) == -1
+    huge = C.c_int(-1)
+    assert L.cswap_swap_out(engine._h, x.data_ptr(), 1 << 14, 1 << 14, 8, 2, None, C.byref(huge)) == -4
+
+
+def test_calibration_gives_sane_costs(torch_cuda, engine):
+    c = engine.calibrate()
+    assert 5 < c.bw_d2h_gbs < 200 and 5 < c.bw_h2d_gbs < 200
+    assert c.zfp_compress_gbs > 50 and c.zfp_decompress_gbs > 50
+    assert c.zvc_compress_gbs > 50 and c.zvc_expand_gbs > 50
+
+
+def test_reference_named_entry_points(torch_cuda):
+    """cuda_compress / cuda_decompress with the reference's struct layout and
+    device pointers (CSWAP+/simple.c:26-74 with device memory), compress /
+    decompress / setRatio (CSWAP+/Execution.h:63,113) and the four ZVC launchers."""
+    torch = torch_cuda
+    import oracle
+    from cswap_amd._lib import ZfpBitstream, ZfpField, ZfpStream, lib
+
+    L = lib()
+    rng = np.random.default_rng(5)
+    f = rng.standard_normal((12, 8, 16)).astype(np.float32)
+    t = torch.from_numpy(f).cuda()
+    cap = L.cswap_zfp_stream_capacity(16, 8, 12, 1024)
+    sbuf = torch.zeros(cap, dtype=torch.uint8, device="cuda")
+    bs = ZfpBitstream(0, 0, sbuf.data_ptr(), sbuf.data_ptr(), sbuf.data_ptr() + cap)
+    zs = ZfpStream(1, 1024, 64, -1074, C.pointer(bs), 0, 0, 0)     # zfp_stream_open defaults: maxbits 1024
+    fld = ZfpField(3, 16, 8, 12, 0, 0, 0, 0, 0, t.data_ptr())
+    n = L.cuda_compress(C.byref(zs), C.byref(fld))
+    assert n == cap == bs.ptr - bs.begin
+    want = oracle.zfp_encode3(f, 1024)
+    assert np.array_equal(sbuf.cpu().numpy().view(np.uint64), want)
+    t.zero_()
+    bs.ptr = bs.begin
+    L.cuda_decompress(C.byref(zs), C.byref(fld))
+    assert bs.ptr - bs.begin == cap
+    assert np.array_equal(t.cpu().numpy().view(np.uint32), oracle.zfp_decode3(want, f.shape, 1024).view(np.uint32))
+    # host pointers are staged like the reference does
+    hs = np.zeros(cap, dtype=np.uint8)
+    bs2 = ZfpBitstream(0, 0, hs.ctypes.data, hs.ctypes.data, hs.ctypes.data + cap)
+    zs2 = ZfpStream(1, 1024, 64, -1074, C.pointer(bs2), 0, 0, 0)
+    fh = f.copy()
+    fld2 = ZfpField(3, 16, 8, 12, 0, 0, 0, 0, 0, fh.ctypes.data)
+    assert L.cuda_compress(C.byref(zs2), C.byref(fld2)) == cap
+    assert np.array_equal(hs.view(np.uint64), want)
+    fh[:] = 0
+    L.cuda_decompress(C.byref(zs2), C.byref(fld2))
+    assert np.array_equal(fh.view(np.uint32), oracle.zfp_decode3(want, f.shape, 1024).view(np.uint32))
+    # unsupported: double fields -> failure value 0
+    fld3 = ZfpField(4, 16, 8, 12, 0, 0, 0, 0, 0, t.data_ptr())
+    assert L.cuda_compress(C.byref(zs), C.byref(fld3)) == 0
+
+    # compress / decompress / setRatio on a flat activation (viewed as 32x32 rows)
+    x = torch.randn(64 * 1024, device="cuda")
+    L.setRatio(128)
+    nbytes = C.c_size_t(0)
+    buf = L.compress(x.data_ptr(), x.numel(), C.byref(nbytes))
+    assert buf and nbytes.value == x.numel()
+    y = torch.empty_like(x)
+    assert L.decompress(buf, x.numel(), y.data_ptr()) == 0
+    xf = x.cpu().numpy().reshape(-1, 32, 32)
+    wantx = oracle.zfp_decode3(oracle.zfp_encode3(xf, 512), xf.shape, 512)
+    assert np.array_equal(y.cpu().numpy().reshape(xf.shape).view(np.uint32), wantx.view(np.uint32))
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipFree.argtypes = [ctypes.c_void_p]
+    assert hip.hipFree(buf) == 0
+
+    # ZVC launchers in the reference's order
+    r = torch.relu(torch.randn(16384 * 96, device="cuda"))
+    nE = r.numel()
+    idx = torch.zeros(16384, dtype=torch.int32, device="cuda")
+    num = torch.zeros(1, dtype=torch.int32, device="cuda")
+    L.PreGPUcompression(nE, 16384, r.data_ptr(), idx.data_ptr(), 512, 32, None)
+    L.PreAcc(idx.data_ptr(), 16384, num.data_ptr(), 1, 1, None)
+    k = int(num.item())
+    vals = torch.empty(k, dtype=torch.float32, device="cuda")
+    mask = torch.empty(3 * 16384, dtype=torch.int32, device="cuda")
+    L.GPUcompression(nE, 16384, r.data_ptr(), vals.data_ptr(), idx.data_ptr(), mask.data_ptr(), 512, 32, None)
+    dest = torch.full_like(r, 9.0)
+    L.GPUdecompression(vals.data_ptr(), dest.data_ptr(), nE, 16384, mask.data_ptr(), idx.data_ptr(), 512, 32)
+    torch.cuda.synchronize()
+    assert torch.equal(dest, r) and k == int((r != 0).sum().item())
