@@ -1,0 +1,56 @@
+"""Host build of the PRODUCT's per-block codec (cswap_amd/csrc/zfp_block.h, the
+code every GPU lane runs) against the zfp 0.5.5 golden vectors.  Not a GPU test:
+it catches logic errors in the block codec before any kernel is launched."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from conftest import ROOT, golden_cases
+
+SO = os.path.join(ROOT, "tests", "libhost_block_codec.so")
+SRC = os.path.join(ROOT, "tests", "host_block_codec.cpp")
+HDR = os.path.join(ROOT, "cswap_amd", "csrc", "zfp_block.h")
+
+
+@pytest.fixture(scope="module")
+def host():
+    if (not os.path.exists(SO) or os.path.getmtime(SO) < max(os.path.getmtime(SRC), os.path.getmtime(HDR))):
+        subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-o", SO, SRC])
+    L = C.CDLL(SO)
+    L.host_zfp_encode3.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
+    L.host_zfp_decode3.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
+    L.host_transpose32.argtypes = [C.c_void_p]
+    return L
+
+
+def test_transpose32_is_a_bit_matrix_transpose(host):
+    a = np.random.default_rng(0).integers(0, 2**32, 32, dtype=np.uint32)
+    b = a.copy()
+    host.host_transpose32(b.ctypes.data)
+    A = np.unpackbits(a.view(np.uint8).reshape(32, 4), axis=1, bitorder="little")
+    B = np.unpackbits(b.view(np.uint8).reshape(32, 4), axis=1, bitorder="little")
+    assert np.array_equal(B, A.T)
+
+
+def test_block_codec_matches_golden_vectors(host, golden):
+    n = 0
+    for name, rate, maxbits, f, stream, dec in golden_cases(golden):
+        nz, ny, nx = f.shape
+        blocks = -(-nx // 4) * -(-ny // 4) * -(-nz // 4)
+        words = (blocks * maxbits + 63) // 64
+        s = np.zeros(words + 1, dtype=np.uint64)
+        host.host_zfp_encode3(f.ctypes.data, nx, ny, nz, maxbits, s.ctypes.data)
+        sb = s[:words].view(np.uint8)
+        k = min(sb.size, stream.size)
+        assert np.array_equal(sb[:k], stream[:k]), (name, rate)
+        assert not sb[k:].any() and not stream[k:].any()
+        g = np.zeros((words + 1) * 8, dtype=np.uint8)
+        g[:k] = stream[:k]
+        o = np.zeros_like(f)
+        host.host_zfp_decode3(g.ctypes.data, nx, ny, nz, maxbits, o.ctypes.data)
+        assert np.array_equal(o.view(np.uint32), dec.view(np.uint32)), (name, rate)
+        n += 1
+    assert n >= 100
