@@ -3,8 +3,8 @@
 //
 // The same source compiles for the device (hipcc) and for the host (any C++17
 // compiler), so the block logic can be checked on a CPU before it ever runs on
-// a GPU.  Nothing here touches memory except through the Sink/Source objects
-// the caller passes in.
+// a GPU.  Nothing here touches memory except through the Mem object (or32 / ld32
+// on a bit region) the caller passes in.
 //
 // What it implements (reference: the cuZFP snapshot of zfp 0.5.5 in
 // CSWAP+/zfp): block-floating-point cast (encode.cuh:40-71,120-149), the
@@ -16,11 +16,14 @@
 // How it differs from the reference's formulation (results are identical):
 //  * The 64x32 bit matrix of coefficients is transposed once with a butterfly
 //    network instead of extracting each plane bit by bit.
-//  * The coder emits whole runs: "group test 1, t zeros, terminating 1" is one
-//    64-bit append found with a count-trailing-zeros, not t+2 single-bit writes.
+//  * The coder emits whole runs: "group test 1, t zeros, terminating 1" is two
+//    single-bit ORs into a zeroed bit region, placed with a count-trailing-zeros,
+//    not t+2 single-bit writes; nothing is accumulated or flushed.
 //  * The bit budget is applied as a cut of the unconstrained code at maxbits
 //    (the reference's per-bit budget counter stops the same sequence of writes
 //    at the same place, so the kept prefix is the same).
+//  * The low 16 bit planes are only transposed and coded when some block of the
+//    wavefront still has budget left after the top 16.
 #pragma once
 #include <stdint.h>
 
@@ -156,15 +159,18 @@ CSWAP_HD void inv_xform3(int32_t (&b)[64])
 
 // ---------------------------------------------------------------- bit transpose
 // In-place transpose of a 32x32 bit matrix held as 32 words: afterwards bit i
-// of a[k] is what bit k of a[i] was.  Five butterfly stages; each swaps the
-// upper-right and lower-left sub-blocks of every 2j x 2j tile.
-template <int J>
+// of a[k] is what bit k of a[i] was.  Five butterfly stages; stage J swaps the
+// upper-right and lower-left JxJ sub-blocks of every 2Jx2J tile.  The stages
+// commute (each exchanges one row-index bit with one column-index bit), and
+// after stage 16 the rows 16..31 hold only the high 16 bit-columns of the input,
+// so the top 16 planes can be finished without touching rows 0..15.
+template <int J, int R0, int R1>
 CSWAP_HD void tr_stage(uint32_t (&a)[32])
 {
   constexpr uint32_t m = J == 16 ? 0x0000ffffu : J == 8 ? 0x00ff00ffu : J == 4 ? 0x0f0f0f0fu
                          : J == 2 ? 0x33333333u : 0x55555555u;
 #pragma unroll
-  for (int r = 0; r < 32; r++) {
+  for (int r = R0; r < R1; r++) {
     if (r & J) continue;
     uint32_t lo = a[r], hi = a[r + J];
     a[r] = (lo & m) | ((hi << J) & ~m);
@@ -172,13 +178,21 @@ CSWAP_HD void tr_stage(uint32_t (&a)[32])
   }
 }
 
+// stages 8,4,2,1 on rows [R0, R0+16)
+template <int R0>
+CSWAP_HD void tr_half(uint32_t (&a)[32])
+{
+  tr_stage<8, R0, R0 + 16>(a);
+  tr_stage<4, R0, R0 + 16>(a);
+  tr_stage<2, R0, R0 + 16>(a);
+  tr_stage<1, R0, R0 + 16>(a);
+}
+
 CSWAP_HD void transpose32(uint32_t (&a)[32])
 {
-  tr_stage<16>(a);
-  tr_stage<8>(a);
-  tr_stage<4>(a);
-  tr_stage<2>(a);
-  tr_stage<1>(a);
+  tr_stage<16, 0, 32>(a);
+  tr_half<16>(a);
+  tr_half<0>(a);
 }
 
 // ---------------------------------------------------------------- block cast
@@ -188,100 +202,100 @@ CSWAP_HD void transpose32(uint32_t (&a)[32])
 // block, so the 8-bit header exponent e = emax + 127 is E + 1, or 0.
 CSWAP_HD uint32_t block_header_e(const float (&f)[64])
 {
-  uint32_t m = 0;  // |x| compares like its bit pattern
+  float m = 0.0f;
 #pragma unroll
-  for (int i = 0; i < 64; i++) {
-    uint32_t a = f32_bits(f[i]) & 0x7fffffffu;
-    m = a > m ? a : m;
-  }
-  return m ? (m >> 23) + 1 : 0;
+  for (int i = 0; i < 64; i++) m = fmaxf(m, fabsf(f[i]));
+  uint32_t b = f32_bits(m);
+  return b ? (b >> 23) + 1 : 0;
+}
+
+// "does any block of this wavefront still ..." -- on the host a block is alone
+#if defined(__HIP_DEVICE_COMPILE__)
+#define CSWAP_ANY(pred) (__builtin_amdgcn_ballot_w64(pred) != 0)
+#else
+#define CSWAP_ANY(pred) (pred)
+#endif
+
+CSWAP_HD uint32_t funnel_shr(uint32_t hi, uint32_t lo, unsigned s)  // ({hi,lo} >> (s & 31)) low word
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_alignbit(hi, lo, s);
+#else
+  s &= 31;
+  return s ? (lo >> s) | (hi << (32 - s)) : lo;
+#endif
 }
 
 // ---------------------------------------------------------------- encoder
-// Appends bit strings to the block's own stream and hands out finished 64-bit
-// words to the sink: sink.put(j, word) receives word j (bits 64j..64j+63 of
-// the block); words at or past maxbits are dropped and the word that straddles
-// maxbits is cut.
-template <class Sink>
-struct BitAppender {
-  Sink& sink;
-  uint64_t acc;
-  unsigned accn;   // valid bits in acc, 0..63
-  unsigned j;      // index of the word acc will become
-  unsigned maxbits;
+// The block's bits are OR-ed into a zero-initialised bit region through
+// mem.or32(dword_index, value); bit positions are absolute within that region.
+// The block owns [pos0, pos0 + maxbits).  GUARD = true cuts every write at the
+// end of the block (needed when the next block's bits follow immediately);
+// GUARD = false lets the last plane spill up to 96 bits past the end, which the
+// caller must provide as slack and ignore.
+template <class Mem, bool GUARD>
+struct BlockEncoder {
+  Mem& mem;
+  unsigned pos, limit;
+  unsigned n;  // coefficients already known significant
 
-  CSWAP_HD BitAppender(Sink& s, unsigned mb) : sink(s), acc(0), accn(0), j(0), maxbits(mb) {}
+  CSWAP_HD BlockEncoder(Mem& m, unsigned pos0, unsigned maxbits) : mem(m), pos(pos0), limit(pos0 + maxbits), n(0) {}
 
-  CSWAP_HD unsigned emitted() const { return 64 * j + accn; }
-  CSWAP_HD bool full() const { return emitted() >= maxbits; }
+  CSWAP_HD bool active() const { return pos < limit; }
 
-  CSWAP_HD void out(uint64_t w)
-  {
-    unsigned base = 64 * j;
-    if (base < maxbits) {
-      unsigned room = maxbits - base;
-      if (room < 64) w &= low_mask(room);
-      sink.put(j, w);
-    }
-    j++;
-  }
-
-  // append the low len (0..64) bits of v; bits of v at or above len must be 0
+  // append the low len (0..64) bits of v (bits at or above len must be 0); needs pos < limit
   CSWAP_HD void put(uint64_t v, unsigned len)
   {
-    acc |= v << accn;
-    unsigned tot = accn + len;
-    if (tot >= 64) {
-      out(acc);
-      unsigned used = 64 - accn;              // 1..64 bits of v went out
-      acc = used >= 64 ? 0 : (v >> used);
-      tot -= 64;
+    if (GUARD) {
+      unsigned room = limit - pos;
+      if (len > room) v &= low_mask(room);
     }
-    accn = tot;
+    unsigned d = pos >> 5, s = pos & 31;
+    uint64_t lo = v << s;
+    uint32_t hi = ((uint32_t)(v >> 32) >> 1) >> (31 - s);
+    mem.or32(d, (uint32_t)lo);
+    mem.or32(d + 1, (uint32_t)(lo >> 32));
+    mem.or32(d + 2, hi);
+    pos += len;
   }
 
-  CSWAP_HD void finish()
+  CSWAP_HD void set_bit(unsigned b, bool on)
   {
-    if (accn) { out(acc); acc = 0; accn = 0; }
+    if (GUARD) on = on && b < limit;
+    mem.or32(b >> 5, on ? (1u << (b & 31)) : 0u);
+  }
+
+  // one bit plane: x bit i = this plane's bit of coefficient i (encode.cuh:331-344)
+  CSWAP_HD void plane(uint64_t x)
+  {
+    if (!active()) return;
+    put(x & low_mask(n), n);  // first n coefficients verbatim
+    if (n < 64) {
+      uint64_t rest = x >> n;
+      while (rest != 0 && n < 64 && pos < limit) {
+        unsigned t = (unsigned)ctz64(rest);  // zeros before the next one-bit
+        unsigned nt = n + t;
+        bool more = nt < 63;                 // a one-bit at position 63 is implied, not written
+        unsigned q = pos + t + 1;
+        set_bit(pos, true);                  // positive group test
+        set_bit(q, more);                    // t zeros, then the one-bit
+        pos = q + (more ? 1u : 0u);
+        n = nt + 1;
+        rest = (rest >> t) >> 1;
+      }
+      if (rest == 0 && n < 64 && pos < limit) pos++;  // negative group test: a zero bit
+    }
   }
 };
 
-// Code the 32 bit planes x[31]..x[0] (x[k] bit i = bit k of coefficient i) into
-// the appender until the block's bit budget is used up.
-template <class Sink>
-CSWAP_HD void encode_planes(BitAppender<Sink>& bs, const uint32_t (&plo)[32], const uint32_t (&phi)[32])
-{
-  unsigned n = 0;  // coefficients already known significant
-#pragma unroll
-  for (int k = 31; k >= 0; k--) {
-    if (bs.full()) break;
-    uint64_t x = ((uint64_t)phi[k] << 32) | plo[k];
-    // first n coefficients: verbatim
-    bs.put(x & low_mask(n), n);
-    if (n < 64) {
-      uint64_t rest = x >> n;
-      for (;;) {
-        if (rest == 0) { bs.put(0, 1); break; }       // negative group test
-        unsigned t = (unsigned)ctz64(rest);            // zeros before the next one-bit
-        bool last = (n + t == 63);                     // one-bit at position 63 is implied
-        uint64_t v = last ? (uint64_t)1 : ((uint64_t)1 | ((uint64_t)2 << t));
-        bs.put(v, t + (last ? 1u : 2u));               // test '1', t zeros, then '1'
-        n += t + 1;
-        rest = (rest >> t) >> 1;
-        if (n >= 64 || bs.full()) break;
-      }
-    }
-  }
-}
-
 // Full block encode: f[x + 4y + 16z] (already padded for partial blocks).
-template <class Sink>
-CSWAP_HD void encode_block(const float (&f)[64], unsigned maxbits, Sink& sink)
+template <bool GUARD, class Mem>
+CSWAP_HD void encode_block(const float (&f)[64], unsigned pos0, unsigned maxbits, Mem& mem)
 {
   uint32_t e = block_header_e(f);
   if (e == 0) return;  // all-zero block: every bit stays 0 (encode.cuh:357-358)
-  BitAppender<Sink> bs(sink, maxbits);
-  bs.put(2 * e + 1, 9);
+  BlockEncoder<Mem, GUARD> enc(mem, pos0, maxbits);
+  enc.put(2 * e + 1, 9);
 
   // block-floating-point cast: scale 2^(30-emax) as a float, truncate
   float s = pow2f(30 - ((int)e - 127));
@@ -297,67 +311,109 @@ CSWAP_HD void encode_block(const float (&f)[64], unsigned maxbits, Sink& sink)
     lo[i] = int2nb(ib[kPerm3.v[i]]);
     hi[i] = int2nb(ib[kPerm3.v[32 + i]]);
   }
-  transpose32(lo);
-  transpose32(hi);
-
-  encode_planes(bs, lo, hi);
-  bs.finish();
-}
-
-// ---------------------------------------------------------------- decoder
-// Source: src.window(pos) returns the 64 stream bits of this block starting at
-// block-relative bit position pos (bits past the end of the stream may be
-// anything; they are never used).
-template <class Source>
-CSWAP_HD void decode_planes(Source& src, unsigned maxbits, uint32_t (&plo)[32], uint32_t (&phi)[32])
-{
-  unsigned pos = 9;
-  unsigned n = 0;
+  // top 16 planes first; the low 16 are only transposed if some block of the
+  // wavefront still has bit budget left after them
+  tr_stage<16, 0, 32>(lo);
+  tr_stage<16, 0, 32>(hi);
+  tr_half<16>(lo);
+  tr_half<16>(hi);
 #pragma unroll
-  for (int k = 31; k >= 0; k--) {
-    uint64_t x = 0;
-    if (pos < maxbits) {
-      unsigned left = maxbits - pos;
-      unsigned m = n < left ? n : left;
-      if (m) {
-        x = src.window(pos) & low_mask(m);
-        pos += m;
-      }
-      while (n < 64 && pos < maxbits) {
-        uint64_t w = src.window(pos);
-        pos++;
-        if (!(w & 1)) break;                       // negative group test: plane done
-        w >>= 1;                                   // 63 valid bits
-        unsigned avail = maxbits - pos;
-        unsigned maxrun = 63 - n < avail ? 63 - n : avail;
-        unsigned t = (unsigned)ctz64(w);
-        if (t < maxrun) { pos += t + 1; n += t; }  // t zeros then a one
-        else { pos += maxrun; n += maxrun; }       // ran into position 63 or the budget
-        x |= (uint64_t)1 << n;
-        n++;
-      }
-    }
-    plo[k] = (uint32_t)x;
-    phi[k] = (uint32_t)(x >> 32);
+  for (int k = 31; k >= 16; k--) enc.plane(((uint64_t)hi[k] << 32) | lo[k]);
+  if (CSWAP_ANY(enc.active())) {
+    tr_half<0>(lo);
+    tr_half<0>(hi);
+#pragma unroll
+    for (int k = 15; k >= 0; k--) enc.plane(((uint64_t)hi[k] << 32) | lo[k]);
   }
 }
 
+// ---------------------------------------------------------------- decoder
+// mem.ld32(dword_index) reads the bit region; positions are absolute within it
+// and the block owns [pos0, pos0 + maxbits).  Reads may run up to 96 bits past
+// the end of the block (the values are never used).
+template <class Mem>
+struct BlockDecoder {
+  Mem& mem;
+  unsigned pos, limit;
+  unsigned n;
+
+  CSWAP_HD BlockDecoder(Mem& m, unsigned pos0, unsigned maxbits) : mem(m), pos(pos0), limit(pos0 + maxbits), n(0) {}
+
+  CSWAP_HD bool active() const { return pos < limit; }
+
+  CSWAP_HD uint64_t window(unsigned p) const  // 64 stream bits starting at bit p
+  {
+    unsigned d = p >> 5;
+    uint32_t w0 = mem.ld32(d), w1 = mem.ld32(d + 1), w2 = mem.ld32(d + 2);
+    return ((uint64_t)funnel_shr(w2, w1, p) << 32) | funnel_shr(w1, w0, p);
+  }
+
+  // mirror of BlockEncoder::plane (decode.cuh:141-173)
+  CSWAP_HD uint64_t plane()
+  {
+    uint64_t x = 0;
+    if (!active()) return x;
+    unsigned left = limit - pos;
+    unsigned m = n < left ? n : left;
+    x = window(pos) & low_mask(m);
+    pos += m;
+    while (n < 64 && pos < limit) {
+      uint64_t w = window(pos);
+      pos++;
+      if (!(w & 1)) break;  // negative group test: plane done
+      w >>= 1;              // 63 valid bits
+      unsigned avail = limit - pos;
+      unsigned maxrun = 63 - n < avail ? 63 - n : avail;
+      unsigned t = (unsigned)ctz64(w);
+      bool found = t < maxrun;  // t zeros then a one; else ran into position 63 or the budget
+      unsigned r = found ? t : maxrun;
+      pos += r + (found ? 1u : 0u);
+      n += r;
+      x |= (uint64_t)1 << n;
+      n++;
+    }
+    return x;
+  }
+};
+
 // Full block decode into f[x + 4y + 16z]; an empty block gives +0.0 everywhere.
-template <class Source>
-CSWAP_HD void decode_block(Source& src, unsigned maxbits, float (&f)[64])
+template <class Mem>
+CSWAP_HD void decode_block(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)[64])
 {
-  uint64_t h = src.window(0);
+  BlockDecoder<Mem> dec(mem, pos0, maxbits);
+  uint32_t h = (uint32_t)dec.window(pos0);
   if (!(h & 1)) {
 #pragma unroll
     for (int i = 0; i < 64; i++) f[i] = 0.0f;
     return;
   }
   int emax = (int)((h >> 1) & 0xff) - 127;
+  dec.pos = pos0 + 9;
 
   uint32_t lo[32], hi[32];
-  decode_planes(src, maxbits, lo, hi);
-  transpose32(lo);
-  transpose32(hi);
+#pragma unroll
+  for (int k = 31; k >= 16; k--) {
+    uint64_t x = dec.plane();
+    lo[k] = (uint32_t)x;
+    hi[k] = (uint32_t)(x >> 32);
+  }
+  tr_half<16>(lo);
+  tr_half<16>(hi);
+  if (CSWAP_ANY(dec.active())) {
+#pragma unroll
+    for (int k = 15; k >= 0; k--) {
+      uint64_t x = dec.plane();
+      lo[k] = (uint32_t)x;
+      hi[k] = (uint32_t)(x >> 32);
+    }
+    tr_half<0>(lo);
+    tr_half<0>(hi);
+  } else {
+#pragma unroll
+    for (int k = 0; k < 16; k++) lo[k] = hi[k] = 0;  // transposing zeros gives zeros
+  }
+  tr_stage<16, 0, 32>(lo);
+  tr_stage<16, 0, 32>(hi);
 
   int32_t ib[64];
 #pragma unroll

@@ -5,8 +5,8 @@
 // through cast, lifting, reorder, bit transpose and the embedded coder
 // (zfp_block.h), so there is no cross-lane traffic at all.  The wave's slice of
 // the stream (64 blocks x maxbits bits = maxbits 64-bit words, always a whole
-// number of words) is staged in LDS in its final layout and moved to/from HBM
-// with fully coalesced 8-byte accesses.  Because the stream is fixed-rate,
+// number of words) is staged in LDS, which the coder addresses bit by bit, and
+// moved to/from HBM in 16-byte pieces.  Because the stream is fixed-rate,
 // stream offsets are closed-form and no device-wide scan, atomic or memset of
 // the stream is needed (the reference pre-zeroes the stream and adds every bit
 // with a global atomic, CSWAP+/zfp/encode.cuh:252-299, encode3.cuh:152).
@@ -23,37 +23,36 @@ struct Field3 {
   uint32_t nblocks;
   long long sx, sy, sz;    // strides in elements
   int rows16;              // 1: x-rows of every block are contiguous, 16-byte aligned
+  int stream16;            // 1: the stream pointer is 16-byte aligned
 };
 
-// ------------------------------------------------------------- LDS adapters
-struct LdsSink {
-  uint64_t* lds;
-  unsigned bit0;     // first bit of this lane's block inside the wave's slice
-  bool whole_words;  // maxbits % 64 == 0: the block owns its words outright
-  __device__ __forceinline__ void put(unsigned j, uint64_t w)
+// ------------------------------------------------------------- LDS adapter
+// The bit region the block codec ORs into / reads from is LDS, addressed in
+// dwords: it serves as the dynamically indexable extension of the register
+// file (a lane cannot index its registers with a run-time bit position).
+struct LdsBits {
+  uint32_t* lds;
+  __device__ __forceinline__ void or32(unsigned d, uint32_t v) const
   {
-    unsigned p = bit0 + 64 * j;
-    unsigned i = p >> 6, s = p & 63;
-    if (whole_words) {
-      lds[i] = w;
-    } else {
-      atomicOr((unsigned long long*)&lds[i], (unsigned long long)(w << s));
-      if (s) atomicOr((unsigned long long*)&lds[i + 1], (unsigned long long)(w >> (64 - s)));
-    }
+    __hip_atomic_fetch_or(&lds[d], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);  // ds_or_b32
   }
+  __device__ __forceinline__ uint32_t ld32(unsigned d) const { return lds[d]; }
 };
 
-struct LdsSource {
-  const uint64_t* lds;
-  unsigned bit0;
-  __device__ __forceinline__ uint64_t window(unsigned pos) const
-  {
-    unsigned p = bit0 + pos;
-    unsigned i = p >> 6, s = p & 63;
-    uint64_t lo = lds[i], hi = lds[i + 1];
-    return (lo >> s) | ((hi << 1) << (63 - s));
-  }
-};
+// Layout of the wave's LDS bit region.
+//  whole-word rates (maxbits % 64 == 0): every lane owns a private slot of
+//    maxbits + slack bits (slot a multiple of 128 bits), so the coder needs no
+//    end-of-block guards and each lane moves its own words to/from HBM;
+//  other rates: the 64 blocks are packed back to back exactly as in the stream
+//    (always a whole number of words per wave) and moved cooperatively.
+__host__ __device__ inline unsigned slot_bits(unsigned maxbits)
+{
+  return (maxbits & 63u) ? maxbits : ((maxbits + 128u + 127u) & ~127u);
+}
+__host__ __device__ inline unsigned region_dwords(unsigned maxbits)
+{
+  return ((2u * slot_bits(maxbits) + 4u) + 3u) & ~3u;  // + padding for the 96-bit over-read / over-write
+}
 
 // ------------------------------------------------------------- block <-> field
 __device__ __forceinline__ void block_origin(const Field3& fd, uint32_t b, uint32_t& x0, uint32_t& y0,
@@ -128,57 +127,99 @@ __device__ __forceinline__ void store_block(float* __restrict__ out, const Field
 
 // ------------------------------------------------------------- kernels
 // grid.x = ceil(nblocks/64) workgroups of one wavefront; dynamic LDS =
-// (maxbits + 1) 64-bit words.
+// region_dwords(maxbits) dwords.
+template <bool WHOLE>
 __global__ __launch_bounds__(64) void zfp_encode3_f32_kernel(const float* __restrict__ in, Field3 fd,
                                                              unsigned maxbits,
                                                              uint64_t* __restrict__ stream)
 {
-  extern __shared__ uint64_t lds[];
+  extern __shared__ uint4 lds_raw[];
+  uint32_t* lds = reinterpret_cast<uint32_t*>(lds_raw);
   const unsigned lane = threadIdx.x;
   const uint32_t first = blockIdx.x * 64u;
   const uint32_t valid = min(64u, fd.nblocks - first);
+  const unsigned slot = slot_bits(maxbits);
 
-  for (unsigned i = lane; i <= maxbits; i += 64) lds[i] = 0;
+  // zero the region: each lane clears slot bits (+ the shared padding)
+  {
+    const unsigned n16 = region_dwords(maxbits) / 4;
+    for (unsigned i = lane; i < n16; i += 64) lds_raw[i] = make_uint4(0, 0, 0, 0);
+  }
   __syncthreads();
 
   if (lane < valid) {
     float f[64];
     load_block(in, fd, first + lane, f);
-    LdsSink sink{lds, lane * maxbits, (maxbits & 63u) == 0};
-    encode_block(f, maxbits, sink);
+    LdsBits mem{lds};
+    encode_block<!WHOLE>(f, lane * slot, maxbits, mem);
   }
   __syncthreads();
 
-  const unsigned nwords = (valid * maxbits + 63u) >> 6;
-  uint64_t* dst = stream + (size_t)blockIdx.x * maxbits;
-  for (unsigned i = lane; i < nwords; i += 64) dst[i] = lds[i];
+  if (WHOLE) {
+    // each lane stores the words of its own block (16-byte stores where aligned)
+    if (lane < valid) {
+      const unsigned W = maxbits >> 6;
+      const uint64_t* src = reinterpret_cast<const uint64_t*>(lds + lane * (slot / 32));
+      uint64_t* dst = stream + (size_t)(first + lane) * W;
+      if ((W & 1u) == 0 && fd.stream16) {
+        for (unsigned j = 0; j < W; j += 2)
+          *reinterpret_cast<ulonglong2*>(dst + j) = *reinterpret_cast<const ulonglong2*>(src + j);
+      } else {
+        for (unsigned j = 0; j < W; j++) dst[j] = src[j];
+      }
+    }
+  } else {
+    const unsigned nwords = (valid * maxbits + 63u) >> 6;
+    const uint64_t* src = reinterpret_cast<const uint64_t*>(lds);
+    uint64_t* dst = stream + (size_t)blockIdx.x * maxbits;
+    for (unsigned i = lane; i < nwords; i += 64) dst[i] = src[i];
+  }
 }
 
+template <bool WHOLE>
 __global__ __launch_bounds__(64) void zfp_decode3_f32_kernel(const uint64_t* __restrict__ stream, Field3 fd,
                                                              unsigned maxbits, float* __restrict__ out)
 {
-  extern __shared__ uint64_t lds[];
+  extern __shared__ uint4 lds_raw[];
+  uint32_t* lds = reinterpret_cast<uint32_t*>(lds_raw);
   const unsigned lane = threadIdx.x;
   const uint32_t first = blockIdx.x * 64u;
   const uint32_t valid = min(64u, fd.nblocks - first);
+  const unsigned slot = slot_bits(maxbits);
 
-  const unsigned nwords = (valid * maxbits + 63u) >> 6;
-  const uint64_t* src = stream + (size_t)blockIdx.x * maxbits;
-  for (unsigned i = lane; i <= maxbits; i += 64) lds[i] = i < nwords ? src[i] : 0;
+  if (WHOLE) {
+    if (lane < valid) {
+      const unsigned W = maxbits >> 6;
+      uint64_t* dst = reinterpret_cast<uint64_t*>(lds + lane * (slot / 32));
+      const uint64_t* src = stream + (size_t)(first + lane) * W;
+      if ((W & 1u) == 0 && fd.stream16) {
+        for (unsigned j = 0; j < W; j += 2)
+          *reinterpret_cast<ulonglong2*>(dst + j) = *reinterpret_cast<const ulonglong2*>(src + j);
+      } else {
+        for (unsigned j = 0; j < W; j++) dst[j] = src[j];
+      }
+    }
+  } else {
+    const unsigned nwords = (valid * maxbits + 63u) >> 6;
+    const uint64_t* src = stream + (size_t)blockIdx.x * maxbits;
+    uint64_t* dst = reinterpret_cast<uint64_t*>(lds);
+    for (unsigned i = lane; i < nwords + 2; i += 64) dst[i] = i < nwords ? src[i] : 0;
+  }
   __syncthreads();
 
   if (lane < valid) {
     float f[64];
-    LdsSource source{lds, lane * maxbits};
-    decode_block(source, maxbits, f);
+    LdsBits mem{lds};
+    decode_block(mem, lane * slot, maxbits, f);
     store_block(out, fd, first + lane, f);
   }
 }
 
 // ------------------------------------------------------------- host side
-static int make_field(Field3& fd, const void* base, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
-                      ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits)
+static int make_field(Field3& fd, const void* base, const void* stream, size_t nx, size_t ny, size_t nz,
+                      ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits)
 {
+  if (((uintptr_t)stream % 8) != 0 || ((uintptr_t)base % 4) != 0) return CSWAP_E_ARG;
   if (!nx || !ny || !nz) return CSWAP_E_ARG;
   if (maxbits < 16 || maxbits > 4096) return CSWAP_E_ARG;
   if (nx > 0x7fffffffu || ny > 0x7fffffffu || nz > 0x7fffffffu) return CSWAP_E_ARG;
@@ -192,6 +233,7 @@ static int make_field(Field3& fd, const void* base, size_t nx, size_t ny, size_t
   fd.sy = sy ? sy : (ptrdiff_t)nx;
   fd.sz = sz ? sz : (ptrdiff_t)(nx * ny);
   fd.rows16 = fd.sx == 1 && (fd.sy % 4) == 0 && (fd.sz % 4) == 0 && ((uintptr_t)base % 16) == 0;
+  fd.stream16 = ((uintptr_t)stream % 16) == 0;
   return CSWAP_OK;
 }
 
@@ -217,12 +259,16 @@ extern "C" int cswap_zfp_compress_f32(const float* d_in, size_t nx, size_t ny, s
 {
   if (!d_in || !d_stream) return CSWAP_E_ARG;
   Field3 fd;
-  int rc = make_field(fd, d_in, nx, ny, nz, sx, sy, sz, maxbits);
+  int rc = make_field(fd, d_in, d_stream, nx, ny, nz, sx, sy, sz, maxbits);
   if (rc) return rc;
   unsigned grid = (fd.nblocks + 63) / 64;
-  size_t lds_bytes = ((size_t)maxbits + 1) * 8;
-  hipLaunchKernelGGL(zfp_encode3_f32_kernel, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream, d_in, fd,
-                     maxbits, d_stream);
+  size_t lds_bytes = (size_t)region_dwords(maxbits) * 4;
+  if ((maxbits & 63u) == 0)
+    hipLaunchKernelGGL(zfp_encode3_f32_kernel<true>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
+                       d_in, fd, maxbits, d_stream);
+  else
+    hipLaunchKernelGGL(zfp_encode3_f32_kernel<false>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
+                       d_in, fd, maxbits, d_stream);
   return check_launch();
 }
 
@@ -232,11 +278,15 @@ extern "C" int cswap_zfp_decompress_f32(const uint64_t* d_stream, size_t nx, siz
 {
   if (!d_out || !d_stream) return CSWAP_E_ARG;
   Field3 fd;
-  int rc = make_field(fd, d_out, nx, ny, nz, sx, sy, sz, maxbits);
+  int rc = make_field(fd, d_out, d_stream, nx, ny, nz, sx, sy, sz, maxbits);
   if (rc) return rc;
   unsigned grid = (fd.nblocks + 63) / 64;
-  size_t lds_bytes = ((size_t)maxbits + 1) * 8;
-  hipLaunchKernelGGL(zfp_decode3_f32_kernel, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream, d_stream,
-                     fd, maxbits, d_out);
+  size_t lds_bytes = (size_t)region_dwords(maxbits) * 4;
+  if ((maxbits & 63u) == 0)
+    hipLaunchKernelGGL(zfp_decode3_f32_kernel<true>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
+                       d_stream, fd, maxbits, d_out);
+  else
+    hipLaunchKernelGGL(zfp_decode3_f32_kernel<false>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
+                       d_stream, fd, maxbits, d_out);
   return check_launch();
 }

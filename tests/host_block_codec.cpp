@@ -7,28 +7,16 @@
 #include "../cswap_amd/csrc/zfp_block.h"
 
 namespace {
-struct ArraySink {            // ORs block-relative words into the global stream
-  uint64_t* words; size_t bit0;
-  void put(unsigned j, uint64_t w) {
-    size_t p = bit0 + 64 * (size_t)j; size_t i = p >> 6; unsigned s = p & 63;
-    words[i] |= w << s;
-    if (s) words[i + 1] |= w >> (64 - s);
-  }
-};
-struct ArraySource {
-  const uint64_t* words; size_t bit0;
-  uint64_t window(unsigned pos) const {
-    size_t p = bit0 + pos; size_t i = p >> 6; unsigned s = p & 63;
-    uint64_t v = words[i] >> s;
-    if (s) v |= words[i + 1] << (64 - s);
-    return v;
-  }
+struct ArrayBits {            // the bit region is the whole stream, addressed in dwords
+  uint32_t* dw;
+  void or32(unsigned d, uint32_t v) const { dw[d] |= v; }
+  uint32_t ld32(unsigned d) const { return dw[d]; }
 };
 }
 
 extern "C" {
 
-// stream must hold ceil(blocks*maxbits/64)+1 zeroed words
+// stream must hold ceil(blocks*maxbits/64)+2 zeroed words (the codec may touch 96 bits past a block)
 void host_zfp_encode3(const float* in, size_t nx, size_t ny, size_t nz, unsigned maxbits, uint64_t* stream)
 {
   size_t mx = (nx + 3) / 4, my = (ny + 3) / 4, mz = (nz + 3) / 4;
@@ -40,8 +28,8 @@ void host_zfp_encode3(const float* in, size_t nx, size_t ny, size_t nz, unsigned
     for (unsigned z = 0; z < bz; z++) for (unsigned y = 0; y < by; y++) for (unsigned x = 0; x < bx; x++)
       f[x + 4 * y + 16 * z] = in[(x0 + x) + nx * ((y0 + y) + ny * (z0 + z))];
     if (bx < 4 || by < 4 || bz < 4) cswap::pad_block3(f, bx, by, bz);
-    ArraySink sink{stream, b * (size_t)maxbits};
-    cswap::encode_block(f, maxbits, sink);
+    ArrayBits mem{reinterpret_cast<uint32_t*>(stream)};
+    cswap::encode_block<true>(f, (unsigned)(b * (size_t)maxbits), maxbits, mem);
   }
 }
 
@@ -52,8 +40,8 @@ void host_zfp_decode3(const uint64_t* stream, size_t nx, size_t ny, size_t nz, u
     size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
     unsigned bx = nx - x0 < 4 ? nx - x0 : 4, by = ny - y0 < 4 ? ny - y0 : 4, bz = nz - z0 < 4 ? nz - z0 : 4;
     float f[64];
-    ArraySource src{stream, b * (size_t)maxbits};
-    cswap::decode_block(src, maxbits, f);
+    ArrayBits mem{reinterpret_cast<uint32_t*>(const_cast<uint64_t*>(stream))};
+    cswap::decode_block(mem, (unsigned)(b * (size_t)maxbits), maxbits, f);
     for (unsigned z = 0; z < bz; z++) for (unsigned y = 0; y < by; y++) for (unsigned x = 0; x < bx; x++)
       out[(x0 + x) + nx * ((y0 + y) + ny * (z0 + z))] = f[x + 4 * y + 16 * z];
   }

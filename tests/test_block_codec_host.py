@@ -41,13 +41,13 @@ def test_block_codec_matches_golden_vectors(host, golden):
         nz, ny, nx = f.shape
         blocks = -(-nx // 4) * -(-ny // 4) * -(-nz // 4)
         words = (blocks * maxbits + 63) // 64
-        s = np.zeros(words + 1, dtype=np.uint64)
+        s = np.zeros(words + 2, dtype=np.uint64)
         host.host_zfp_encode3(f.ctypes.data, nx, ny, nz, maxbits, s.ctypes.data)
         sb = s[:words].view(np.uint8)
         k = min(sb.size, stream.size)
         assert np.array_equal(sb[:k], stream[:k]), (name, rate)
         assert not sb[k:].any() and not stream[k:].any()
-        g = np.zeros((words + 1) * 8, dtype=np.uint8)
+        g = np.zeros((words + 2) * 8, dtype=np.uint8)
         g[:k] = stream[:k]
         o = np.zeros_like(f)
         host.host_zfp_decode3(g.ctypes.data, nx, ny, nz, maxbits, o.ctypes.data)
