@@ -123,11 +123,14 @@ CSWAP_HD void fwd_lift4(int32_t& x, int32_t& y, int32_t& z, int32_t& w)
 
 CSWAP_HD void inv_lift4(int32_t& x, int32_t& y, int32_t& z, int32_t& w)
 {
+  // The reference's steps of the form "a += b; b <<= 1; b -= a" (shared.h:241-245)
+  // leave a' = a + b and b' = 2b - (a + b) = b - a: two operations in wrap-around
+  // arithmetic instead of three.
   y = wadd(y, w >> 1); w = wsub(w, y >> 1);
-  y = wadd(y, w); w = wdbl(w); w = wsub(w, y);
-  z = wadd(z, x); x = wdbl(x); x = wsub(x, z);
-  y = wadd(y, z); z = wdbl(z); z = wsub(z, y);
-  w = wadd(w, x); x = wdbl(x); x = wsub(x, w);
+  { int32_t y0 = y; y = wadd(y, w); w = wsub(w, y0); }
+  { int32_t z0 = z; z = wadd(z, x); x = wsub(x, z0); }
+  { int32_t y0 = y; y = wadd(y, z); z = wsub(z, y0); }
+  { int32_t w0 = w; w = wadd(w, x); x = wsub(x, w0); }
 }
 
 // b[x + 4y + 16z]; forward order x, y, z; inverse z, y, x

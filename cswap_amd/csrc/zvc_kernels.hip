@@ -70,38 +70,73 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_count_kernel(const fl
 }
 
 // ------------------------------------------------------------------ scan
-// In-place exclusive scan of k ints by one workgroup; total to *nnz.
+// In-place exclusive scan of k ints by one workgroup of 1024 threads; total to
+// *nnz.  Each thread owns 16 consecutive entries per 16384-entry tile.
 __global__ __launch_bounds__(1024) void zvc_scan_kernel(int* __restrict__ v, int k, int* __restrict__ nnz)
 {
   __shared__ int wave_tot[16];
-  __shared__ int carry_s;
   const unsigned tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6;
-  if (tid == 0) carry_s = 0;
-  __syncthreads();
-  for (int base = 0; base < k; base += 1024) {
-    int i = base + (int)tid;
-    int x = i < k ? v[i] : 0;
-    // inclusive scan inside the wave
-    int s = x;
+  int carry = 0;
+  for (int base = 0; base < k; base += 16384) {
+    const int i0 = base + (int)tid * 16;
+    int x[16];
+    if (i0 + 16 <= k) {
+      const int4* p = reinterpret_cast<const int4*>(v + i0);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        int4 q = p[j];
+        x[4 * j] = q.x; x[4 * j + 1] = q.y; x[4 * j + 2] = q.z; x[4 * j + 3] = q.w;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 16; j++) x[j] = i0 + j < k ? v[i0 + j] : 0;
+    }
+    int tsum = 0;
+#pragma unroll
+    for (int j = 0; j < 16; j++) tsum += x[j];
+    int s = tsum;  // inclusive scan of thread sums inside the wave
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
       int t = __shfl_up(s, o, 64);
       if ((int)lane >= o) s += t;
     }
+    __syncthreads();  // wave_tot of the previous tile has been consumed
     if (lane == 63) wave_tot[wv] = s;
     __syncthreads();
-    int wave_off = 0;
-    for (unsigned w = 0; w < wv; w++) wave_off += wave_tot[w];
-    int carry = carry_s;
-    if (i < k) v[i] = carry + wave_off + s - x;
-    __syncthreads();
-    if (tid == 1023) carry_s = carry + wave_off + s;
-    __syncthreads();
+    int wave_off = 0, total = 0;
+#pragma unroll
+    for (unsigned w = 0; w < 16; w++) {
+      int t = wave_tot[w];
+      if (w < wv) wave_off += t;
+      total += t;
+    }
+    int run = carry + wave_off + s - tsum;
+    if (i0 + 16 <= k) {
+      int4* p = reinterpret_cast<int4*>(v + i0);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        int4 q;
+        q.x = run; run += x[4 * j];
+        q.y = run; run += x[4 * j + 1];
+        q.z = run; run += x[4 * j + 2];
+        q.w = run; run += x[4 * j + 3];
+        p[j] = q;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 16; j++) {
+        if (i0 + j < k) v[i0 + j] = run;
+        run += x[j];
+      }
+    }
+    carry += total;
   }
-  if (tid == 0) *nnz = carry_s;
+  if (tid == 0) *nnz = carry;
 }
 
 // ------------------------------------------------------------------ compact
+constexpr int kUnroll = 8;  // independent 256-byte rows in flight per wave
+
 __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_compact_kernel(
     const float* __restrict__ in, Geometry g, const int* __restrict__ begin, float* __restrict__ values,
     uint32_t* __restrict__ mask)
@@ -120,22 +155,30 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_compact_kernel(
   unsigned off = (unsigned)begin[c];
   const int iters = (g.E + 63) >> 6;
   uint32_t held = 0;  // lane l holds mask word (64*(t/32) + l) of the chunk until flushed
-  for (int t = 0; t < iters; t++) {
-    const int k = t * 64 + (int)lane;
-    const bool valid = k < len;
-    const float x = valid ? p[k] : 0.0f;
-    const bool nz = valid && (x != 0.0f);
-    const unsigned long long m = __ballot(nz);
-    if (nz) values[off + rank_below(m)] = x;
-    off += popc64(m);
-    const unsigned slot = (unsigned)(2 * t) & 63u;
-    if (lane == slot) held = (uint32_t)m;
-    if (lane == slot + 1) held = (uint32_t)(m >> 32);
-    if ((t & 31) == 31 || t == iters - 1) {
-      const int w = (t >> 5) * 64 + (int)lane;
-      const int filled = 2 * (t & 31) + 2;
-      if ((int)lane < filled && w < g.W) mrow[w] = held;
-      held = 0;
+  for (int t0 = 0; t0 < iters; t0 += kUnroll) {
+    float x[kUnroll];
+#pragma unroll
+    for (int j = 0; j < kUnroll; j++) {
+      const int k = (t0 + j) * 64 + (int)lane;
+      x[j] = k < len ? p[k] : 0.0f;  // out-of-range elements read as zero: no bit, no value
+    }
+#pragma unroll
+    for (int j = 0; j < kUnroll; j++) {
+      const int t = t0 + j;
+      const bool nz = x[j] != 0.0f;
+      const unsigned long long m = __ballot(nz);
+      if (nz) values[off + rank_below(m)] = x[j];
+      off += popc64(m);
+      if (t >= iters) continue;  // tail of the unrolled group: nothing left in this chunk
+      const unsigned slot = (unsigned)(2 * t) & 63u;
+      if (lane == slot) held = (uint32_t)m;
+      if (lane == slot + 1) held = (uint32_t)(m >> 32);
+      if ((t & 31) == 31 || t == iters - 1) {
+        const int w = (t >> 5) * 64 + (int)lane;
+        const int filled = 2 * (t & 31) + 2;
+        if ((int)lane < filled && w < g.W) mrow[w] = held;
+        held = 0;
+      }
     }
   }
 }
@@ -155,23 +198,30 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand_kernel(
   unsigned off = (unsigned)begin[c];
   const int iters = (len + 63) >> 6;
   uint32_t held = 0;
-  for (int t = 0; t < iters; t++) {
-    if ((t & 31) == 0) {  // refill: lane l takes mask word 64*(t/32)+l of this chunk
-      const int w = (t >> 5) * 64 + (int)lane;
+  for (int t0 = 0; t0 < iters; t0 += kUnroll) {
+    if ((t0 & 31) == 0) {  // refill: lane l takes mask word 64*(t0/32)+l of this chunk
+      const int w = (t0 >> 5) * 64 + (int)lane;
       held = w < g.W ? mrow[w] : 0u;
     }
-    const unsigned slot = (unsigned)(2 * t) & 63u;
-    const uint32_t lo = (uint32_t)__shfl((int)held, (int)slot, 64);
-    const uint32_t hi = (uint32_t)__shfl((int)held, (int)slot + 1, 64);
-    const int k = t * 64 + (int)lane;
-    // bits past the end of the chunk carry no data
-    const int rem = len - t * 64;
-    unsigned long long m = ((unsigned long long)hi << 32) | lo;
-    if (rem < 64) m &= (1ull << rem) - 1ull;
-    const bool nz = (m >> lane) & 1ull;
-    const float x = nz ? values[off + rank_below(m)] : 0.0f;
-    if (k < len) q[k] = x;
-    off += popc64(m);
+    float x[kUnroll];
+#pragma unroll
+    for (int j = 0; j < kUnroll; j++) {
+      const int t = t0 + j;
+      const int slot = (2 * t) & 63;
+      const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)held, slot);
+      const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)held, slot + 1);
+      unsigned long long m = ((unsigned long long)hi << 32) | lo;
+      const int rem = len - t * 64;  // bits past the end of the chunk carry no data
+      if (rem < 64) m = rem > 0 ? (m & ((1ull << rem) - 1ull)) : 0ull;
+      const bool nz = (m >> lane) & 1ull;
+      x[j] = nz ? values[off + rank_below(m)] : 0.0f;
+      off += popc64(m);
+    }
+#pragma unroll
+    for (int j = 0; j < kUnroll; j++) {
+      const int k = (t0 + j) * 64 + (int)lane;
+      if (k < len) q[k] = x[j];
+    }
   }
 }
 
