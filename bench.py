@@ -50,6 +50,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch one plain copy kernel of the same tensor (known traffic: 4N read, 4N "
+                         "written) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE can be scaled")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; run with --gpus 1 "
@@ -81,6 +84,9 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    if args.copy_probe:
+        out.copy_(x)
+        torch.cuda.synchronize()
 
     # ---- timed region: exactly K steps, per-kernel HIP events inside it
     evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]

@@ -29,6 +29,8 @@ class Costs(C.Structure):
                 ("kernel_latency_us", C.c_double), ("zvc_compress_gbs", C.c_double),
                 ("zvc_expand_gbs", C.c_double), ("zfp_compress_gbs", C.c_double),
                 ("zfp_decompress_gbs", C.c_double), ("sparse_max_ratio", C.c_double), ("lossy_min_gain", C.c_double),
+                ("probe_latency_us", C.c_double), ("probe_gbs", C.c_double), ("min_gain", C.c_double),
+                ("d2h_hidden", C.c_int),
                 ("size_floor_bytes", C.c_size_t), ("allow_lossy", C.c_int), ("process", C.c_int)]
 
 
@@ -85,6 +87,7 @@ _SIGNATURES = {
     "cswap_costs_default": (None, [C.POINTER(Costs)]),
     "cswap_policy_bytes": (sz, [i32, sz, sz, u, i32, sz, sz, sz]),
     "cswap_select": (i32, [sz, sz, u, C.POINTER(Costs), C.POINTER(Choice)]),
+    "cswap_select_field": (i32, [sz, sz, sz, sz, u, C.POINTER(Costs), C.POINTER(Choice)]),
     "cswap_engine_config_default": (None, [C.POINTER(EngineConfig)]),
     "cswap_engine_create": (i32, [C.POINTER(vp), C.POINTER(EngineConfig)]),
     "cswap_engine_destroy": (None, [vp]),

@@ -23,6 +23,10 @@ extern "C" void cswap_costs_default(cswap_costs* c)
   c->zfp_decompress_gbs = 1900.0;
   c->sparse_max_ratio = 0.90;
   c->lossy_min_gain = 0.5;
+  c->probe_latency_us = 30.0;
+  c->probe_gbs = 4000.0;
+  c->min_gain = 0.75;
+  c->d2h_hidden = 1;
   c->size_floor_bytes = 256 * 1024;
   c->allow_lossy = 1;
   c->process = 512 * 32;
@@ -46,39 +50,49 @@ extern "C" size_t cswap_policy_bytes(int policy, size_t n, size_t nnz, unsigned 
   }
 }
 
-extern "C" int cswap_select(size_t n, size_t nnz, unsigned maxbits, const cswap_costs* costs, cswap_choice* out)
+static int select_core(size_t n, size_t nnz, size_t b_zfp, const cswap_costs* costs, cswap_choice* out)
 {
   if (!out || !n || nnz > n) return CSWAP_E_ARG;
   cswap_costs c;
   if (costs) c = *costs; else cswap_costs_default(&c);
   if (c.bw_d2h_gbs <= 0 || c.bw_h2d_gbs <= 0) return CSWAP_E_ARG;
   const double in_bytes = 4.0 * (double)n;
+  // With d2h_hidden the outbound copy is taken to overlap with the layer's
+  // compute (what the copy stream is for), so only the inbound copy is on the
+  // critical path: the conservative view for a compressed option, whose kernels
+  // and probe are not hidden.
   auto link_us = [&](double bytes) {
-    return 2.0 * c.copy_latency_us + bytes / (c.bw_d2h_gbs * 1e3) + bytes / (c.bw_h2d_gbs * 1e3);
+    double t = c.copy_latency_us + bytes / (c.bw_h2d_gbs * 1e3);
+    if (!c.d2h_hidden) t += c.copy_latency_us + bytes / (c.bw_d2h_gbs * 1e3);
+    return t;
   };
   const double inf = 1e300;
+  // what deciding costs: the counting pass plus one host round trip for nnz; the
+  // raw swap does not pay it, so every compressed option carries it
+  const double t_probe = c.probe_latency_us + (c.probe_gbs > 0 ? in_bytes / (c.probe_gbs * 1e3) : 0.0);
   double t_none = link_us(in_bytes);
   double t_sparse = inf, t_zfp = inf;
-  size_t b_sparse = 0, b_zfp = 0;
+  size_t b_sparse = 0;
 
   if (n <= 0x7fffffffull && c.process > 0 && c.zvc_compress_gbs > 0 && c.zvc_expand_gbs > 0) {
-    b_sparse = cswap_policy_bytes(CSWAP_POLICY_SPARSE, n, nnz, maxbits, c.process, 0, 0, 0);
+    b_sparse = cswap_policy_bytes(CSWAP_POLICY_SPARSE, n, nnz, 0, c.process, 0, 0, 0);
     if ((double)b_sparse < c.sparse_max_ratio * in_bytes)
-      t_sparse = 4.0 * c.kernel_latency_us + in_bytes / (c.zvc_compress_gbs * 1e3) +
+      t_sparse = t_probe + 4.0 * c.kernel_latency_us + in_bytes / (c.zvc_compress_gbs * 1e3) +
                  in_bytes / (c.zvc_expand_gbs * 1e3) + link_us((double)b_sparse);
   }
-  if (c.allow_lossy && maxbits >= 16 && maxbits <= 4096 && c.zfp_compress_gbs > 0 && c.zfp_decompress_gbs > 0) {
-    b_zfp = cswap_policy_bytes(CSWAP_POLICY_ZFP, n, nnz, maxbits, c.process, 0, 0, 0);
+  if (c.allow_lossy && b_zfp && c.zfp_compress_gbs > 0 && c.zfp_decompress_gbs > 0) {
     if ((double)b_zfp < in_bytes)
-      t_zfp = 2.0 * c.kernel_latency_us + in_bytes / (c.zfp_compress_gbs * 1e3) +
+      t_zfp = t_probe + 2.0 * c.kernel_latency_us + in_bytes / (c.zfp_compress_gbs * 1e3) +
               in_bytes / (c.zfp_decompress_gbs * 1e3) + link_us((double)b_zfp);
   }
 
   int pol = CSWAP_POLICY_NONE;
   double best = t_none;
   if ((size_t)in_bytes >= c.size_floor_bytes) {
-    if (t_sparse < best) { best = t_sparse; pol = CSWAP_POLICY_SPARSE; }   // strict: ties stay lossless/raw
-    const double need = pol == CSWAP_POLICY_SPARSE ? c.lossy_min_gain * best : best;
+    const double gain = c.min_gain > 0 && c.min_gain <= 1.0 ? c.min_gain : 1.0;
+    double bar = gain * t_none;            // a compressed option must beat the raw swap by this margin
+    if (t_sparse < bar) { best = t_sparse; pol = CSWAP_POLICY_SPARSE; }   // strict: ties stay raw
+    const double need = pol == CSWAP_POLICY_SPARSE ? c.lossy_min_gain * best : bar;
     if (t_zfp < need) { best = t_zfp; pol = CSWAP_POLICY_ZFP; }
   }
   out->policy = pol;
@@ -88,4 +102,22 @@ extern "C" int cswap_select(size_t n, size_t nnz, unsigned maxbits, const cswap_
   out->t_sparse_us = t_sparse >= inf ? -1.0 : t_sparse;
   out->t_zfp_us = t_zfp >= inf ? -1.0 : t_zfp;
   return CSWAP_OK;
+}
+
+extern "C" int cswap_select(size_t n, size_t nnz, unsigned maxbits, const cswap_costs* costs, cswap_choice* out)
+{
+  size_t b_zfp = 0;
+  if (maxbits >= 16 && maxbits <= 4096) b_zfp = cswap_policy_bytes(CSWAP_POLICY_ZFP, n, 0, maxbits, 0, 0, 0, 0);
+  return select_core(n, nnz, b_zfp, costs, out);
+}
+
+extern "C" int cswap_select_field(size_t nx, size_t ny, size_t nz, size_t nnz, unsigned maxbits,
+                                  const cswap_costs* costs, cswap_choice* out)
+{
+  if (!nx || !ny || !nz) return CSWAP_E_ARG;
+  size_t n = nx * ny * nz;
+  if (n / nz != nx * ny) return CSWAP_E_ARG;
+  size_t b_zfp = 0;
+  if (maxbits >= 16 && maxbits <= 4096) b_zfp = cswap_zfp_stream_capacity(nx, ny, nz, maxbits);
+  return select_core(n, nnz, b_zfp, costs, out);
 }

@@ -14,6 +14,7 @@
 // the pinned allocator per tensor, Execution.h:76,97-99,114); several tensors
 // can be in flight at once (the reference has one dataptr_/buffer per Execution,
 // Execution.h:432-441).
+#include <chrono>
 #include <map>
 #include <mutex>
 #include <new>
@@ -229,7 +230,18 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   t.dev_held = false;
 
   int rc;
-  const bool want_probe = (policy == CSWAP_POLICY_AUTO && zvc_ok) || policy == CSWAP_POLICY_SPARSE;
+  bool want_probe = (policy == CSWAP_POLICY_AUTO && zvc_ok) || policy == CSWAP_POLICY_SPARSE;
+  if (policy == CSWAP_POLICY_AUTO) {
+    // Do not even probe a tensor that cannot pay for it: if neither ZFP nor the
+    // best conceivable ZVC outcome (all zeros) is modelled to beat the raw swap,
+    // the raw swap it is.
+    cswap_choice best_case;
+    if ((rc = cswap_select_field(nx, ny, nz, 0, e->maxbits, &e->costs, &best_case))) return rc;
+    if (best_case.policy == CSWAP_POLICY_NONE) {
+      policy = t.policy = CSWAP_POLICY_NONE;
+      want_probe = false;
+    }
+  }
   if (want_probe) {
     // Worst-case ZVC staging; the chunk counts go straight into its header so
     // that a later compaction needs no second counting pass.
@@ -261,7 +273,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     cswap_choice ch;
     cswap_costs c = e->costs;
     if (!t.dev_held) c.sparse_max_ratio = 0.0;  // not probed: ZVC is not an option
-    if ((rc = cswap_select(n, t.nnz, e->maxbits, &c, &ch))) { drop_device(e, t); return rc; }
+    if ((rc = cswap_select_field(nx, ny, nz, t.nnz, e->maxbits, &c, &ch))) { drop_device(e, t); return rc; }
     t.policy = ch.policy;
   }
 
@@ -514,6 +526,28 @@ extern "C" int cswap_engine_calibrate(cswap_engine* e, cswap_costs* out_costs)
     if ((rc = ms(fdc, 2, &t))) break;
     if ((rc = ms(fdc, 10, &t))) break;
     c.zfp_decompress_gbs = gb / (t * 1e-3);
+    // the probe: counting pass throughput, and the fixed cost of count + scan +
+    // 4-byte copy + host wait measured on a tensor too small to matter
+    auto cnt = [&]() { return cswap_zvc_count(d_x, (int)n, e->process, d_begin, s); };
+    if ((rc = ms(cnt, 2, &t))) break;
+    if ((rc = ms(cnt, 10, &t))) break;
+    c.probe_gbs = gb / (t * 1e-3);
+    {
+      const int small_n = 1 << 16, reps = 10;
+      hipError_t er2 = hipStreamSynchronize(s);
+      auto t0 = std::chrono::steady_clock::now();
+      for (int i = 0; i < reps && er2 == hipSuccess && !rc; i++) {
+        rc = cswap_zvc_count(d_x, small_n, e->process, d_begin, s);
+        if (!rc) rc = cswap_zvc_scan(d_begin, cswap_zvc_active_chunks(small_n, e->process), e->d_nnz, s);
+        if (!rc) er2 = hipMemcpyAsync(e->h_nnz, e->d_nnz, sizeof(int), hipMemcpyDeviceToHost, s);
+        if (!rc && er2 == hipSuccess) er2 = hipEventRecord(e->ev_probe, s);
+        if (!rc && er2 == hipSuccess) er2 = hipEventSynchronize(e->ev_probe);
+      }
+      auto t1 = std::chrono::steady_clock::now();
+      if (rc) break;
+      if (er2 != hipSuccess) { rc = hip_fail(er2); break; }
+      c.probe_latency_us = std::chrono::duration<double, std::micro>(t1 - t0).count() / reps;
+    }
     e->costs = c;
   } while (0);
   (void)hipStreamSynchronize(s);

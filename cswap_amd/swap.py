@@ -33,6 +33,13 @@ def select(n: int, nnz: int, maxbits: int = 512, costs: Costs | None = None) -> 
     return ch
 
 
+def select_field(nx: int, ny: int, nz: int, nnz: int, maxbits: int = 512, costs: Costs | None = None) -> Choice:
+    ch = Choice()
+    check(lib().cswap_select_field(nx, ny, nz, nnz, maxbits, C.byref(costs) if costs is not None else None,
+                                   C.byref(ch)), "cswap_select_field")
+    return ch
+
+
 class SwapEngine:
     def __init__(self, pinned_bytes: int = 1 << 30, device_bytes: int = 1 << 30, maxbits: int = 512,
                  process: int = 512 * 32, max_tickets: int = 256, costs: Costs | None = None):
@@ -120,7 +127,7 @@ def bench_schedule(dev, batch: int = 128, seed: int = 0) -> dict:
         chosen = None
         for label, pol in (("none", NONE), ("auto", AUTO)):
             best = None
-            for _ in range(3):
+            for _ in range(5):
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
                 tk = eng.pre(x, pol)

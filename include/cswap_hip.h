@@ -114,8 +114,10 @@ int cswap_probe_nnz(const float* d_in, size_t n, unsigned long long* d_nnz, cswa
  * describes it as weighing compression ratio, size and algorithm
  * characteristics at run time.  This one minimises a modelled swap-out +
  * swap-in latency:  t(option) = t_compress + bytes_out/bw_d2h + bytes_out/bw_h2d
- * + t_decompress (+ fixed per-kernel and per-copy overheads), with kernel times
- * = bytes_in / throughput.  Ties go to the lossless option; ZVC is only
+ * + t_decompress (+ fixed per-kernel and per-copy overheads, + the cost of the
+ * probe itself for the compressed options), with kernel times
+ * = bytes_in / throughput; a compressed option is taken only if it is modelled
+ * faster than min_gain * the raw swap.  Ties go to the lossless option; ZVC is only
  * eligible when its size ratio is below sparse_max_ratio; tensors below
  * size_floor_bytes are never compressed.  Lossless is preferred: when ZVC beats
  * the raw swap, lossy ZFP replaces it only if it is modelled at least
@@ -134,6 +136,11 @@ typedef struct {
   double zfp_compress_gbs, zfp_decompress_gbs;
   double sparse_max_ratio;               /* ZVC eligible only below this size ratio */
   double lossy_min_gain;                 /* ZFP replaces a winning ZVC only if t_zfp < gain * t_zvc */
+  double probe_latency_us;               /* fixed cost of deciding: counting kernels + host round trip */
+  double probe_gbs;                      /* throughput of the counting pass, GB/s of fp32 in */
+  double min_gain;                       /* compress only if modelled time < min_gain * raw swap time */
+  int    d2h_hidden;                     /* 1: assume the outbound copy overlaps compute (only the
+                                            inbound copy, kernels and probe are on the critical path) */
   size_t size_floor_bytes;               /* never compress smaller tensors */
   int    allow_lossy;                    /* 0: ZFP is never chosen */
   int    process;                        /* ZVC chunk count (512*32 in the reference) */
@@ -151,8 +158,13 @@ void cswap_costs_default(cswap_costs* c);
 /* Bytes a tensor of n elements with nnz non-zeros occupies under each policy. */
 size_t cswap_policy_bytes(int policy, size_t n, size_t nnz, unsigned maxbits, int process,
                           size_t nx, size_t ny, size_t nz);
-/* Pure host function, no GPU work. */
+/* Pure host functions, no GPU work.  cswap_select sees a flat tensor (ZFP size
+ * = ceil(n/64) blocks); cswap_select_field uses the true block count of the
+ * field a[nz][ny][nx], which matters when nx or ny is not a multiple of 4
+ * (a 2x2xN field pays the full rate for blocks that are 3/4 padding). */
 int cswap_select(size_t n, size_t nnz, unsigned maxbits, const cswap_costs* costs, cswap_choice* out);
+int cswap_select_field(size_t nx, size_t ny, size_t nz, size_t nnz, unsigned maxbits,
+                       const cswap_costs* costs, cswap_choice* out);
 
 /* ----------------------------------------------------------- swap engine -----
  * Mirror of Execution::init_/pre/post (Execution.h:46-133,217-310) and of the

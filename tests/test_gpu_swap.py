@@ -75,7 +75,8 @@ def test_auto_policy_follows_selector(torch_cuda, engine):
         engine.post(tk)
         info = engine.info(tk)
         assert info.policy == want
-        assert info.policy == swap.select(x.numel(), info.nnz).policy
+        from cswap_amd.workloads import field_dims
+        assert info.policy == swap.select_field(*field_dims(x.shape), info.nnz).policy
         out = torch.empty_like(x)
         engine.swap_in(tk, out)
         torch.cuda.synchronize()
@@ -133,8 +134,13 @@ def test_state_machine_errors(torch_cuda, engine):
     assert L.cswap_swap_out(engine._h, x.data_ptr(), 1 << 14, 1 << 14, 8, 2, None, C.byref(huge)) == -4
 
 
-def test_calibration_gives_sane_costs(torch_cuda, engine):
-    c = engine.calibrate()
+def test_calibration_gives_sane_costs(torch_cuda):
+    from cswap_amd import swap
+
+    eng = swap.SwapEngine(pinned_bytes=256 << 20, device_bytes=64 << 20)
+    c = eng.calibrate()
+    eng.close()
+    assert 1 < c.probe_latency_us < 1000 and c.probe_gbs > 100
     assert 5 < c.bw_d2h_gbs < 200 and 5 < c.bw_h2d_gbs < 200
     assert c.zfp_compress_gbs > 50 and c.zfp_decompress_gbs > 50
     assert c.zvc_compress_gbs > 50 and c.zvc_expand_gbs > 50

@@ -83,6 +83,29 @@ def test_chosen_option_never_modelled_slower_than_raw():
                 assert ch.t_zfp_us < c.lossy_min_gain * ch.t_sparse_us
 
 
+def test_partial_block_fields_pay_full_rate():
+    """A 2x2xN field (the [128,512,2,2] activation) fills only 1/4 of every 4x4x4
+    block: rate 8 gives no size gain, so ZFP must not be chosen for it."""
+    ch = swap.select_field(2, 2, 65536, 2 * 2 * 65536)
+    assert ch.policy == NONE
+    flat = swap.select(2 * 2 * 65536, 2 * 2 * 65536)
+    assert flat.bytes_out in (2 * 2 * 65536, 4 * 2 * 2 * 65536)
+    big = swap.select_field(2, 2, 1 << 24, 4 << 24)
+    assert big.policy == NONE and big.t_zfp_us == -1.0
+
+
+def test_margin_and_probe_cost_keep_small_tensors_raw():
+    c = swap.default_costs()
+    n = 1 << 20                                   # 4 MiB: the inbound copy takes ~85 us, the probe ~30 us
+    assert swap.select(n, n, costs=c).policy == NONE
+    assert swap.select(1 << 22, 1 << 22, costs=c).policy == ZFP    # 16 MiB pays
+    c.probe_latency_us = 0.0
+    c.min_gain = 1.0
+    assert swap.select(n, n, costs=c).policy == ZFP
+    c.min_gain = 0.1                              # demand a 10x gain: nothing qualifies
+    assert swap.select(1 << 26, 1 << 26, costs=c).policy == NONE
+
+
 def test_ties_stay_lossless():
     c = swap.default_costs()
     # an infinitely fast link makes all options equal up to kernel time: raw wins
