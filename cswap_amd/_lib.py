@@ -83,6 +83,8 @@ _SIGNATURES = {
     "cswap_zvc_compact": (i32, [vp, i32, i32, vp, vp, vp, vp]),
     "cswap_zvc_expand": (i32, [vp, vp, vp, i32, i32, vp, vp]),
     "cswap_zvc_compress": (i32, [vp, i32, i32, vp, vp, vp, vp, vp]),
+    "cswap_zvc_workspace_bytes": (sz, [i32]),
+    "cswap_zvc_compress_fused": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp]),
     "cswap_probe_nnz": (i32, [vp, sz, vp, vp]),
     "cswap_costs_default": (None, [C.POINTER(Costs)]),
     "cswap_policy_bytes": (sz, [i32, sz, sz, u, i32, sz, sz, sz]),

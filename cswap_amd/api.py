@@ -113,8 +113,9 @@ def GPUdecompression(values: torch.Tensor, dest: torch.Tensor, mask: torch.Tenso
                                  process, dest.data_ptr(), _stream()), "cswap_zvc_expand")
 
 
-def zvc_compress(t: torch.Tensor, process: int = PROCESS):
-    """count + scan + compact without a host round trip.  Returns
+def zvc_compress(t: torch.Tensor, process: int = PROCESS, fused: bool = False):
+    """count + scan + compact without a host round trip (``fused``: in a single
+    pass over the tensor).  Returns
     (values[n] (first nnz valid), mask uint32[W*process], begin int32[process], nnz int32[1])."""
     _need_f32_cuda(t)
     n = t.numel()
@@ -124,8 +125,14 @@ def zvc_compress(t: torch.Tensor, process: int = PROCESS):
     mask = torch.empty(W * process, dtype=torch.int32, device=dev)
     begin = torch.zeros(process, dtype=torch.int32, device=dev)
     nnz = torch.zeros(1, dtype=torch.int32, device=dev)
-    check(lib().cswap_zvc_compress(t.data_ptr(), n, process, begin.data_ptr(), nnz.data_ptr(),
-                                   values.data_ptr(), mask.data_ptr(), _stream()), "cswap_zvc_compress")
+    if fused:
+        ws = torch.empty(lib().cswap_zvc_workspace_bytes(process), dtype=torch.uint8, device=dev)
+        check(lib().cswap_zvc_compress_fused(t.data_ptr(), n, process, ws.data_ptr(), begin.data_ptr(),
+                                             nnz.data_ptr(), values.data_ptr(), mask.data_ptr(), _stream()),
+              "cswap_zvc_compress_fused")
+    else:
+        check(lib().cswap_zvc_compress(t.data_ptr(), n, process, begin.data_ptr(), nnz.data_ptr(),
+                                       values.data_ptr(), mask.data_ptr(), _stream()), "cswap_zvc_compress")
     return values, mask, begin, nnz
 
 

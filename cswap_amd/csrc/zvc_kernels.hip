@@ -225,6 +225,129 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand_kernel(
   }
 }
 
+// ------------------------------------------------------------------ fused
+// count + scan + compact in ONE pass over the tensor: a wavefront keeps its whole
+// chunk in registers (IT values per lane), counts it, obtains its exclusive
+// offset by a decoupled look-back over the chunk-granular status words and then
+// writes mask and packed values from the registers.  HBM traffic is the
+// algorithmic 4 + 1/8 + 4d bytes per element.
+//
+// Workspace (zeroed by zvc_ws_zero_kernel before every launch):
+//   ws[0]  ticket counter: chunks are handed out in the order waves start, so
+//          every chunk a wave waits for belongs to a wave that is already
+//          running (no dependence on the dispatch order of workgroups)
+//   ws[1]  error flag: set if a bounded wait ran out (never in a healthy run)
+//   ws[16 + c]  status of chunk c: bits 31..30 = 0 nothing yet, 1 = count of the
+//          chunk alone, 2 = inclusive prefix; bits 29..0 = the value
+constexpr uint32_t kFlagAgg = 1u << 30, kFlagPre = 2u << 30, kValMask = (1u << 30) - 1u;
+constexpr unsigned kSpinLimit = 1u << 22;
+
+__global__ void zvc_ws_zero_kernel(uint32_t* ws, int words)
+{
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < words) ws[i] = 0;
+}
+
+__device__ __forceinline__ uint32_t ld_status(const uint32_t* p)
+{
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_status(uint32_t* p, uint32_t v)
+{
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int IT>
+__global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_fused_kernel(
+    const float* __restrict__ in, Geometry g, uint32_t* __restrict__ ws, int* __restrict__ begin,
+    int* __restrict__ nnz, float* __restrict__ values, uint32_t* __restrict__ mask)
+{
+  const unsigned lane = lane_id();
+  uint32_t* status = ws + 16;
+  int c = 0;
+  if (lane == 0) c = (int)atomicAdd(&ws[0], 1u);
+  c = __builtin_amdgcn_readfirstlane(c);
+  if (c >= g.process) return;
+  uint32_t* mrow = mask + (size_t)c * g.W;
+  if (c >= g.active) {
+    for (int w = lane; w < g.W; w += 64) mrow[w] = 0;
+    return;
+  }
+  const long long b = (long long)g.E * c;
+  const int len = (int)min((long long)g.E, (long long)g.n - b);
+  const float* p = in + b;
+  const int iters = (g.E + 63) >> 6;  // <= IT
+
+  // ---- phase 1: the chunk into registers, and its count
+  float x[IT];
+#pragma unroll
+  for (int t = 0; t < IT; t++) {
+    const int k = t * 64 + (int)lane;
+    x[t] = (t < iters && k < len) ? p[k] : 0.0f;
+  }
+  unsigned agg = 0;
+#pragma unroll
+  for (int t = 0; t < IT; t++) agg += popc64(__ballot(x[t] != 0.0f));
+
+  // ---- decoupled look-back over the chunks before this one
+  unsigned excl = 0;
+  if (c == 0) {
+    if (lane == 0) st_status(&status[0], kFlagPre | agg);
+  } else {
+    if (lane == 0) st_status(&status[c], kFlagAgg | agg);
+    int idx = c - 1;
+    bool done = false;
+    while (!done) {
+      const int j = idx - (int)lane;
+      uint32_t v = kFlagPre;  // before the first chunk: prefix 0
+      unsigned spins = 0;
+      for (;;) {
+        if (j >= 0) v = ld_status(&status[j]);
+        if (__ballot((v >> 30) == 0u) == 0ull) break;
+        if (++spins > kSpinLimit) {  // give up: flag the error and make the wave finish
+          if (lane == 0) atomicOr(&ws[1], 1u);
+          v |= kFlagPre;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+      const unsigned long long pre = __ballot((v >> 30) == 2u);
+      unsigned take = 64;  // lanes 0..take-1 contribute
+      if (pre) { take = (unsigned)__builtin_ctzll(pre) + 1u; done = true; }
+      unsigned contrib = lane < take ? (v & kValMask) : 0u;
+      excl += (unsigned)wave_sum((int)contrib);
+      idx -= 64;
+    }
+    if (lane == 0) st_status(&status[c], kFlagPre | ((excl + agg) & kValMask));
+  }
+  if (lane == 0) {
+    begin[c] = (int)excl;
+    if (c == g.active - 1) *nnz = (int)(excl + agg);
+  }
+
+  // ---- phase 2: mask words and packed values from the registers
+  unsigned off = excl;
+  uint32_t held = 0;
+#pragma unroll
+  for (int t = 0; t < IT; t++) {
+    if (t < iters) {
+      const bool nz = x[t] != 0.0f;
+      const unsigned long long m = __ballot(nz);
+      if (nz) values[off + rank_below(m)] = x[t];
+      off += popc64(m);
+      const unsigned slot = (unsigned)(2 * t) & 63u;
+      if (lane == slot) held = (uint32_t)m;
+      if (lane == slot + 1) held = (uint32_t)(m >> 32);
+      if ((t & 31) == 31 || t == iters - 1) {
+        const int w = (t >> 5) * 64 + (int)lane;
+        const int filled = 2 * (t & 31) + 2;
+        if ((int)lane < filled && w < g.W) mrow[w] = held;
+        held = 0;
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------------ probe
 __global__ void zero_u64_kernel(unsigned long long* p) { *p = 0ull; }
 
@@ -345,6 +468,39 @@ extern "C" int cswap_zvc_compress(const float* d_in, int n, int process, int* d_
   rc = cswap_zvc_scan(d_begin, cswap_zvc_active_chunks(n, process), d_nnz, stream);
   if (rc) return rc;
   return cswap_zvc_compact(d_in, n, process, d_begin, d_values, d_mask, stream);
+}
+
+extern "C" size_t cswap_zvc_workspace_bytes(int process)
+{
+  return process > 0 ? ((size_t)process + 16) * sizeof(uint32_t) : 0;
+}
+
+extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, void* d_ws, int* d_begin,
+                                        int* d_nnz, float* d_values, uint32_t* d_mask, cswap_stream_t stream)
+{
+  if (!d_in || !d_ws || !d_begin || !d_nnz || !d_values || !d_mask) return CSWAP_E_ARG;
+  Geometry g;
+  int rc = make_geometry(g, n, process);
+  if (rc) return rc;
+  // chunks that do not fit a wavefront's registers, or prefixes that do not fit
+  // the 30-bit status value, take the three-kernel path
+  if (g.E > 64 * 128 || n >= (1 << 30)) return cswap_zvc_compress(d_in, n, process, d_begin, d_nnz, d_values, d_mask, stream);
+  uint32_t* ws = (uint32_t*)d_ws;
+  const int words = process + 16;
+  hipLaunchKernelGGL(zvc_ws_zero_kernel, dim3((words + 255) / 256), dim3(256), 0, (hipStream_t)stream, ws, words);
+  const unsigned grid = (g.process + kWavesPerGroup - 1) / kWavesPerGroup;
+  const dim3 blk(64 * kWavesPerGroup);
+  const int iters = (g.E + 63) >> 6;
+#define CSWAP_FUSED(IT_)                                                                                  \
+  hipLaunchKernelGGL(zvc_fused_kernel<IT_>, dim3(grid), blk, 0, (hipStream_t)stream, d_in, g, ws, d_begin, \
+                     d_nnz, d_values, d_mask)
+  if (iters <= 8) CSWAP_FUSED(8);
+  else if (iters <= 16) CSWAP_FUSED(16);
+  else if (iters <= 32) CSWAP_FUSED(32);
+  else if (iters <= 64) CSWAP_FUSED(64);
+  else CSWAP_FUSED(128);
+#undef CSWAP_FUSED
+  return check_launch();
 }
 
 extern "C" int cswap_probe_nnz(const float* d_in, size_t n, unsigned long long* d_nnz, cswap_stream_t stream)

@@ -102,6 +102,16 @@ int cswap_zvc_expand(const float* d_values, const uint32_t* d_mask, const int* d
 int cswap_zvc_compress(const float* d_in, int n, int process, int* d_begin, int* d_nnz,
                        float* d_values, uint32_t* d_mask, cswap_stream_t stream);
 
+/* The same result in a single pass over the tensor (each wavefront keeps its
+ * chunk in registers and finds its offset by a decoupled look-back), so HBM
+ * traffic is the algorithmic 4 + 1/8 + 4*density bytes per element.  d_ws is
+ * scratch of cswap_zvc_workspace_bytes(process) bytes, cleared by the call
+ * itself; calls that share a workspace must not overlap.  Tensors whose chunks
+ * exceed 8192 elements (n > 8192*process) fall back to the three-kernel path. */
+size_t cswap_zvc_workspace_bytes(int process);
+int cswap_zvc_compress_fused(const float* d_in, int n, int process, void* d_ws, int* d_begin,
+                             int* d_nnz, float* d_values, uint32_t* d_mask, cswap_stream_t stream);
+
 /* ---------------------------------------------------------------- probe -----
  * One fused read pass: *d_nnz = number of elements != 0 (the quantity the
  * reference derives from PreGPUcompression + PreAcc, Execution.h:89-92). */

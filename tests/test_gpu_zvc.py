@@ -15,11 +15,11 @@ def torch_cuda():
     return torch
 
 
-def run_gpu(torch, x, process=P):
+def run_gpu(torch, x, process=P, fused=False):
     from cswap_amd import api
 
     t = torch.from_numpy(x).cuda()
-    values, mask, begin, nnz = api.zvc_compress(t, process)
+    values, mask, begin, nnz = api.zvc_compress(t, process, fused=fused)
     out = torch.full_like(t, -1.0)                      # NOT pre-zeroed on purpose
     api.GPUdecompression(values, out, mask, begin, process)
     probe = api.probe_nnz(t)
@@ -66,6 +66,49 @@ def test_other_chunk_counts(torch_cuda, process):
     rng = np.random.default_rng(process)
     x = np.maximum(rng.standard_normal(300_001), 0).astype(np.float32)
     check_against_oracle(x, run_gpu(torch_cuda, x, process), process)
+
+
+@pytest.mark.parametrize("pct", [30, 50, 70, 90])
+def test_fused_single_pass_config2(torch_cuda, pct):
+    from cswap_amd.workloads import config2_tensor
+
+    x = config2_tensor(pct).reshape(-1)
+    check_against_oracle(x, run_gpu(torch_cuda, x, fused=True))
+
+
+@pytest.mark.parametrize("n,process", [(1, P), (33, P), (1000, P), (P - 1, P), (P + 1, P), (1_000_003, P),
+                                        (P * 62 + 17, P), (P * 96 + 5, P), (P * 2048, P), (P * 4100 + 3, P),
+                                        (300_001, 7), (64 * 9000 + 1, 64), (5000, 1)])
+def test_fused_single_pass_ragged(torch_cuda, n, process):
+    """Every register-tile size of the fused kernel (8..128 values per lane), the
+    fallback for chunks above 8192 elements, partial last chunks, idle chunks."""
+    rng = np.random.default_rng(n % 1000 + process)
+    x = (rng.standard_normal(n, dtype=np.float32) * (rng.random(n, dtype=np.float32) < 0.35)).astype(np.float32)
+    print("n", n, "process", process, flush=True)
+    check_against_oracle(x, run_gpu(torch_cuda, x, process, fused=True), process)
+
+
+def test_fused_repeated_calls_share_a_workspace(torch_cuda):
+    """The workspace is cleared by every call: back-to-back calls on one stream
+    with the same scratch buffer give the same result."""
+    torch = torch_cuda
+    from cswap_amd._lib import check, lib
+
+    L = lib()
+    ws = torch.empty(L.cswap_zvc_workspace_bytes(P), dtype=torch.uint8, device="cuda")
+    g = torch.Generator(device="cuda"); g.manual_seed(3)
+    outs = []
+    for rep, n in enumerate((P * 512, P * 64, P * 512)):
+        t = torch.relu(torch.randn(n, generator=g, device="cuda"))
+        values = torch.empty(n, device="cuda"); mask = torch.empty(n // 32, dtype=torch.int32, device="cuda")
+        begin = torch.zeros(P, dtype=torch.int32, device="cuda"); nnz = torch.zeros(1, dtype=torch.int32, device="cuda")
+        check(L.cswap_zvc_compress_fused(t.data_ptr(), n, P, ws.data_ptr(), begin.data_ptr(), nnz.data_ptr(),
+                                         values.data_ptr(), mask.data_ptr(), None), "fused")
+        torch.cuda.synchronize()
+        k = int(nnz.item())
+        assert k == int((t != 0).sum().item())
+        assert torch.equal(values[:k], t[t != 0])
+        assert int(ws.view(torch.int32)[1].item()) == 0      # no bounded wait ran out
 
 
 def test_special_values_and_extremes(torch_cuda):
@@ -117,7 +160,12 @@ def test_full_size_round_trip(torch_cuda):
 
     g = torch.Generator(device="cuda"); g.manual_seed(1)
     t = torch.relu(torch.randn(64 * 1024 * 1024, generator=g, device="cuda"))
+    v2, m2, b2, n2 = api.zvc_compress(t, fused=True)
     values, mask, begin, nnz = api.zvc_compress(t)
+    torch.cuda.synchronize()
+    k2 = int(n2.item())
+    assert k2 == int(nnz.item()) and torch.equal(m2, mask) and torch.equal(b2, begin)
+    assert torch.equal(v2[:k2], values[:k2])
     out = torch.full_like(t, 3.0)
     api.GPUdecompression(values, out, mask, begin)
     torch.cuda.synchronize()
