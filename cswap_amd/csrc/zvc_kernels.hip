@@ -227,18 +227,21 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand_kernel(
 
 // ------------------------------------------------------------------ fused
 // count + scan + compact in ONE pass over the tensor: a wavefront keeps its whole
-// chunk in registers (IT values per lane), counts it, obtains its exclusive
-// offset by a decoupled look-back over the chunk-granular status words and then
-// writes mask and packed values from the registers.  HBM traffic is the
-// algorithmic 4 + 1/8 + 4d bytes per element.
+// chunk in registers (IT values per lane) and counts it; the WAVES chunks of a
+// workgroup form a tile whose exclusive offset comes from a decoupled look-back
+// over tile-granular status words; then every wave writes mask and packed values
+// from its registers.  HBM traffic is the algorithmic 4 + 1/8 + 4d bytes per
+// element.  Tiles (not chunks) are the unit of the look-back, and one memory
+// round trip covers a window of 256 tiles, because a workgroup that starts while
+// thousands of others are in flight has to walk back over all of them.
 //
 // Workspace (zeroed by zvc_ws_zero_kernel before every launch):
-//   ws[0]  ticket counter: chunks are handed out in the order waves start, so
-//          every chunk a wave waits for belongs to a wave that is already
-//          running (no dependence on the dispatch order of workgroups)
+//   ws[0]  ticket counter: tiles are handed out in the order workgroups start,
+//          so every tile a workgroup waits for belongs to a workgroup that is
+//          already running (no dependence on the dispatch order)
 //   ws[1]  error flag: set if a bounded wait ran out (never in a healthy run)
-//   ws[16 + c]  status of chunk c: bits 31..30 = 0 nothing yet, 1 = count of the
-//          chunk alone, 2 = inclusive prefix; bits 29..0 = the value
+//   ws[16 + t]  status of tile t: bits 31..30 = 0 nothing yet, 1 = count of the
+//          tile alone, 2 = inclusive prefix; bits 29..0 = the value
 constexpr uint32_t kFlagAgg = 1u << 30, kFlagPre = 2u << 30, kValMask = (1u << 30) - 1u;
 constexpr unsigned kSpinLimit = 1u << 22;
 
@@ -257,24 +260,25 @@ __device__ __forceinline__ void st_status(uint32_t* p, uint32_t v)
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int IT>
-__global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_fused_kernel(
+template <int IT, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void zvc_fused_kernel(
     const float* __restrict__ in, Geometry g, uint32_t* __restrict__ ws, int* __restrict__ begin,
     int* __restrict__ nnz, float* __restrict__ values, uint32_t* __restrict__ mask)
 {
+  __shared__ unsigned s_agg[WAVES];
+  __shared__ unsigned s_tile;   // ticket, then the tile's exclusive offset
   const unsigned lane = lane_id();
+  const int wv = (int)(threadIdx.x >> 6);
   uint32_t* status = ws + 16;
-  int c = 0;
-  if (lane == 0) c = (int)atomicAdd(&ws[0], 1u);
-  c = __builtin_amdgcn_readfirstlane(c);
-  if (c >= g.process) return;
-  uint32_t* mrow = mask + (size_t)c * g.W;
-  if (c >= g.active) {
-    for (int w = lane; w < g.W; w += 64) mrow[w] = 0;
-    return;
-  }
+  if (threadIdx.x == 0) s_tile = atomicAdd(&ws[0], 1u);
+  __syncthreads();
+  const int tile = (int)s_tile;
+  const int c = tile * WAVES + wv;
+  const bool in_layout = c < g.process;
+  const bool has_data = c < g.active;
+
   const long long b = (long long)g.E * c;
-  const int len = (int)min((long long)g.E, (long long)g.n - b);
+  const int len = has_data ? (int)min((long long)g.E, (long long)g.n - b) : 0;
   const float* p = in + b;
   const int iters = (g.E + 63) >> 6;  // <= IT
 
@@ -288,45 +292,75 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_fused_kernel(
   unsigned agg = 0;
 #pragma unroll
   for (int t = 0; t < IT; t++) agg += popc64(__ballot(x[t] != 0.0f));
+  if (lane == 0) s_agg[wv] = agg;
+  __syncthreads();  // also orders the read of the ticket before s_tile is reused
 
-  // ---- decoupled look-back over the chunks before this one
-  unsigned excl = 0;
-  if (c == 0) {
-    if (lane == 0) st_status(&status[0], kFlagPre | agg);
-  } else {
-    if (lane == 0) st_status(&status[c], kFlagAgg | agg);
-    int idx = c - 1;
-    bool done = false;
-    while (!done) {
-      const int j = idx - (int)lane;
-      uint32_t v = kFlagPre;  // before the first chunk: prefix 0
-      unsigned spins = 0;
-      for (;;) {
-        if (j >= 0) v = ld_status(&status[j]);
-        if (__ballot((v >> 30) == 0u) == 0ull) break;
-        if (++spins > kSpinLimit) {  // give up: flag the error and make the wave finish
-          if (lane == 0) atomicOr(&ws[1], 1u);
-          v |= kFlagPre;
-          break;
+  // ---- wave 0: decoupled look-back over the tiles before this one
+  if (wv == 0) {
+    unsigned tile_agg = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; w++) tile_agg += s_agg[w];
+    unsigned excl = 0;
+    if (tile == 0) {
+      if (lane == 0) st_status(&status[0], kFlagPre | tile_agg);
+    } else {
+      if (lane == 0) st_status(&status[tile], kFlagAgg | tile_agg);
+      int idx = tile - 1;
+      bool done = false;
+      while (!done) {
+        // one round trip fetches a window of 256 predecessors (4 per lane)
+        uint32_t v[4];
+        unsigned spins = 0;
+        for (;;) {
+          bool missing = false;
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            const int j = idx - 64 * r - (int)lane;
+            v[r] = j >= 0 ? ld_status(&status[j]) : kFlagPre;  // before the first tile: prefix 0
+            missing |= (v[r] >> 30) == 0u;
+          }
+          if (__ballot(missing) == 0ull) break;
+          if (++spins > kSpinLimit) {  // give up: flag the error and let the grid drain
+            if (lane == 0) atomicOr(&ws[1], 1u);
+#pragma unroll
+            for (int r = 0; r < 4; r++) v[r] |= kFlagPre;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(1);
         }
-        __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          if (!done) {
+            const unsigned long long pre = __ballot((v[r] >> 30) == 2u);
+            unsigned take = 64;  // lanes 0..take-1 of this row contribute
+            if (pre) { take = (unsigned)__builtin_ctzll(pre) + 1u; done = true; }
+            unsigned contrib = lane < take ? (v[r] & kValMask) : 0u;
+            excl += (unsigned)wave_sum((int)contrib);
+          }
+        }
+        idx -= 256;
       }
-      const unsigned long long pre = __ballot((v >> 30) == 2u);
-      unsigned take = 64;  // lanes 0..take-1 contribute
-      if (pre) { take = (unsigned)__builtin_ctzll(pre) + 1u; done = true; }
-      unsigned contrib = lane < take ? (v & kValMask) : 0u;
-      excl += (unsigned)wave_sum((int)contrib);
-      idx -= 64;
+      if (lane == 0) st_status(&status[tile], kFlagPre | ((excl + tile_agg) & kValMask));
     }
-    if (lane == 0) st_status(&status[c], kFlagPre | ((excl + agg) & kValMask));
+    if (lane == 0) s_tile = excl;
+  }
+  __syncthreads();
+  unsigned off = s_tile;
+#pragma unroll
+  for (int w = 0; w < WAVES; w++) off += w < wv ? s_agg[w] : 0u;
+
+  if (!in_layout) return;
+  uint32_t* mrow = mask + (size_t)c * g.W;
+  if (!has_data) {  // chunk without data: the reference leaves these words untouched; define them
+    for (int w = lane; w < g.W; w += 64) mrow[w] = 0;
+    return;
   }
   if (lane == 0) {
-    begin[c] = (int)excl;
-    if (c == g.active - 1) *nnz = (int)(excl + agg);
+    begin[c] = (int)off;
+    if (c == g.active - 1) *nnz = (int)(off + agg);
   }
 
   // ---- phase 2: mask words and packed values from the registers
-  unsigned off = excl;
   uint32_t held = 0;
 #pragma unroll
   for (int t = 0; t < IT; t++) {
@@ -363,7 +397,15 @@ __global__ __launch_bounds__(256) void probe_nnz_kernel(const float* __restrict_
   for (size_t i = tid; i < head; i += nthreads) acc += (in[i] != 0.0f);
   const float4* p4 = reinterpret_cast<const float4*>(in + head);
   const size_t n4 = (n - head) >> 2;
-  for (size_t i = tid; i < n4; i += nthreads) {
+  size_t i = tid;
+  for (; i + 3 * nthreads < n4; i += 4 * nthreads) {  // four independent 16-byte loads in flight per lane
+    float4 v0 = p4[i], v1 = p4[i + nthreads], v2 = p4[i + 2 * nthreads], v3 = p4[i + 3 * nthreads];
+    acc += (v0.x != 0.0f) + (v0.y != 0.0f) + (v0.z != 0.0f) + (v0.w != 0.0f);
+    acc += (v1.x != 0.0f) + (v1.y != 0.0f) + (v1.z != 0.0f) + (v1.w != 0.0f);
+    acc += (v2.x != 0.0f) + (v2.y != 0.0f) + (v2.z != 0.0f) + (v2.w != 0.0f);
+    acc += (v3.x != 0.0f) + (v3.y != 0.0f) + (v3.z != 0.0f) + (v3.w != 0.0f);
+  }
+  for (; i < n4; i += nthreads) {
     float4 v = p4[i];
     acc += (v.x != 0.0f) + (v.y != 0.0f) + (v.z != 0.0f) + (v.w != 0.0f);
   }
@@ -488,17 +530,15 @@ extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, v
   uint32_t* ws = (uint32_t*)d_ws;
   const int words = process + 16;
   hipLaunchKernelGGL(zvc_ws_zero_kernel, dim3((words + 255) / 256), dim3(256), 0, (hipStream_t)stream, ws, words);
-  const unsigned grid = (g.process + kWavesPerGroup - 1) / kWavesPerGroup;
-  const dim3 blk(64 * kWavesPerGroup);
   const int iters = (g.E + 63) >> 6;
-#define CSWAP_FUSED(IT_)                                                                                  \
-  hipLaunchKernelGGL(zvc_fused_kernel<IT_>, dim3(grid), blk, 0, (hipStream_t)stream, d_in, g, ws, d_begin, \
-                     d_nnz, d_values, d_mask)
-  if (iters <= 8) CSWAP_FUSED(8);
-  else if (iters <= 16) CSWAP_FUSED(16);
-  else if (iters <= 32) CSWAP_FUSED(32);
-  else if (iters <= 64) CSWAP_FUSED(64);
-  else CSWAP_FUSED(128);
+#define CSWAP_FUSED(IT_, WAVES_)                                                                          \
+  hipLaunchKernelGGL((zvc_fused_kernel<IT_, WAVES_>), dim3((g.process + WAVES_ - 1) / WAVES_),            \
+                     dim3(64 * WAVES_), 0, (hipStream_t)stream, d_in, g, ws, d_begin, d_nnz, d_values, d_mask)
+  if (iters <= 8) CSWAP_FUSED(8, 16);
+  else if (iters <= 16) CSWAP_FUSED(16, 16);
+  else if (iters <= 32) CSWAP_FUSED(32, 16);
+  else if (iters <= 64) CSWAP_FUSED(64, 8);
+  else CSWAP_FUSED(128, 8);
 #undef CSWAP_FUSED
   return check_launch();
 }
@@ -508,7 +548,7 @@ extern "C" int cswap_probe_nnz(const float* d_in, size_t n, unsigned long long* 
   if (!d_in || !d_nnz || !n) return CSWAP_E_ARG;
   hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, d_nnz);
   size_t want = (n / 4 + 255) / 256;
-  unsigned grid = (unsigned)(want < 1 ? 1 : (want > 256 * 16 ? 256 * 16 : want));
+  unsigned grid = (unsigned)(want < 1 ? 1 : (want > 256 * 32 ? 256 * 32 : want));
   hipLaunchKernelGGL(probe_nnz_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, d_in, n, d_nnz);
   return check_launch();
 }

@@ -20,9 +20,26 @@ def as_field(t: np.ndarray) -> np.ndarray:
 
 
 def field_dims(shape):
-    """(nx, ny, nz) of the field an activation tensor of ``shape`` maps to."""
-    nx, ny = int(shape[-1]), int(shape[-2])
+    """(nx, ny, nz) of the field an activation tensor of ``shape`` maps to.
+
+    nx = last dim, ny = second to last, nz = product of the rest.  Tensors with
+    fewer than three useful dimensions would leave nz (or ny) at 1 and pay for
+    4x4x4 blocks that are mostly padding, so they are folded: a matrix [B, F]
+    with B a multiple of 4 becomes (F, 4, B/4); a flat vector becomes 32x32 or
+    4x4 rows when its length allows.  Any such view of contiguous memory is a
+    valid field as long as both directions use the same one."""
+    shape = [int(d) for d in shape]
+    if len(shape) <= 1:
+        n = shape[0] if shape else 1
+        if n % 1024 == 0:
+            return 32, 32, n // 1024
+        if n % 16 == 0:
+            return 4, 4, n // 16
+        return n, 1, 1
+    nx, ny = shape[-1], shape[-2]
     nz = int(np.prod(shape[:-2])) if len(shape) > 2 else 1
+    if nz < 4 and ny >= 16 and ny % 4 == 0:
+        nz, ny = nz * (ny // 4), 4
     return nx, ny, nz
 
 
