@@ -27,6 +27,10 @@ import sys
 import time
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the two ZFP kernels on this workload, from two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE), each scaled by what the counter reads for a plain copy of the same tensor
+# (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): profiles/zfp_rate8_attn402MB_hbm_traffic.txt
+HBM_TRAFFIC_BYTES_PER_LAUNCH = {"zfp_encode3_f32_kernel": 503603085, "zfp_decode3_f32_kernel": 503628556}
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
@@ -116,12 +120,7 @@ def main():
                 "compress_ms": round(enc_ms, 4), "decompress_ms": round(dec_ms, 4),
                 "compress_frac": round(bytes_per_value * n / (enc_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                 "decompress_frac": round(bytes_per_value * n / (dec_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
-    traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(traffic_file):
-        try:
-            roofline["traffic"] = json.load(open(traffic_file)).get(dom)
-        except Exception:
-            pass
+    roofline["traffic"] = HBM_TRAFFIC_BYTES_PER_LAUNCH.get(dom)
 
     result = {
         "metric": "compress+decompress GB/s (fp32 in), ZFP fixed-rate 8 bits/value, 1xMI355X",

@@ -271,6 +271,12 @@ struct BlockEncoder {
   // one bit plane: x bit i = this plane's bit of coefficient i (encode.cuh:331-344)
   CSWAP_HD void plane(uint64_t x)
   {
+    // Once every block of the wavefront has all 64 coefficients significant
+    // (typically after 4-6 planes) a plane is just its 64 bits verbatim.
+    if (!CSWAP_ANY(active() && n < 64)) {
+      if (active()) put(x, 64);
+      return;
+    }
     if (!active()) return;
     put(x & low_mask(n), n);  // first n coefficients verbatim
     if (n < 64) {
@@ -355,6 +361,15 @@ struct BlockDecoder {
   CSWAP_HD uint64_t plane()
   {
     uint64_t x = 0;
+    if (!CSWAP_ANY(active() && n < 64)) {  // every block of the wavefront is past discovery
+      if (active()) {
+        unsigned left = limit - pos;
+        x = window(pos);
+        if (left < 64) x &= low_mask(left);
+        pos += left < 64 ? left : 64;
+      }
+      return x;
+    }
     if (!active()) return x;
     unsigned left = limit - pos;
     unsigned m = n < left ? n : left;

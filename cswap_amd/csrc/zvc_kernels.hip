@@ -385,7 +385,7 @@ __global__ __launch_bounds__(64 * WAVES) void zvc_fused_kernel(
 // ------------------------------------------------------------------ probe
 __global__ void zero_u64_kernel(unsigned long long* p) { *p = 0ull; }
 
-__global__ __launch_bounds__(256) void probe_nnz_kernel(const float* __restrict__ in, size_t n,
+__global__ __launch_bounds__(1024) void probe_nnz_kernel(const float* __restrict__ in, size_t n,
                                                         unsigned long long* __restrict__ nnz)
 {
   const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -411,11 +411,14 @@ __global__ __launch_bounds__(256) void probe_nnz_kernel(const float* __restrict_
   }
   for (size_t i = head + (n4 << 2) + tid; i < n; i += nthreads) acc += (in[i] != 0.0f);
   acc = (unsigned)wave_sum((int)acc);
-  __shared__ unsigned part[4];
+  // one atomic per workgroup, and few workgroups: same-address atomics from
+  // different XCDs serialise at the memory side (~12 ns each)
+  __shared__ unsigned part[16];
   if ((threadIdx.x & 63u) == 0) part[threadIdx.x >> 6] = acc;
   __syncthreads();
   if (threadIdx.x == 0) {
-    unsigned long long s = (unsigned long long)part[0] + part[1] + part[2] + part[3];
+    unsigned long long s = 0;
+    for (unsigned w = 0; w < (blockDim.x >> 6); w++) s += part[w];
     if (s) atomicAdd(nnz, s);
   }
 }
@@ -547,8 +550,8 @@ extern "C" int cswap_probe_nnz(const float* d_in, size_t n, unsigned long long* 
 {
   if (!d_in || !d_nnz || !n) return CSWAP_E_ARG;
   hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, d_nnz);
-  size_t want = (n / 4 + 255) / 256;
-  unsigned grid = (unsigned)(want < 1 ? 1 : (want > 256 * 32 ? 256 * 32 : want));
-  hipLaunchKernelGGL(probe_nnz_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, d_in, n, d_nnz);
+  size_t want = (n / 16 + 1023) / 1024;  // 4 float4 per thread and pass
+  unsigned grid = (unsigned)(want < 1 ? 1 : (want > 512 ? 512 : want));
+  hipLaunchKernelGGL(probe_nnz_kernel, dim3(grid), dim3(1024), 0, (hipStream_t)stream, d_in, n, d_nnz);
   return check_launch();
 }
