@@ -29,7 +29,7 @@ import time
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the two ZFP kernels on this workload, from two rocprofv3 --pmc runs
 # (FETCH_SIZE, WRITE_SIZE), each scaled by what the counter reads for a plain copy of the same tensor
-# (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): profiles/zfp_rate8_attn402MB_hbm_traffic.txt
+# (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the summary of those runs is kept under profiles/
 HBM_TRAFFIC_BYTES_PER_LAUNCH = {"zfp_encode3_f32_kernel": 503603085, "zfp_decode3_f32_kernel": 503628556}
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
@@ -60,7 +60,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; run with --gpus 1 "
-              "(DESIGN.md says how it would shard)", file=sys.stderr)
+              "(blocks and chunks are independent, so it would shard by splitting the field along nz "
+              "or the tensor by chunk ranges, with no exchange)", file=sys.stderr)
         sys.exit(2)
 
     import torch

@@ -271,12 +271,6 @@ struct BlockEncoder {
   // one bit plane: x bit i = this plane's bit of coefficient i (encode.cuh:331-344)
   CSWAP_HD void plane(uint64_t x)
   {
-    // Once every block of the wavefront has all 64 coefficients significant
-    // (typically after 4-6 planes) a plane is just its 64 bits verbatim.
-    if (!CSWAP_ANY(active() && n < 64)) {
-      if (active()) put(x, 64);
-      return;
-    }
     if (!active()) return;
     put(x & low_mask(n), n);  // first n coefficients verbatim
     if (n < 64) {
