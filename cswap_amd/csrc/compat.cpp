@@ -27,6 +27,26 @@ bool is_device_ptr(const void* p)
   return a.type == hipMemoryTypeDevice || a.type == hipMemoryTypeManaged;
 }
 
+// number of dimensions = leading non-zero extents, as zfp_field_dimensionality
+// (zfp/zfp.c:60-64); 0 for an empty or 4-D field
+int field_dims_of(const cswap_zfp_field* f)
+{
+  if (!f->nx || f->nw) return 0;
+  if (!f->ny) return f->nz ? 0 : 1;
+  return f->nz ? 3 : 2;
+}
+
+size_t field_elems(const cswap_zfp_field* f)
+{
+  return f->nx * (f->ny ? f->ny : 1) * (f->nz ? f->nz : 1);
+}
+
+bool host_field_contiguous(const cswap_zfp_field* f)
+{
+  return !((f->sx && f->sx != 1) || (f->ny && f->sy && f->sy != (ptrdiff_t)f->nx) ||
+           (f->nz && f->sz && f->sz != (ptrdiff_t)(f->nx * f->ny)));
+}
+
 void flat_dims(long long numel, size_t& nx, size_t& ny, size_t& nz)
 {
   size_t n = (size_t)numel;
@@ -83,10 +103,11 @@ void setRatio(int ratio)
 size_t cuda_compress(cswap_zfp_stream* zs, const cswap_zfp_field* f)
 {
   if (!zs || !f || !zs->stream || !f->data || !zs->stream->begin) return 0;
-  if (f->type != 3 || !f->nx || !f->ny || !f->nz || f->nw) return 0;  // 3-D float only
+  const int dims = field_dims_of(f);
+  if (f->type != 3 || !dims) return 0;  // float fields of 1, 2 or 3 dimensions
   const unsigned maxbits = zs->maxbits;
-  const size_t cap = cswap_zfp_stream_capacity(f->nx, f->ny, f->nz, maxbits);
-  const size_t bytes = cswap_zfp_stream_bytes(f->nx, f->ny, f->nz, maxbits);
+  const size_t cap = cswap_zfp_stream_capacity_nd(dims, f->nx, f->ny, f->nz, maxbits);
+  const size_t bytes = cswap_zfp_stream_bytes_nd(dims, f->nx, f->ny, f->nz, maxbits);
   const bool field_dev = is_device_ptr(f->data), stream_dev = is_device_ptr(zs->stream->begin);
   const float* d_in = (const float*)f->data;
   uint64_t* d_stream = zs->stream->begin;
@@ -94,10 +115,8 @@ size_t cuda_compress(cswap_zfp_stream* zs, const cswap_zfp_field* f)
   size_t ok = 0;
   do {
     if (!field_dev) {  // host field: contiguous only, staged like zfp/cuZFP.cu:265-312
-      if ((f->sx && f->sx != 1) || (f->sy && f->sy != (ptrdiff_t)f->nx) ||
-          (f->sz && f->sz != (ptrdiff_t)(f->nx * f->ny)))
-        break;
-      size_t fb = 4 * f->nx * f->ny * f->nz;
+      if (!host_field_contiguous(f)) break;
+      size_t fb = 4 * field_elems(f);
       if (hipMalloc(&tmp_in, fb) != hipSuccess) break;
       if (hipMemcpy(tmp_in, f->data, fb, hipMemcpyHostToDevice) != hipSuccess) break;
       d_in = (const float*)tmp_in;
@@ -106,8 +125,8 @@ size_t cuda_compress(cswap_zfp_stream* zs, const cswap_zfp_field* f)
       if (hipMalloc(&tmp_s, cap) != hipSuccess) break;
       d_stream = (uint64_t*)tmp_s;
     }
-    if (cswap_zfp_compress_f32(d_in, f->nx, f->ny, f->nz, field_dev ? f->sx : 0, field_dev ? f->sy : 0,
-                               field_dev ? f->sz : 0, maxbits, d_stream, nullptr))
+    if (cswap_zfp_compress_f32_nd(d_in, dims, f->nx, f->ny, f->nz, field_dev ? f->sx : 0, field_dev ? f->sy : 0,
+                                  field_dev ? f->sz : 0, maxbits, d_stream, nullptr))
       break;
     if (!stream_dev) {
       if (hipMemcpy(zs->stream->begin, tmp_s, cap, hipMemcpyDeviceToHost) != hipSuccess) break;
@@ -128,21 +147,20 @@ size_t cuda_compress(cswap_zfp_stream* zs, const cswap_zfp_field* f)
 void cuda_decompress(cswap_zfp_stream* zs, cswap_zfp_field* f)
 {
   if (!zs || !f || !zs->stream || !f->data || !zs->stream->begin) return;
-  if (f->type != 3 || !f->nx || !f->ny || !f->nz || f->nw) return;
+  const int dims = field_dims_of(f);
+  if (f->type != 3 || !dims) return;
   const unsigned maxbits = zs->maxbits;
-  const size_t cap = cswap_zfp_stream_capacity(f->nx, f->ny, f->nz, maxbits);
-  const size_t bytes = cswap_zfp_stream_bytes(f->nx, f->ny, f->nz, maxbits);
+  const size_t cap = cswap_zfp_stream_capacity_nd(dims, f->nx, f->ny, f->nz, maxbits);
+  const size_t bytes = cswap_zfp_stream_bytes_nd(dims, f->nx, f->ny, f->nz, maxbits);
   const bool field_dev = is_device_ptr(f->data), stream_dev = is_device_ptr(zs->stream->begin);
   float* d_out = (float*)f->data;
   const uint64_t* d_stream = zs->stream->begin;
   void *tmp_out = nullptr, *tmp_s = nullptr;
-  const size_t fb = 4 * f->nx * f->ny * f->nz;
+  const size_t fb = 4 * field_elems(f);
   bool ok = false;
   do {
     if (!field_dev) {
-      if ((f->sx && f->sx != 1) || (f->sy && f->sy != (ptrdiff_t)f->nx) ||
-          (f->sz && f->sz != (ptrdiff_t)(f->nx * f->ny)))
-        break;
+      if (!host_field_contiguous(f)) break;
       if (hipMalloc(&tmp_out, fb) != hipSuccess) break;
       d_out = (float*)tmp_out;
     }
@@ -151,8 +169,8 @@ void cuda_decompress(cswap_zfp_stream* zs, cswap_zfp_field* f)
       if (hipMemcpy(tmp_s, zs->stream->begin, cap, hipMemcpyHostToDevice) != hipSuccess) break;
       d_stream = (const uint64_t*)tmp_s;
     }
-    if (cswap_zfp_decompress_f32(d_stream, f->nx, f->ny, f->nz, field_dev ? f->sx : 0, field_dev ? f->sy : 0,
-                                 field_dev ? f->sz : 0, maxbits, d_out, nullptr))
+    if (cswap_zfp_decompress_f32_nd(d_stream, dims, f->nx, f->ny, f->nz, field_dev ? f->sx : 0,
+                                    field_dev ? f->sy : 0, field_dev ? f->sz : 0, maxbits, d_out, nullptr))
       break;
     if (!field_dev) {
       if (hipMemcpy(f->data, tmp_out, fb, hipMemcpyDeviceToHost) != hipSuccess) break;

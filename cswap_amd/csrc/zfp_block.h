@@ -236,7 +236,7 @@ CSWAP_HD uint32_t funnel_shr(uint32_t hi, uint32_t lo, unsigned s)  // ({hi,lo} 
 // end of the block (needed when the next block's bits follow immediately);
 // GUARD = false lets the last plane spill up to 96 bits past the end, which the
 // caller must provide as slack and ignore.
-template <class Mem, bool GUARD>
+template <class Mem, bool GUARD, int SIZE = 64>
 struct BlockEncoder {
   Mem& mem;
   unsigned pos, limit;
@@ -273,12 +273,12 @@ struct BlockEncoder {
   {
     if (!active()) return;
     put(x & low_mask(n), n);  // first n coefficients verbatim
-    if (n < 64) {
+    if (n < SIZE) {
       uint64_t rest = x >> n;
-      while (rest != 0 && n < 64 && pos < limit) {
+      while (rest != 0 && n < SIZE && pos < limit) {
         unsigned t = (unsigned)ctz64(rest);  // zeros before the next one-bit
         unsigned nt = n + t;
-        bool more = nt < 63;                 // a one-bit at position 63 is implied, not written
+        bool more = nt < SIZE - 1;           // a one-bit at the last position is implied, not written
         unsigned q = pos + t + 1;
         set_bit(pos, true);                  // positive group test
         set_bit(q, more);                    // t zeros, then the one-bit
@@ -286,7 +286,7 @@ struct BlockEncoder {
         n = nt + 1;
         rest = (rest >> t) >> 1;
       }
-      if (rest == 0 && n < 64 && pos < limit) pos++;  // negative group test: a zero bit
+      if (rest == 0 && n < SIZE && pos < limit) pos++;  // negative group test: a zero bit
     }
   }
 };
@@ -334,7 +334,7 @@ CSWAP_HD void encode_block(const float (&f)[64], unsigned pos0, unsigned maxbits
 // mem.ld32(dword_index) reads the bit region; positions are absolute within it
 // and the block owns [pos0, pos0 + maxbits).  Reads may run up to 96 bits past
 // the end of the block (the values are never used).
-template <class Mem>
+template <class Mem, int SIZE = 64>
 struct BlockDecoder {
   Mem& mem;
   unsigned pos, limit;
@@ -355,12 +355,12 @@ struct BlockDecoder {
   CSWAP_HD uint64_t plane()
   {
     uint64_t x = 0;
-    if (!CSWAP_ANY(active() && n < 64)) {  // every block of the wavefront is past discovery
+    if (!CSWAP_ANY(active() && n < SIZE)) {  // every block of the wavefront is past discovery
       if (active()) {
         unsigned left = limit - pos;
-        x = window(pos);
-        if (left < 64) x &= low_mask(left);
-        pos += left < 64 ? left : 64;
+        unsigned m = left < (unsigned)SIZE ? left : (unsigned)SIZE;
+        x = window(pos) & low_mask(m);
+        pos += m;
       }
       return x;
     }
@@ -369,13 +369,13 @@ struct BlockDecoder {
     unsigned m = n < left ? n : left;
     x = window(pos) & low_mask(m);
     pos += m;
-    while (n < 64 && pos < limit) {
+    while (n < SIZE && pos < limit) {
       uint64_t w = window(pos);
       pos++;
       if (!(w & 1)) break;  // negative group test: plane done
       w >>= 1;              // 63 valid bits
       unsigned avail = limit - pos;
-      unsigned maxrun = 63 - n < avail ? 63 - n : avail;
+      unsigned maxrun = SIZE - 1 - n < avail ? SIZE - 1 - n : avail;
       unsigned t = (unsigned)ctz64(w);
       bool found = t < maxrun;  // t zeros then a one; else ran into position 63 or the budget
       unsigned r = found ? t : maxrun;
@@ -438,6 +438,93 @@ CSWAP_HD void decode_block(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)
   float w = pow2f(emax - 30);
 #pragma unroll
   for (int i = 0; i < 64; i++) f[i] = w * (float)ib[i];
+}
+
+// ---------------------------------------------------------------- 2-D and 1-D blocks
+// Blocks of 4x4 = 16 and 4 values (CSWAP+/zfp/encode2.cuh, encode1.cuh,
+// decode2.cuh, decode1.cuh): same cast and coder with 16 / 4 coefficients, lifting
+// along x then y (encode.cuh:177-201; inverse y then x, decode.cuh:203-226),
+// coefficient order perm_2 / identity (constants.h:95-133).  The bit planes are
+// formed with the same 32x32 transpose on zero-padded rows.
+#define CSWAP_P2(i, j) ((i) + 4 * (j))
+struct Perm2 {
+  int v[16];
+};
+constexpr Perm2 kPerm2 = {{CSWAP_P2(0,0), CSWAP_P2(1,0), CSWAP_P2(0,1), CSWAP_P2(1,1), CSWAP_P2(2,0), CSWAP_P2(0,2),
+                           CSWAP_P2(2,1), CSWAP_P2(1,2), CSWAP_P2(3,0), CSWAP_P2(0,3), CSWAP_P2(2,2), CSWAP_P2(3,1),
+                           CSWAP_P2(1,3), CSWAP_P2(3,2), CSWAP_P2(2,3), CSWAP_P2(3,3)}};
+
+template <int DIMS, bool GUARD, class Mem>
+CSWAP_HD void encode_block_low(const float (&f)[16], unsigned pos0, unsigned maxbits, Mem& mem)
+{
+  constexpr int SIZE = DIMS == 2 ? 16 : 4;
+  float m = 0.0f;
+#pragma unroll
+  for (int i = 0; i < SIZE; i++) m = fmaxf(m, fabsf(f[i]));
+  uint32_t mb = f32_bits(m);
+  uint32_t e = mb ? (mb >> 23) + 1 : 0;
+  if (e == 0) return;
+  BlockEncoder<Mem, GUARD, SIZE> enc(mem, pos0, maxbits);
+  enc.put(2 * e + 1, 9);
+  float s = pow2f(30 - ((int)e - 127));
+  int32_t ib[16];
+#pragma unroll
+  for (int i = 0; i < SIZE; i++) ib[i] = (int32_t)(s * f[i]);
+  uint32_t a[32];
+#pragma unroll
+  for (int i = 0; i < 32; i++) a[i] = 0;
+  if (DIMS == 2) {
+#pragma unroll
+    for (int y = 0; y < 4; y++) fwd_lift4(ib[4 * y], ib[4 * y + 1], ib[4 * y + 2], ib[4 * y + 3]);
+#pragma unroll
+    for (int x = 0; x < 4; x++) fwd_lift4(ib[x], ib[x + 4], ib[x + 8], ib[x + 12]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) a[i] = int2nb(ib[kPerm2.v[i]]);
+  } else {
+    fwd_lift4(ib[0], ib[1], ib[2], ib[3]);
+#pragma unroll
+    for (int i = 0; i < 4; i++) a[i] = int2nb(ib[i]);
+  }
+  transpose32(a);
+#pragma unroll
+  for (int k = 31; k >= 0; k--) enc.plane((uint64_t)a[k]);
+}
+
+template <int DIMS, class Mem>
+CSWAP_HD void decode_block_low(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)[16])
+{
+  constexpr int SIZE = DIMS == 2 ? 16 : 4;
+  BlockDecoder<Mem, SIZE> dec(mem, pos0, maxbits);
+  uint32_t h = (uint32_t)dec.window(pos0);
+  if (!(h & 1)) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) f[i] = 0.0f;
+    return;
+  }
+  int emax = (int)((h >> 1) & 0xff) - 127;
+  dec.pos = pos0 + 9;
+  uint32_t a[32];
+#pragma unroll
+  for (int k = 31; k >= 0; k--) a[k] = (uint32_t)dec.plane();
+  transpose32(a);
+  int32_t ib[16];
+  if (DIMS == 2) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) ib[kPerm2.v[i]] = nb2int(a[i]);
+#pragma unroll
+    for (int x = 0; x < 4; x++) inv_lift4(ib[x], ib[x + 4], ib[x + 8], ib[x + 12]);
+#pragma unroll
+    for (int y = 0; y < 4; y++) inv_lift4(ib[4 * y], ib[4 * y + 1], ib[4 * y + 2], ib[4 * y + 3]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; i++) ib[i] = nb2int(a[i]);
+    inv_lift4(ib[0], ib[1], ib[2], ib[3]);
+  }
+  float w = pow2f(emax - 30);
+#pragma unroll
+  for (int i = 0; i < SIZE; i++) f[i] = w * (float)ib[i];
+#pragma unroll
+  for (int i = SIZE; i < 16; i++) f[i] = 0.0f;
 }
 
 // ---------------------------------------------------------------- partial blocks

@@ -215,6 +215,119 @@ __global__ __launch_bounds__(64) void zfp_decode3_f32_kernel(const uint64_t* __r
   }
 }
 
+// ------------------------------------------------------------- 2-D / 1-D fields
+// Same decomposition (one lane per block of 16 or 4 values, 64 blocks per
+// wave, LDS bit region); element accesses are predicated scalars.
+struct FieldLow {
+  uint32_t nx, ny;   // ny = 1 for a 1-D field
+  uint32_t mx;       // blocks along x
+  uint32_t nblocks;
+  long long sx, sy;
+};
+
+template <int DIMS>
+__device__ __forceinline__ void load_block_low(const float* __restrict__ in, const FieldLow& fd, uint32_t b,
+                                               float (&f)[16])
+{
+  const uint32_t q = b / fd.mx;
+  const uint32_t x0 = (b - q * fd.mx) * 4, y0 = DIMS == 2 ? q * 4 : 0;
+  const float* p = in + (long long)x0 * fd.sx + (long long)y0 * fd.sy;
+  const uint32_t bx = min(4u, fd.nx - x0), by = DIMS == 2 ? min(4u, fd.ny - y0) : 1u;
+#pragma unroll
+  for (int y = 0; y < 4; y++)
+#pragma unroll
+    for (int x = 0; x < 4; x++) {
+      bool ok = (uint32_t)x < bx && (uint32_t)y < by;
+      f[4 * y + x] = ok ? p[x * fd.sx + y * fd.sy] : 0.0f;
+    }
+#pragma unroll
+  for (int y = 0; y < (DIMS == 2 ? 4 : 1); y++) pad4(f[4 * y], f[4 * y + 1], f[4 * y + 2], f[4 * y + 3], bx);
+  if (DIMS == 2) {
+#pragma unroll
+    for (int x = 0; x < 4; x++) pad4(f[x], f[x + 4], f[x + 8], f[x + 12], by);
+  }
+}
+
+template <int DIMS>
+__device__ __forceinline__ void store_block_low(float* __restrict__ out, const FieldLow& fd, uint32_t b,
+                                                const float (&f)[16])
+{
+  const uint32_t q = b / fd.mx;
+  const uint32_t x0 = (b - q * fd.mx) * 4, y0 = DIMS == 2 ? q * 4 : 0;
+  float* p = out + (long long)x0 * fd.sx + (long long)y0 * fd.sy;
+  const uint32_t bx = min(4u, fd.nx - x0), by = DIMS == 2 ? min(4u, fd.ny - y0) : 1u;
+#pragma unroll
+  for (int y = 0; y < 4; y++)
+#pragma unroll
+    for (int x = 0; x < 4; x++)
+      if ((uint32_t)x < bx && (uint32_t)y < by) p[x * fd.sx + y * fd.sy] = f[4 * y + x];
+}
+
+// The wave's 64 blocks are packed back to back in LDS exactly as in the stream
+// (64 * maxbits bits = maxbits whole words) and moved cooperatively.
+template <int DIMS>
+__global__ __launch_bounds__(64) void zfp_encode_low_f32_kernel(const float* __restrict__ in, FieldLow fd,
+                                                                unsigned maxbits, uint64_t* __restrict__ stream)
+{
+  extern __shared__ uint4 lds_raw[];
+  uint32_t* lds = reinterpret_cast<uint32_t*>(lds_raw);
+  const unsigned lane = threadIdx.x;
+  const uint32_t first = blockIdx.x * 64u;
+  const uint32_t valid = min(64u, fd.nblocks - first);
+  const unsigned n16 = (2u * maxbits + 4u + 3u) / 4u;
+  for (unsigned i = lane; i < n16; i += 64) lds_raw[i] = make_uint4(0, 0, 0, 0);
+  __syncthreads();
+  if (lane < valid) {
+    float f[16];
+    load_block_low<DIMS>(in, fd, first + lane, f);
+    LdsBits mem{lds};
+    encode_block_low<DIMS, true>(f, lane * maxbits, maxbits, mem);
+  }
+  __syncthreads();
+  const unsigned nwords = (valid * maxbits + 63u) >> 6;
+  const uint64_t* src = reinterpret_cast<const uint64_t*>(lds);
+  uint64_t* dst = stream + (size_t)blockIdx.x * maxbits;
+  for (unsigned i = lane; i < nwords; i += 64) dst[i] = src[i];
+}
+
+template <int DIMS>
+__global__ __launch_bounds__(64) void zfp_decode_low_f32_kernel(const uint64_t* __restrict__ stream, FieldLow fd,
+                                                                unsigned maxbits, float* __restrict__ out)
+{
+  extern __shared__ uint4 lds_raw[];
+  uint32_t* lds = reinterpret_cast<uint32_t*>(lds_raw);
+  const unsigned lane = threadIdx.x;
+  const uint32_t first = blockIdx.x * 64u;
+  const uint32_t valid = min(64u, fd.nblocks - first);
+  const unsigned nwords = (valid * maxbits + 63u) >> 6;
+  const uint64_t* src = stream + (size_t)blockIdx.x * maxbits;
+  uint64_t* dst = reinterpret_cast<uint64_t*>(lds);
+  for (unsigned i = lane; i < nwords + 2; i += 64) dst[i] = i < nwords ? src[i] : 0;
+  __syncthreads();
+  if (lane < valid) {
+    float f[16];
+    LdsBits mem{lds};
+    decode_block_low<DIMS>(mem, lane * maxbits, maxbits, f);
+    store_block_low<DIMS>(out, fd, first + lane, f);
+  }
+}
+
+static int make_field_low(FieldLow& fd, int dims, const void* base, const void* stream, size_t nx, size_t ny,
+                          ptrdiff_t sx, ptrdiff_t sy, unsigned maxbits)
+{
+  if (dims == 1) ny = 1;
+  if (!nx || !ny || maxbits < 16 || maxbits > 4096) return CSWAP_E_ARG;
+  if (nx > 0x7fffffffu || ny > 0x7fffffffu) return CSWAP_E_ARG;
+  if (((uintptr_t)stream % 8) != 0 || ((uintptr_t)base % 4) != 0) return CSWAP_E_ARG;
+  size_t mx = (nx + 3) / 4, my = dims == 2 ? (ny + 3) / 4 : 1;
+  size_t nb = mx * my;
+  if (nb > 0xfffffff0ull) return CSWAP_E_ARG;
+  fd.nx = (uint32_t)nx; fd.ny = (uint32_t)ny; fd.mx = (uint32_t)mx; fd.nblocks = (uint32_t)nb;
+  fd.sx = sx ? sx : 1;
+  fd.sy = sy ? sy : (ptrdiff_t)nx;
+  return CSWAP_OK;
+}
+
 // ------------------------------------------------------------- host side
 static int make_field(Field3& fd, const void* base, const void* stream, size_t nx, size_t ny, size_t nz,
                       ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits)
@@ -287,6 +400,68 @@ extern "C" int cswap_zfp_decompress_f32(const uint64_t* d_stream, size_t nx, siz
                        d_stream, fd, maxbits, d_out);
   else
     hipLaunchKernelGGL(zfp_decode3_f32_kernel<false>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
+                       d_stream, fd, maxbits, d_out);
+  return check_launch();
+}
+
+// ------------------------------------------------------------- any dimensionality
+static size_t blocks_nd(int dims, size_t nx, size_t ny, size_t nz)
+{
+  size_t nb = (nx + 3) / 4;
+  if (dims >= 2) nb *= (ny + 3) / 4;
+  if (dims >= 3) nb *= (nz + 3) / 4;
+  return nb;
+}
+
+extern "C" size_t cswap_zfp_stream_capacity_nd(int dims, size_t nx, size_t ny, size_t nz, unsigned maxbits)
+{
+  if (dims < 1 || dims > 3) return 0;
+  return ((blocks_nd(dims, nx, ny, nz) * maxbits + 63) / 64) * 8;
+}
+
+extern "C" size_t cswap_zfp_stream_bytes_nd(int dims, size_t nx, size_t ny, size_t nz, unsigned maxbits)
+{
+  if (dims < 1 || dims > 3) return 0;
+  if (dims == 3) return cswap_zfp_stream_bytes(nx, ny, nz, maxbits);
+  return cswap_zfp_stream_capacity_nd(dims, nx, ny, nz, maxbits);  // 1-D and 2-D round up (zfp/shared.h:42-71)
+}
+
+extern "C" int cswap_zfp_compress_f32_nd(const float* d_in, int dims, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
+                                         ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream,
+                                         cswap_stream_t stream)
+{
+  if (dims == 3) return cswap_zfp_compress_f32(d_in, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
+  if (!d_in || !d_stream || (dims != 1 && dims != 2)) return CSWAP_E_ARG;
+  FieldLow fd;
+  int rc = make_field_low(fd, dims, d_in, d_stream, nx, ny, sx, sy, maxbits);
+  if (rc) return rc;
+  unsigned grid = (fd.nblocks + 63) / 64;
+  size_t lds_bytes = (size_t)((2u * maxbits + 4u + 3u) / 4u) * 16;
+  if (dims == 2)
+    hipLaunchKernelGGL(zfp_encode_low_f32_kernel<2>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream, d_in,
+                       fd, maxbits, d_stream);
+  else
+    hipLaunchKernelGGL(zfp_encode_low_f32_kernel<1>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream, d_in,
+                       fd, maxbits, d_stream);
+  return check_launch();
+}
+
+extern "C" int cswap_zfp_decompress_f32_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
+                                           ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, float* d_out,
+                                           cswap_stream_t stream)
+{
+  if (dims == 3) return cswap_zfp_decompress_f32(d_stream, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
+  if (!d_out || !d_stream || (dims != 1 && dims != 2)) return CSWAP_E_ARG;
+  FieldLow fd;
+  int rc = make_field_low(fd, dims, d_out, d_stream, nx, ny, sx, sy, maxbits);
+  if (rc) return rc;
+  unsigned grid = (fd.nblocks + 63) / 64;
+  size_t lds_bytes = (size_t)((2u * maxbits + 4u + 3u) / 4u) * 16;
+  if (dims == 2)
+    hipLaunchKernelGGL(zfp_decode_low_f32_kernel<2>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
+                       d_stream, fd, maxbits, d_out);
+  else
+    hipLaunchKernelGGL(zfp_decode_low_f32_kernel<1>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
                        d_stream, fd, maxbits, d_out);
   return check_launch();
 }

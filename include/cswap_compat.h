@@ -57,7 +57,8 @@ void GPUcompression(int arraySize, int kernelSize, float* arrayGPU, float* compr
 void GPUdecompression(float* arrayGPU, float* destiGPU, int arraySize, int kernelSize, uint32_t* gpuDataindex,
                       int* beginIndex, int dimsize, int blocksize);
 
-/* CSWAP+/zfp/cuZFP.h:11-12.  3-D float fields; returns the stream size in bytes
+/* CSWAP+/zfp/cuZFP.h:11-12.  Float fields of 1, 2 or 3 dimensions (trailing zero
+ * extents, zfp/zfp.c:60-64); returns the stream size in bytes
  * (0 = failure) and, like the reference, has finished when it returns. */
 size_t cuda_compress(cswap_zfp_stream* stream, const cswap_zfp_field* field);
 void   cuda_decompress(cswap_zfp_stream* stream, cswap_zfp_field* field);

@@ -63,6 +63,21 @@ int cswap_zfp_decompress_f32(const uint64_t* d_stream, size_t nx, size_t ny, siz
                              ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
                              float* d_out, cswap_stream_t stream);
 
+/* 1-D (4-value blocks) and 2-D (4x4 blocks) fields, as dispatched by
+ * internal::encode / internal::decode on the number of non-zero dimensions
+ * (zfp/cuZFP.cu:105-203; zfp/encode1.cuh, encode2.cuh, decode1.cuh, decode2.cuh).
+ * dims = 1, 2 or 3; unused extents and strides are ignored; dims = 3 is the call
+ * above.  maxbits is bits per block of 4^dims values.  For 1-D and 2-D the
+ * reference reports the stream size rounded up to whole words (zfp/shared.h:42-71). */
+size_t cswap_zfp_stream_capacity_nd(int dims, size_t nx, size_t ny, size_t nz, unsigned maxbits);
+size_t cswap_zfp_stream_bytes_nd(int dims, size_t nx, size_t ny, size_t nz, unsigned maxbits);
+int cswap_zfp_compress_f32_nd(const float* d_in, int dims, size_t nx, size_t ny, size_t nz,
+                              ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
+                              uint64_t* d_stream, cswap_stream_t stream);
+int cswap_zfp_decompress_f32_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
+                                ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
+                                float* d_out, cswap_stream_t stream);
+
 /* ------------------------------------------------------------------ ZVC -----
  * Zero-value compaction in the reference's format (zfp/compression.cu).  The
  * tensor of n fp32 elements is cut into `process` chunks of

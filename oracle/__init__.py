@@ -41,6 +41,19 @@ def _sig(lib: C.CDLL) -> C.CDLL:
     lib.orc_zfp_encode3_f32.argtypes = [vp, sz, sz, sz, pd, pd, pd, u, vp]
     lib.orc_zfp_decode3_f32.restype = None
     lib.orc_zfp_decode3_f32.argtypes = [vp, sz, sz, sz, pd, pd, pd, u, vp]
+    lib.orc_zfp_stream_bytes2.restype = sz
+    lib.orc_zfp_stream_bytes2.argtypes = [sz, sz, u]
+    lib.orc_zfp_stream_bytes1.restype = sz
+    lib.orc_zfp_stream_bytes1.argtypes = [sz, u]
+    lib.orc_zfp_encode2_f32.restype = sz
+    lib.orc_zfp_encode2_f32.argtypes = [vp, sz, sz, pd, pd, u, vp]
+    lib.orc_zfp_decode2_f32.restype = None
+    lib.orc_zfp_decode2_f32.argtypes = [vp, sz, sz, pd, pd, u, vp]
+    lib.orc_zfp_encode1_f32.restype = sz
+    lib.orc_zfp_encode1_f32.argtypes = [vp, sz, pd, u, vp]
+    lib.orc_zfp_decode1_f32.restype = None
+    lib.orc_zfp_decode1_f32.argtypes = [vp, sz, pd, u, vp]
+    lib.orc_perm2.argtypes = [vp]
     lib.orc_zfp_encode_block_f32.restype = None
     lib.orc_zfp_encode_block_f32.argtypes = [vp, u, sz, vp]
     lib.orc_zfp_decode_block_f32.restype = None
@@ -112,6 +125,37 @@ def zfp_decode3(stream: np.ndarray, shape, maxbits: int, omp: bool = False) -> n
     s[: w.size] = w
     out = np.zeros(shape, dtype=np.float32)
     lib(omp).orc_zfp_decode3_f32(_p(s), nx, ny, nz, 0, 0, 0, maxbits, _p(out))
+    return out
+
+
+def zfp_encode_nd(field: np.ndarray, maxbits: int) -> np.ndarray:
+    """1-D (nx,), 2-D (ny,nx) or 3-D (nz,ny,nx) C-contiguous fp32 field -> stream words."""
+    assert field.dtype == np.float32 and field.flags.c_contiguous
+    if field.ndim == 3:
+        return zfp_encode3(field, maxbits)
+    shp = field.shape
+    blocks = int(np.prod([(n + 3) // 4 for n in shp]))
+    out = np.zeros((blocks * maxbits + 63) // 64 + 1, dtype=np.uint64)
+    if field.ndim == 2:
+        lib().orc_zfp_encode2_f32(_p(field), shp[1], shp[0], 0, 0, maxbits, _p(out))
+    else:
+        lib().orc_zfp_encode1_f32(_p(field), shp[0], 0, maxbits, _p(out))
+    return out[:-1]
+
+
+def zfp_decode_nd(stream: np.ndarray, shape, maxbits: int) -> np.ndarray:
+    shape = tuple(shape)
+    if len(shape) == 3:
+        return zfp_decode3(stream, shape, maxbits)
+    blocks = int(np.prod([(n + 3) // 4 for n in shape]))
+    s = np.zeros((blocks * maxbits + 63) // 64 + 1, dtype=np.uint64)
+    w = np.ascontiguousarray(stream).view(np.uint64)
+    s[: w.size] = w
+    out = np.zeros(shape, dtype=np.float32)
+    if len(shape) == 2:
+        lib().orc_zfp_decode2_f32(_p(s), shape[1], shape[0], 0, 0, maxbits, _p(out))
+    else:
+        lib().orc_zfp_decode1_f32(_p(s), shape[0], 0, maxbits, _p(out))
     return out
 
 

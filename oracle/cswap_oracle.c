@@ -25,6 +25,8 @@
  *       near-inverse bound, wrap-around brute force.
  *   orc_int2uint / orc_uint2int : bijection + negabinary closed form.
  *   orc_perm3 : permutation sorted by (i+j+k, i^2+j^2+k^2).
+ *   orc_zfp_encode2/decode2/encode1/decode1 : byte-exact against zfp 0.5.5 2-D and
+ *       1-D golden vectors (tests/golden/zfp_golden_12d.npz).
  *   orc_zvc_* : numpy boolean indexing / packbits / cumsum.
  *
  * Undefined in the reference and therefore unpinned here: blocks whose largest
@@ -191,10 +193,12 @@ void orc_inv_xform3(int32_t *b)
 
 /* block exponent (encode.cuh:40-71): frexp exponent of the largest magnitude,
  * -127 for an all-zero block, clamped to >= -126 for subnormals. */
-int orc_block_emax(const float *f)
+static int block_emax_n(const float *f, int count);
+int orc_block_emax(const float *f) { return block_emax_n(f, 64); }
+static int block_emax_n(const float *f, int count)
 {
     float m = 0.0f;
-    for (int i = 0; i < 64; i++) m = fmaxf(m, fabsf(f[i]));
+    for (int i = 0; i < count; i++) m = fmaxf(m, fabsf(f[i]));
     int e = -127;
     if (m > 0.0f) {
         frexpf(m, &e);
@@ -213,26 +217,26 @@ void orc_fwd_cast(int32_t *ib, const float *fb, int emax)
 
 /* embedded bit-plane coder (encode.cuh:306-345).  budget = bits available for
  * the 64 coefficients; returns the number of bits written. */
-static unsigned encode_ints(bitcur *c, unsigned budget, const uint32_t *u)
+static unsigned encode_ints(bitcur *c, unsigned budget, const uint32_t *u, unsigned size)
 {
     unsigned bits = budget;
     unsigned n = 0;
     for (int k = 31; k >= 0 && bits; k--) {
         /* gather bit plane k: bit i of x is bit k of u[i] */
         word_t x = 0;
-        for (int i = 0; i < 64; i++) x |= (word_t)((u[i] >> k) & 1u) << i;
+        for (unsigned i = 0; i < size; i++) x |= (word_t)((u[i] >> k) & 1u) << i;
         /* first n coefficients are already significant: verbatim */
         unsigned m = n < bits ? n : bits;
         bits -= m;
         put_bits(c, x, m);
         x = (m < 64) ? (x >> m) : 0;
         /* group tests + unary run lengths for the rest */
-        while (n < 64 && bits) {
+        while (n < size && bits) {
             bits--;
             unsigned any = (x != 0);
             put_bits(c, any, 1);
             if (!any) break;
-            while (n < 63 && bits) {
+            while (n < size - 1 && bits) {
                 bits--;
                 unsigned b = (unsigned)(x & 1u);
                 put_bits(c, b, 1);
@@ -246,19 +250,19 @@ static unsigned encode_ints(bitcur *c, unsigned budget, const uint32_t *u)
 }
 
 /* mirror of the coder (decode.cuh:127-179) */
-static void decode_ints(bitcur *c, unsigned budget, uint32_t *u)
+static void decode_ints(bitcur *c, unsigned budget, uint32_t *u, unsigned size)
 {
     unsigned bits = budget;
     unsigned n = 0;
-    memset(u, 0, 64 * sizeof(uint32_t));
+    memset(u, 0, size * sizeof(uint32_t));
     for (int k = 31; k >= 0 && bits; k--) {
         unsigned m = n < bits ? n : bits;
         bits -= m;
         word_t x = get_bits(c, m);
-        while (bits && n < 64) {
+        while (bits && n < size) {
             bits--;
             if (!get_bit(c)) break;
-            while (bits && n < 63) {
+            while (bits && n < size - 1) {
                 bits--;
                 if (get_bit(c)) break;
                 n++;
@@ -266,7 +270,7 @@ static void decode_ints(bitcur *c, unsigned budget, uint32_t *u)
             x += (word_t)1 << n;
             n++;
         }
-        for (int i = 0; i < 64; i++, x >>= 1) u[i] += (uint32_t)(x & 1u) << k;
+        for (unsigned i = 0; i < size; i++, x >>= 1) u[i] += (uint32_t)(x & 1u) << k;
     }
 }
 
@@ -284,7 +288,7 @@ void orc_zfp_encode_block_f32(const float *fb, unsigned maxbits, size_t block_id
     orc_fwd_cast(ib, fb, emax);
     orc_fwd_xform3(ib);
     for (int i = 0; i < 64; i++) ub[i] = orc_int2uint(ib[PERM3[i]]);
-    encode_ints(&c, maxbits - 9, ub);
+    encode_ints(&c, maxbits - 9, ub, 64);
 }
 
 /* decode.cuh:228-288; fb is left untouched (caller pre-zeroes) for an empty block */
@@ -295,7 +299,7 @@ void orc_zfp_decode_block_f32(const word_t *stream, unsigned maxbits, size_t blo
     int emax = (int)get_bits(&c, 8) - 127;
     uint32_t ub[64];
     int32_t ib[64];
-    decode_ints(&c, maxbits - 9, ub);
+    decode_ints(&c, maxbits - 9, ub, 64);
     for (int i = 0; i < 64; i++) ib[PERM3[i]] = orc_uint2int(ub[i]);
     orc_inv_xform3(ib);
     float w = ldexpf(1.0f, emax - 30);
@@ -406,6 +410,146 @@ void orc_zfp_decode3_f32(const word_t *stream, size_t nx, size_t ny, size_t nz,
             for (unsigned y = 0; y < by; y++)
                 for (unsigned x = 0; x < bx; x++)
                     p[x * sx + y * sy + z * sz] = fb[16 * z + 4 * y + x];
+    }
+}
+
+/* ------------------------------------------------------------------------ */
+/* 2-D and 1-D fields (encode2.cuh, encode1.cuh, decode2.cuh, decode1.cuh):    */
+/* blocks of 4x4 = 16 and 4 values, coefficient order perm_2 / identity       */
+/* (constants.h:95-133), transform along x then y (encode.cuh:177-201).        */
+/* ------------------------------------------------------------------------ */
+
+#define P2(i, j) ((unsigned char)((i) + 4 * (j)))
+static const unsigned char PERM2[16] = {
+    P2(0,0), P2(1,0), P2(0,1), P2(1,1), P2(2,0), P2(0,2), P2(2,1), P2(1,2),
+    P2(3,0), P2(0,3), P2(2,2), P2(3,1), P2(1,3), P2(3,2), P2(2,3), P2(3,3),
+};
+#undef P2
+void orc_perm2(unsigned char out[16]) { memcpy(out, PERM2, 16); }
+
+/* dims = 1 or 2; fb holds 4 or 16 gathered (and padded) values */
+static void encode_block_low(const float *fb, int dims, unsigned maxbits, size_t block_idx, word_t *stream)
+{
+    const int size = dims == 2 ? 16 : 4;
+    bitcur c = { stream, block_idx * (size_t)maxbits };
+    int emax = block_emax_n(fb, size);
+    unsigned e = (unsigned)(emax + 127);
+    if (!e) return;
+    put_bits(&c, 2 * e + 1, 9);
+    int32_t ib[16];
+    uint32_t ub[16];
+    float s = (float)ldexp(1.0, 30 - emax);
+    for (int i = 0; i < size; i++) ib[i] = (int32_t)(s * fb[i]);
+    if (dims == 2) {
+        for (int y = 0; y < 4; y++) orc_fwd_lift(ib + 4 * y, 1);
+        for (int x = 0; x < 4; x++) orc_fwd_lift(ib + x, 4);
+        for (int i = 0; i < 16; i++) ub[i] = orc_int2uint(ib[PERM2[i]]);
+    } else {
+        orc_fwd_lift(ib, 1);
+        for (int i = 0; i < 4; i++) ub[i] = orc_int2uint(ib[i]);
+    }
+    encode_ints(&c, maxbits - 9, ub, (unsigned)size);
+}
+
+static void decode_block_low(const word_t *stream, int dims, unsigned maxbits, size_t block_idx, float *fb)
+{
+    const int size = dims == 2 ? 16 : 4;
+    bitcur c = { (word_t *)stream, block_idx * (size_t)maxbits };
+    if (!get_bit(&c)) return;
+    int emax = (int)get_bits(&c, 8) - 127;
+    uint32_t ub[16];
+    int32_t ib[16];
+    decode_ints(&c, maxbits - 9, ub, (unsigned)size);
+    if (dims == 2) {
+        for (int i = 0; i < 16; i++) ib[PERM2[i]] = orc_uint2int(ub[i]);
+        for (int x = 0; x < 4; x++) orc_inv_lift(ib + x, 4);     /* decode.cuh:203-214: y first, then x */
+        for (int y = 0; y < 4; y++) orc_inv_lift(ib + 4 * y, 1);
+    } else {
+        for (int i = 0; i < 4; i++) ib[i] = orc_uint2int(ub[i]);
+        orc_inv_lift(ib, 1);
+    }
+    float w = ldexpf(1.0f, emax - 30);
+    for (int i = 0; i < size; i++) fb[i] = w * (float)ib[i];
+}
+
+/* stream sizes: whole words, rounded UP for 1-D and 2-D (shared.h:42-71) */
+size_t orc_zfp_stream_bytes2(size_t nx, size_t ny, unsigned maxbits)
+{
+    size_t blocks = pad4(nx) * pad4(ny) / 16;
+    return ((blocks * (size_t)maxbits + 63) / 64) * sizeof(word_t);
+}
+size_t orc_zfp_stream_bytes1(size_t nx, unsigned maxbits)
+{
+    size_t blocks = pad4(nx) / 4;
+    return ((blocks * (size_t)maxbits + 63) / 64) * sizeof(word_t);
+}
+
+size_t orc_zfp_encode2_f32(const float *in, size_t nx, size_t ny, ptrdiff_t sx, ptrdiff_t sy,
+                           unsigned maxbits, word_t *stream)
+{
+    if (!sx) sx = 1;
+    if (!sy) sy = (ptrdiff_t)nx;
+    size_t mx = pad4(nx) / 4, my = pad4(ny) / 4, blocks = mx * my;
+    memset(stream, 0, ((blocks * (size_t)maxbits + 63) / 64) * sizeof(word_t));
+    for (size_t b = 0; b < blocks; b++) {
+        float fb[16];
+        size_t x0 = (b % mx) * 4, y0 = (b / mx) * 4;
+        unsigned bx = (unsigned)(nx - x0 < 4 ? nx - x0 : 4), by = (unsigned)(ny - y0 < 4 ? ny - y0 : 4);
+        const float *p = in + (ptrdiff_t)x0 * sx + (ptrdiff_t)y0 * sy;
+        for (unsigned y = 0; y < by; y++) {
+            for (unsigned x = 0; x < bx; x++) fb[4 * y + x] = p[x * sx + y * sy];
+            pad_vec(fb + 4 * y, bx, 1);
+        }
+        for (unsigned x = 0; x < 4; x++) pad_vec(fb + x, by, 4);
+        encode_block_low(fb, 2, maxbits, b, stream);
+    }
+    return orc_zfp_stream_bytes2(nx, ny, maxbits);
+}
+
+void orc_zfp_decode2_f32(const word_t *stream, size_t nx, size_t ny, ptrdiff_t sx, ptrdiff_t sy,
+                         unsigned maxbits, float *out)
+{
+    if (!sx) sx = 1;
+    if (!sy) sy = (ptrdiff_t)nx;
+    size_t mx = pad4(nx) / 4, my = pad4(ny) / 4, blocks = mx * my;
+    for (size_t b = 0; b < blocks; b++) {
+        float fb[16];
+        size_t x0 = (b % mx) * 4, y0 = (b / mx) * 4;
+        unsigned bx = (unsigned)(nx - x0 < 4 ? nx - x0 : 4), by = (unsigned)(ny - y0 < 4 ? ny - y0 : 4);
+        memset(fb, 0, sizeof fb);
+        decode_block_low(stream, 2, maxbits, b, fb);
+        float *p = out + (ptrdiff_t)x0 * sx + (ptrdiff_t)y0 * sy;
+        for (unsigned y = 0; y < by; y++)
+            for (unsigned x = 0; x < bx; x++) p[x * sx + y * sy] = fb[4 * y + x];
+    }
+}
+
+size_t orc_zfp_encode1_f32(const float *in, size_t nx, ptrdiff_t sx, unsigned maxbits, word_t *stream)
+{
+    if (!sx) sx = 1;
+    size_t blocks = pad4(nx) / 4;
+    memset(stream, 0, ((blocks * (size_t)maxbits + 63) / 64) * sizeof(word_t));
+    for (size_t b = 0; b < blocks; b++) {
+        float fb[4];
+        size_t x0 = b * 4;
+        unsigned bx = (unsigned)(nx - x0 < 4 ? nx - x0 : 4);
+        for (unsigned x = 0; x < bx; x++) fb[x] = in[(ptrdiff_t)(x0 + x) * sx];
+        pad_vec(fb, bx, 1);
+        encode_block_low(fb, 1, maxbits, b, stream);
+    }
+    return orc_zfp_stream_bytes1(nx, maxbits);
+}
+
+void orc_zfp_decode1_f32(const word_t *stream, size_t nx, ptrdiff_t sx, unsigned maxbits, float *out)
+{
+    if (!sx) sx = 1;
+    size_t blocks = pad4(nx) / 4;
+    for (size_t b = 0; b < blocks; b++) {
+        float fb[4] = {0, 0, 0, 0};
+        size_t x0 = b * 4;
+        unsigned bx = (unsigned)(nx - x0 < 4 ? nx - x0 : 4);
+        decode_block_low(stream, 1, maxbits, b, fb);
+        for (unsigned x = 0; x < bx; x++) out[(ptrdiff_t)(x0 + x) * sx] = fb[x];
     }
 }
 

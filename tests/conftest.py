@@ -20,6 +20,13 @@ def golden():
 
 
 @pytest.fixture(scope="session")
+def golden_12d():
+    import numpy as np
+
+    return np.load(os.path.join(ROOT, "tests", "golden", "zfp_golden_12d.npz"))
+
+
+@pytest.fixture(scope="session")
 def digests():
     import json
 
@@ -37,5 +44,5 @@ def golden_cases(g):
         for k in sorted(g.files):
             if k.startswith(n + "/r") and k.endswith("/stream"):
                 rate = float(k.split("/")[1][1:])
-                maxbits = int(np.floor(64 * rate + 0.5))
+                maxbits = int(np.floor(4 ** f.ndim * rate + 0.5))   # bits per block of 4^d values
                 yield n, rate, maxbits, f, g[k], g[k[: -len("stream")] + "dec"]

@@ -10,8 +10,9 @@ the committed ``zfp_golden.npz`` / ``zfp_digests.json``.
     python tests/golden/make_zfp_golden.py
 
 Fixture contents
-  zfp_golden.npz   small fields: ``<name>/in`` fp32 (nz,ny,nx), and per rate
+  zfp_golden.npz   small 3-D fields: ``<name>/in`` fp32 (nz,ny,nx), and per rate
                    ``<name>/r<rate>/stream`` (uint8) and ``<name>/r<rate>/dec``.
+  zfp_golden_12d.npz  the same for 2-D (ny,nx) and 1-D (nx,) fields.
   zfp_digests.json SHA-256 of input, stream and decoded output for the large
                    seeded configurations (inputs are re-created from the seed).
 """
@@ -32,11 +33,12 @@ from cswap_amd.workloads import config1_field, config3_fields  # noqa: E402
 
 
 def run_zfp(field: np.ndarray, rate: float):
-    nz, ny, nx = field.shape
+    """field: (nz, ny, nx), (ny, nx) or (nx,) -- x is always the fastest axis."""
+    dims = [str(n) for n in reversed(field.shape)]
     with tempfile.TemporaryDirectory() as d:
         fi, fz, fo = (os.path.join(d, n) for n in ("in.f32", "out.zfp", "out.f32"))
         field.astype("<f4").tofile(fi)
-        subprocess.check_call([ZFP, "-q", "-f", "-3", str(nx), str(ny), str(nz), "-r", repr(rate),
+        subprocess.check_call([ZFP, "-q", "-f", f"-{field.ndim}", *dims, "-r", repr(rate),
                                "-i", fi, "-z", fz, "-o", fo])
         stream = np.fromfile(fz, dtype=np.uint8)
         dec = np.fromfile(fo, dtype="<f4").reshape(field.shape)
@@ -76,6 +78,31 @@ def small_fields():
     return f
 
 
+def low_dim_fields():
+    rng = np.random.default_rng(4321)
+    f = {}
+    f["2d_rand_8x12"] = rng.standard_normal((8, 12)).astype(np.float32)
+    f["2d_partial_7x9"] = rng.standard_normal((7, 9)).astype(np.float32) * 50
+    f["2d_relu_16x16"] = np.maximum(rng.standard_normal((16, 16)), 0).astype(np.float32)
+    f["2d_row_1x5"] = rng.standard_normal((1, 5)).astype(np.float32)
+    z = rng.standard_normal((8, 8)).astype(np.float32)
+    z[0:4, 0:4] = 0.0
+    z[4:8, 4:8] = -2.25
+    f["2d_zero_const"] = z
+    g = np.arange(20, dtype=np.float32)
+    f["2d_smooth_20x20"] = np.exp(-((g[None, :] - 9) ** 2 + (g[:, None] - 11) ** 2) / 40).astype(np.float32)
+    f["1d_rand_64"] = rng.standard_normal(64).astype(np.float32)
+    f["1d_partial_13"] = (rng.standard_normal(13) * 1e-3).astype(np.float32)
+    f["1d_single"] = np.array([-7.5], dtype=np.float32)
+    o = rng.standard_normal(40).astype(np.float32)
+    o[8:16] = 0.0
+    f["1d_with_zero_blocks"] = o
+    f["1d_smooth_100"] = np.sin(np.arange(100, dtype=np.float32) / 9).astype(np.float32)
+    return f
+
+
+RATES_2D = [2, 4, 8, 12.5, 16, 32]      # maxbits = 16 * rate
+RATES_1D = [4, 8, 12, 16, 24, 32]       # maxbits = 4 * rate
 RATES_SMALL = [1, 2.5, 4, 4.5, 8, 9.75, 16, 20, 32]
 RATES_BIG = [4, 8, 16]
 
@@ -93,6 +120,15 @@ def main():
             out[f"{name}/r{r}/stream"] = stream
             out[f"{name}/r{r}/dec"] = dec
     np.savez_compressed(os.path.join(HERE, "zfp_golden.npz"), **out)
+
+    low = {}
+    for name, fld in low_dim_fields().items():
+        low[f"{name}/in"] = fld
+        for r in (RATES_2D if fld.ndim == 2 else RATES_1D):
+            stream, dec = run_zfp(fld, r)
+            low[f"{name}/r{r}/stream"] = stream
+            low[f"{name}/r{r}/dec"] = dec
+    np.savez_compressed(os.path.join(HERE, "zfp_golden_12d.npz"), **low)
 
     dig = {}
     big = {"config1_prelu_4096x32x32": config1_field()}

@@ -47,6 +47,40 @@ void host_zfp_decode3(const uint64_t* stream, size_t nx, size_t ny, size_t nz, u
   }
 }
 
+// 2-D field a[ny][nx] (ny = 0: 1-D field a[nx])
+void host_zfp_encode_low(const float* in, size_t nx, size_t ny, unsigned maxbits, uint64_t* stream)
+{
+  const int dims = ny ? 2 : 1;
+  size_t mx = (nx + 3) / 4, my = ny ? (ny + 3) / 4 : 1;
+  for (size_t b = 0; b < mx * my; b++) {
+    size_t x0 = (b % mx) * 4, y0 = (b / mx) * 4;
+    unsigned bx = nx - x0 < 4 ? nx - x0 : 4, by = dims == 2 ? (ny - y0 < 4 ? ny - y0 : 4) : 1;
+    float f[16];
+    for (int i = 0; i < 16; i++) f[i] = 0.0f;
+    for (unsigned y = 0; y < by; y++) for (unsigned x = 0; x < bx; x++) f[x + 4 * y] = in[(x0 + x) + nx * (y0 + y)];
+    for (unsigned y = 0; y < (dims == 2 ? 4u : 1u); y++) cswap::pad4(f[4 * y], f[4 * y + 1], f[4 * y + 2], f[4 * y + 3], bx);
+    if (dims == 2) for (int x = 0; x < 4; x++) cswap::pad4(f[x], f[x + 4], f[x + 8], f[x + 12], by);
+    ArrayBits mem{reinterpret_cast<uint32_t*>(stream)};
+    if (dims == 2) cswap::encode_block_low<2, true>(f, (unsigned)(b * (size_t)maxbits), maxbits, mem);
+    else cswap::encode_block_low<1, true>(f, (unsigned)(b * (size_t)maxbits), maxbits, mem);
+  }
+}
+
+void host_zfp_decode_low(const uint64_t* stream, size_t nx, size_t ny, unsigned maxbits, float* out)
+{
+  const int dims = ny ? 2 : 1;
+  size_t mx = (nx + 3) / 4, my = ny ? (ny + 3) / 4 : 1;
+  for (size_t b = 0; b < mx * my; b++) {
+    size_t x0 = (b % mx) * 4, y0 = (b / mx) * 4;
+    unsigned bx = nx - x0 < 4 ? nx - x0 : 4, by = dims == 2 ? (ny - y0 < 4 ? ny - y0 : 4) : 1;
+    float f[16];
+    ArrayBits mem{reinterpret_cast<uint32_t*>(const_cast<uint64_t*>(stream))};
+    if (dims == 2) cswap::decode_block_low<2>(mem, (unsigned)(b * (size_t)maxbits), maxbits, f);
+    else cswap::decode_block_low<1>(mem, (unsigned)(b * (size_t)maxbits), maxbits, f);
+    for (unsigned y = 0; y < by; y++) for (unsigned x = 0; x < bx; x++) out[(x0 + x) + nx * (y0 + y)] = f[x + 4 * y];
+  }
+}
+
 void host_transpose32(uint32_t* a) { uint32_t t[32]; memcpy(t, a, sizeof t); cswap::transpose32(t); memcpy(a, t, sizeof t); }
 
 }

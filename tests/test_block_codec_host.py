@@ -23,6 +23,8 @@ def host():
     L.host_zfp_encode3.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     L.host_zfp_decode3.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     L.host_transpose32.argtypes = [C.c_void_p]
+    L.host_zfp_encode_low.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
+    L.host_zfp_decode_low.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     return L
 
 
@@ -54,3 +56,25 @@ def test_block_codec_matches_golden_vectors(host, golden):
         assert np.array_equal(o.view(np.uint32), dec.view(np.uint32)), (name, rate)
         n += 1
     assert n >= 100
+
+
+def test_low_dimensional_block_codecs_match_golden_vectors(host, golden_12d):
+    n = 0
+    for name, rate, maxbits, f, stream, dec in golden_cases(golden_12d):
+        nx = f.shape[-1]
+        ny = f.shape[0] if f.ndim == 2 else 0
+        blocks = -(-nx // 4) * (-(-ny // 4) if ny else 1)
+        words = (blocks * maxbits + 63) // 64
+        s = np.zeros(words + 2, dtype=np.uint64)
+        host.host_zfp_encode_low(f.ctypes.data, nx, ny, maxbits, s.ctypes.data)
+        sb = s[:words].view(np.uint8)
+        k = min(sb.size, stream.size)
+        assert np.array_equal(sb[:k], stream[:k]), (name, rate)
+        assert not sb[k:].any() and not stream[k:].any()
+        g = np.zeros((words + 2) * 8, dtype=np.uint8)
+        g[:k] = stream[:k]
+        o = np.zeros_like(f)
+        host.host_zfp_decode_low(g.ctypes.data, nx, ny, maxbits, o.ctypes.data)
+        assert np.array_equal(o.view(np.uint32), dec.view(np.uint32)), (name, rate)
+        n += 1
+    assert n >= 60

@@ -183,6 +183,20 @@ def test_reference_named_entry_points(torch_cuda):
     fh[:] = 0
     L.cuda_decompress(C.byref(zs2), C.byref(fld2))
     assert np.array_equal(fh.view(np.uint32), oracle.zfp_decode3(want, f.shape, 1024).view(np.uint32))
+    # a 2-D field (nz = 0) goes through the 4x4-block codec (cuZFP.cu:105-151 picks by dimensionality)
+    f2 = rng.standard_normal((20, 36)).astype(np.float32)
+    t2 = torch.from_numpy(f2).cuda()
+    cap2 = L.cswap_zfp_stream_capacity_nd(2, 36, 20, 0, 128)
+    s2 = torch.zeros(cap2, dtype=torch.uint8, device="cuda")
+    bs3 = ZfpBitstream(0, 0, s2.data_ptr(), s2.data_ptr(), s2.data_ptr() + cap2)
+    zs3 = ZfpStream(1, 128, 64, -1074, C.pointer(bs3), 0, 0, 0)
+    fld4 = ZfpField(3, 36, 20, 0, 0, 0, 0, 0, 0, t2.data_ptr())
+    assert L.cuda_compress(C.byref(zs3), C.byref(fld4)) == cap2
+    want2 = oracle.zfp_encode_nd(f2, 128)
+    assert np.array_equal(s2.cpu().numpy().view(np.uint64), want2)
+    t2.zero_()
+    L.cuda_decompress(C.byref(zs3), C.byref(fld4))
+    assert np.array_equal(t2.cpu().numpy().view(np.uint32), oracle.zfp_decode_nd(want2, f2.shape, 128).view(np.uint32))
     # unsupported: double fields -> failure value 0
     fld3 = ZfpField(4, 16, 8, 12, 0, 0, 0, 0, 0, t.data_ptr())
     assert L.cuda_compress(C.byref(zs), C.byref(fld3)) == 0

@@ -163,3 +163,58 @@ def test_large_tensor_properties(torch_cuda):
     # (b) rate 8 keeps ~3 significant bits of the block maximum: the error stays
     # well below the largest value of the field
     assert float((d - x).abs().max()) < 0.125 * float(x.max())
+
+
+def nd_args(shape):
+    """(dims, nx, ny, nz) of a C-contiguous field of 1, 2 or 3 dimensions."""
+    ext = list(reversed(shape)) + [0, 0]
+    return len(shape), ext[0], ext[1], ext[2]
+
+
+def gpu_codec_nd(torch, f, maxbits, stream_bytes=None):
+    from cswap_amd._lib import check, lib
+
+    L = lib()
+    dims, nx, ny, nz = nd_args(f.shape)
+    cap = L.cswap_zfp_stream_capacity_nd(dims, nx, ny, nz, maxbits)
+    t = torch.from_numpy(np.ascontiguousarray(f)).cuda()
+    s = torch.empty(cap, dtype=torch.uint8, device="cuda")
+    check(L.cswap_zfp_compress_f32_nd(t.data_ptr(), dims, nx, ny, nz, 0, 0, 0, maxbits, s.data_ptr(), None), "enc")
+    if stream_bytes is not None:          # decode a given stream instead of our own
+        g = np.zeros(cap, dtype=np.uint8)
+        k = min(cap, stream_bytes.size)
+        g[:k] = stream_bytes[:k]
+        src = torch.from_numpy(g).cuda()
+    else:
+        src = s
+    out = torch.full(f.shape, -3.0, dtype=torch.float32, device="cuda")
+    check(L.cswap_zfp_decompress_f32_nd(src.data_ptr(), dims, nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(), None),
+          "dec")
+    torch.cuda.synchronize()
+    return s.cpu().numpy(), out.cpu().numpy()
+
+
+def test_golden_vectors_1d_2d(torch_cuda, golden_12d):
+    n = 0
+    for name, rate, maxbits, f, stream, dec in golden_cases(golden_12d):
+        print("case", name, rate, flush=True)
+        sb, d = gpu_codec_nd(torch_cuda, f, maxbits, stream_bytes=stream)
+        k = min(sb.size, stream.size)
+        assert np.array_equal(sb[:k], stream[:k]), (name, rate)
+        assert not sb[k:].any() and not stream[k:].any(), (name, rate)
+        assert np.array_equal(d.view(np.uint32), dec.view(np.uint32)), (name, rate)
+        n += 1
+    assert n >= 60
+
+
+@pytest.mark.parametrize("shape,maxbits", [((1000, 333), 128), ((257, 1030), 200), ((4096, 768), 64),
+                                            ((100003,), 32), ((1 << 20,), 48), ((777,), 16)])
+def test_larger_1d_2d_fields_vs_checker(torch_cuda, shape, maxbits):
+    import oracle
+
+    rng = np.random.default_rng(sum(shape) + maxbits)
+    f = np.maximum(rng.standard_normal(shape), -0.2).astype(np.float32)
+    sb, d = gpu_codec_nd(torch_cuda, f, maxbits)
+    want = oracle.zfp_encode_nd(f, maxbits)
+    assert np.array_equal(sb.view(np.uint64), want)
+    assert np.array_equal(d.view(np.uint32), oracle.zfp_decode_nd(want, f.shape, maxbits).view(np.uint32))

@@ -245,3 +245,26 @@ def test_ref_host_bitstream_order_and_max_size():
     # the first 9 bits are what the checker writes as a header for e = 130
     blk = np.zeros(64, np.float32); blk[0] = 5.0  # emax = 3 -> e = 130
     assert int(oracle.zfp_encode_block(blk, 512)[0]) & 0x1ff == int(buf[0]) & 0x1ff
+
+
+def test_golden_streams_and_decodes_1d_2d(golden_12d):
+    """The 2-D and 1-D restatements (4x4 and 4-value blocks) against zfp 0.5.5."""
+    n = 0
+    for name, rate, maxbits, f, stream, dec in golden_cases(golden_12d):
+        s = oracle.zfp_encode_nd(f, maxbits).view(np.uint8)
+        k = min(s.size, stream.size)
+        assert np.array_equal(s[:k], stream[:k]), (name, rate)
+        assert not s[k:].any() and not stream[k:].any(), (name, rate)
+        pad = np.zeros((-stream.size) % 8, dtype=np.uint8)
+        d = oracle.zfp_decode_nd(np.concatenate([stream, pad]).view(np.uint64), f.shape, maxbits)
+        assert np.array_equal(d.view(np.uint32), dec.view(np.uint32)), (name, rate)
+        n += 1
+    assert n >= 60
+
+
+def test_perm2_is_sequency_sorted_permutation():
+    p = np.zeros(16, dtype=np.uint8)
+    oracle.lib().orc_perm2(p.ctypes.data)
+    assert sorted(p) == list(range(16))
+    keys = [((i & 3) + (i >> 2), (i & 3) ** 2 + (i >> 2) ** 2) for i in p]
+    assert keys == sorted(keys)
