@@ -1,0 +1,77 @@
+"""The Execution mirror on a VGG-16-shaped forward walk with the policy vector of
+the reference driver (ZVC for ReLU outputs, ZFP for pooled outputs,
+CSWAP+/vgg16-cifar10.cpp:177-178 and the commented mix at :393-394)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_vgg_walk_with_reference_policy_vector():
+    import torch
+
+    import oracle
+    from cswap_amd import swap
+    from cswap_amd.execution import ACT, Execution
+
+    assert torch.cuda.is_available()
+    torch.manual_seed(0)
+    # first 14 ops of VGG-16 (types as in vgg16-cifar10.cpp:177-178), small batch
+    ops = [("conv", 3, 64), ("bn", 64), ("relu",), ("conv", 64, 64), ("bn", 64), ("relu",), ("pool",),
+           ("conv", 64, 128), ("bn", 128), ("relu",), ("conv", 128, 128), ("bn", 128), ("relu",), ("pool",)]
+    mods = []
+    for o in ops:
+        if o[0] == "conv":
+            mods.append(torch.nn.Conv2d(o[1], o[2], 3, padding=1).cuda())
+        elif o[0] == "bn":
+            mods.append(torch.nn.BatchNorm2d(o[1]).cuda())
+        elif o[0] == "relu":
+            mods.append(torch.nn.ReLU())
+        else:
+            mods.append(torch.nn.MaxPool2d(2))
+    eng = swap.SwapEngine(pinned_bytes=512 << 20, device_bytes=512 << 20)
+    exe = Execution(eng)
+    exe.init_(50)
+    for i in (2, 9):
+        exe.policy[i] = 3        # ReLU outputs feeding a conv: ZVC
+    for i in (6, 13):
+        exe.policy[i] = 6        # pool outputs: ZFP
+    exe.policy[5] = 2            # one raw swap (vDNN style)
+    exe.policy[12] = -1          # and one left to the selector
+
+    x = torch.randn(32, 3, 64, 64, device="cuda")
+    kept = {}
+    with torch.no_grad():
+        exe.preforward()
+        pre, pre_id = x, -1
+        for m in mods:
+            exe.pre(pre, pre_id, ACT)
+            out = m(pre)
+            out_id = exe.post()
+            if exe.swapped(pre_id):
+                kept[pre_id] = pre.clone()     # what the device copy held when it was swapped out
+            pre, pre_id = out, out_id
+        # the consumer of the last tensor (the next conv in the real model)
+        exe.pre(pre, pre_id, ACT)
+        exe.post()
+        if exe.swapped(pre_id):
+            kept[pre_id] = pre.clone()
+        exe.postforward()
+    assert exe.index == len(mods)
+    assert sorted(kept) == [2, 5, 6, 9, 12, 13]
+    assert exe.com_and_tran(2) == 3 and exe.com_and_tran(6) == 6 and exe.com_and_tran(5) == 2
+    assert exe.com_and_tran(12) in (2, 3, 6) and exe.com_and_tran(0) == 0
+
+    for tid in sorted(kept, reverse=True):       # backward order
+        tag = exe.com_and_tran(tid)
+        back = exe.fetch(tid)
+        torch.cuda.synchronize()
+        ref = kept[tid]
+        if tag == 6:
+            f = ref.cpu().numpy().reshape(-1, ref.shape[-2], ref.shape[-1])
+            want = oracle.zfp_decode3(oracle.zfp_encode3(f, 512, omp=True), f.shape, 512, omp=True)
+            assert np.array_equal(back.cpu().numpy().reshape(f.shape).view(np.uint32), want.view(np.uint32))
+        else:
+            assert torch.equal(back, ref)
+        assert not exe.swapped(tid)
+    eng.close()
