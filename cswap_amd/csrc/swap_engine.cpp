@@ -319,7 +319,12 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   }
 
   size_t hoff;
-  if (!e->hpool.alloc(t.bytes_out, &hoff)) { drop_device(e, t); return CSWAP_E_NOMEM; }
+  if (!e->hpool.alloc(t.bytes_out, &hoff)) {
+    // the compression kernel may still be writing the staging block: let it finish before the block is reused
+    (void)hipStreamSynchronize(compute);
+    drop_device(e, t);
+    return CSWAP_E_NOMEM;
+  }
   t.host_off = hoff; t.host_bytes = t.bytes_out;
 
   // ---- copy on the copy stream, ordered after the compression by an event
@@ -328,6 +333,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   if (err == hipSuccess) err = hipMemcpyAsync(e->h_base + hoff, src, t.bytes_out, hipMemcpyDeviceToHost, e->copy);
   if (err == hipSuccess) err = hipEventRecord(t.ev_copy, e->copy);
   if (err != hipSuccess) {
+    (void)hipStreamSynchronize(compute);
     (void)hipStreamSynchronize(e->copy);
     drop_device(e, t);
     e->hpool.free(t.host_off, t.host_bytes);

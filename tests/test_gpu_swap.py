@@ -113,6 +113,37 @@ def test_many_in_flight_and_overlap_ordering(torch_cuda, engine):
         assert torch.equal(x, k)
 
 
+def test_copies_are_ordered_against_compute_by_events(torch_cuda, engine):
+    """The outbound copy must not start before the compute stream has produced the
+    tensor, and consumers on the compute stream must see the swapped-in data
+    without any host synchronisation in between."""
+    torch = torch_cuda
+    from cswap_amd import swap
+
+    a = torch.randn(4096, 4096, device="cuda")
+    for pol in (swap.NONE, swap.SPARSE, swap.ZFP):
+        x = torch.zeros(8, 64, 32, 32, device="cuda")
+        b = a
+        for _ in range(8):                       # tens of ms of queued compute ...
+            b = (b @ a) * 1e-2
+        x.fill_(7.0)                              # ... and only then the data to be swapped
+        x[0, 0, 0, :8] = 0.0
+        tk = engine.pre(x, pol)                   # returns while the matmuls are still running
+        engine.post(tk)
+        want = x.clone()
+        x.fill_(-1.0)
+        out = torch.empty_like(x)
+        engine.swap_in(tk, out)
+        total = out.sum()                         # consumer queued right behind the swap-in, no sync
+        torch.cuda.synchronize()
+        engine.release(tk)
+        if pol == swap.ZFP:
+            assert float((out - want).abs().max()) < 0.1
+        else:
+            assert torch.equal(out, want)
+            assert float(total) == float(want.sum())
+
+
 def test_state_machine_errors(torch_cuda, engine):
     torch = torch_cuda
     from cswap_amd._lib import lib
