@@ -201,6 +201,37 @@ def extras(torch, api, dev):
                 "decompress_hbm_frac": round(bpv * n / d / 1e6 / HBM_PEAK_GBS, 4)}
     del big
 
+    # ---- configuration 5's other tensors (rates 8 and 16) and configuration 3's stack (rates 4/8/16)
+    from cswap_amd.workloads import config3_fields, config5_tensor_torch
+
+    def zfp_case(key, t, rate):
+        n = t.numel()
+        nx, ny, nz = field_dims(t.shape)
+        mb = 64 * rate
+        s = torch.empty(api.zfp_stream_capacity(nx, ny, nz, mb), dtype=torch.uint8, device=dev)
+        o = torch.empty_like(t)
+        api.cuda_compress(t, mb, out=s); api.cuda_decompress(s, t.shape, mb, out=o)
+        reps = 10 if n > 1 << 24 else 50
+        e = ev_ms(torch, lambda: api.cuda_compress(t, mb, out=s), reps)
+        d = ev_ms(torch, lambda: api.cuda_decompress(s, t.shape, mb, out=o), reps)
+        bpv = 4 + rate / 8
+        ex[key] = {"MB": round(4 * n / 1e6, 1), "compress_ms": round(e, 4), "decompress_ms": round(d, 4),
+                   "pair_GBs_fp32": round(4 * n / (e + d) / 1e6, 1),
+                   "compress_hbm_frac": round(bpv * n / e / 1e6 / HBM_PEAK_GBS, 4),
+                   "decompress_hbm_frac": round(bpv * n / d / 1e6 / HBM_PEAK_GBS, 4),
+                   "stream_over_input": round(s.numel() / (4 * n), 4)}
+
+    for name in ("hidden_gelu", "ffn_gelu"):
+        t = config5_tensor_torch(name, dev, seed=0)
+        for rate in (8, 16):
+            zfp_case(f"zfp_config5_{name}_r{rate}", t, rate)
+        del t
+    for name, f in config3_fields(batch=128).items():
+        t = torch.from_numpy(f).to(dev)
+        for rate in (4, 8, 16):
+            zfp_case(f"zfp_config3_{name}_r{rate}", t, rate)
+        del t
+
     # ---- ZVC compact / expand / probe
     def zvc_case(label, t):
         n = t.numel()
