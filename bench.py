@@ -127,7 +127,7 @@ def main():
         "metric": "compress+decompress GB/s (fp32 in), ZFP fixed-rate 8 bits/value, 1xMI355X",
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32->i32/u64 bit planes", "data": "synthetic",
+        "vs_baseline": None, "dtype": "i32", "data": "synthetic",
         "config": {"workload": "config5 attention probabilities fp32 [32,12,512,512] = softmax(N(0,1)), "
                                "zfp field nx=512 ny=512 nz=384, rate 8 (maxbits 512), compress then decompress",
                    "bytes_in": 4 * n, "rate_bits_per_value": rate},

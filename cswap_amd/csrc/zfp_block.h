@@ -219,6 +219,20 @@ CSWAP_HD uint32_t block_header_e(const float (&f)[64])
 #define CSWAP_ANY(pred) (pred)
 #endif
 
+// bit position -> dword index.  On the device the shift is opaque to the compiler
+// so that the LDS byte address becomes one shift-add (index * 4 + base) instead
+// of shift, mask and add.
+CSWAP_HD unsigned dword_of(unsigned bitpos)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  unsigned d;
+  asm("v_lshrrev_b32 %0, 5, %1" : "=v"(d) : "v"(bitpos));
+  return d;
+#else
+  return bitpos >> 5;
+#endif
+}
+
 CSWAP_HD uint32_t funnel_shr(uint32_t hi, uint32_t lo, unsigned s)  // ({hi,lo} >> (s & 31)) low word
 {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -253,7 +267,7 @@ struct BlockEncoder {
       unsigned room = limit - pos;
       if (len > room) v &= low_mask(room);
     }
-    unsigned d = pos >> 5, s = pos & 31;
+    unsigned d = dword_of(pos), s = pos & 31;
     uint64_t lo = v << s;
     uint32_t hi = ((uint32_t)(v >> 32) >> 1) >> (31 - s);
     mem.or32(d, (uint32_t)lo);
@@ -265,16 +279,17 @@ struct BlockEncoder {
   CSWAP_HD void set_bit(unsigned b, bool on)
   {
     if (GUARD) on = on && b < limit;
-    mem.or32(b >> 5, on ? (1u << (b & 31)) : 0u);
+    mem.or32(dword_of(b), on ? (1u << (b & 31)) : 0u);
   }
 
   // one bit plane: x bit i = this plane's bit of coefficient i (encode.cuh:331-344)
   CSWAP_HD void plane(uint64_t x)
   {
     if (!active()) return;
-    put(x & low_mask(n), n);  // first n coefficients verbatim
+    // first n coefficients verbatim: x minus its part at and above bit n
+    uint64_t rest = n < 64 ? x >> n : 0;
+    put(n < 64 ? x ^ (rest << n) : x, n);
     if (n < SIZE) {
-      uint64_t rest = x >> n;
       while (rest != 0 && n < SIZE && pos < limit) {
         unsigned t = (unsigned)ctz64(rest);  // zeros before the next one-bit
         unsigned nt = n + t;
@@ -346,7 +361,7 @@ struct BlockDecoder {
 
   CSWAP_HD uint64_t window(unsigned p) const  // 64 stream bits starting at bit p
   {
-    unsigned d = p >> 5;
+    unsigned d = dword_of(p);
     uint32_t w0 = mem.ld32(d), w1 = mem.ld32(d + 1), w2 = mem.ld32(d + 2);
     return ((uint64_t)funnel_shr(w2, w1, p) << 32) | funnel_shr(w1, w0, p);
   }
