@@ -263,3 +263,52 @@ def test_reference_named_entry_points(torch_cuda):
     L.GPUdecompression(vals.data_ptr(), dest.data_ptr(), nE, 16384, mask.data_ptr(), idx.data_ptr(), 512, 32)
     torch.cuda.synchronize()
     assert torch.equal(dest, r) and k == int((r != 0).sum().item())
+
+
+def test_simple_c_harness(torch_cuda):
+    """What the reference's only executable check does (CSWAP+/simple.c:107-159): a
+    2560x512x50 float field with values (r1 + x+y+z) / (x+y+z + r2) * (-1)^(i+j+k),
+    r1 in 0..19, r2 in 0..2, x,y,z in [0,2), handed to cuda_compress as HOST memory
+    with a freshly opened zfp_stream (maxbits = 1024, CSWAP+/zfp/zfp.h:23), zeroed,
+    cuda_decompress-ed, and compared element by element.  simple.c draws r1, r2 from
+    an unseeded rand() in an unspecified evaluation order, so the same value law is
+    generated here from a seeded generator; simple.c asserts nothing, this test
+    additionally requires bit-equality with the CPU checker."""
+    torch = torch_cuda
+    import oracle
+    from cswap_amd._lib import ZfpBitstream, ZfpField, ZfpStream, lib
+
+    L = lib()
+    nx, ny, nz = 2560, 512, 50
+    rng = np.random.default_rng(2024)
+    i = (2.0 * np.arange(nx) / nx)[None, None, :]
+    j = (2.0 * np.arange(ny) / ny)[None, :, None]
+    k = (2.0 * np.arange(nz) / nz)[:, None, None]
+    base = i + j + k
+    r1 = rng.integers(0, 20, size=(nz, ny, nx))
+    r2 = rng.integers(0, 3, size=(nz, ny, nx))
+    sign = 1.0 - 2.0 * ((np.arange(nx)[None, None, :] + np.arange(ny)[None, :, None]
+                         + np.arange(nz)[:, None, None]) % 2)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        a = ((r1 + base) / (base + r2) * sign)
+    a[~np.isfinite(a)] = 0.0                       # the single 0/0 at the origin when r2 == 0
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    ori = a.copy()
+
+    maxbits = 1024
+    cap = L.cswap_zfp_stream_capacity(nx, ny, nz, maxbits)
+    buf = np.zeros(cap, dtype=np.uint8)            # host buffer, as simple.c's malloc
+    bs = ZfpBitstream(0, 0, buf.ctypes.data, buf.ctypes.data, buf.ctypes.data + cap)
+    zs = ZfpStream(1, maxbits, 64, -1074, C.pointer(bs), 0, 0, 0)
+    fld = ZfpField(3, nx, ny, nz, 0, 0, 0, 0, 0, a.ctypes.data)
+    zfpsize = L.cuda_compress(C.byref(zs), C.byref(fld))
+    assert zfpsize == cap == (nx // 4) * (ny // 4) * 13 * 128   # 16 bits/value over nz padded from 50 to 52
+    a[:] = 0
+    L.cuda_decompress(C.byref(zs), C.byref(fld))
+    cnt = int(np.count_nonzero(a != ori))          # simple.c's "error cnt" (lossy: most values differ)
+    rel = float(np.mean(np.abs((ori.ravel()[:1000] - a.ravel()[:1000]) / ori.ravel()[:1000])))
+    print(f"simple.c harness: zfpsize {zfpsize / 2**20:.1f} MB, error cnt {cnt}, accuracy loss {rel:.3e}")
+    assert rel < 0.05                               # rate 16 on a field with sign flips and 1/x spikes
+    want = oracle.zfp_encode3(ori, maxbits, omp=True)
+    assert np.array_equal(buf.view(np.uint64), want)
+    assert np.array_equal(a.view(np.uint32), oracle.zfp_decode3(want, ori.shape, maxbits, omp=True).view(np.uint32))
