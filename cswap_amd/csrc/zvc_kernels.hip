@@ -225,6 +225,81 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand_kernel(
   }
 }
 
+// Same expansion with one lane = four consecutive elements and 16-byte stores:
+// the per-element form above issues one 4-byte store per lane and is bound by
+// that instruction stream, not by bytes.  A row is 256 elements = 8 mask words;
+// lane l keeps mask word 64*(row/8) + l of the chunk, together with the number
+// of set bits in the words before it inside its row, so a lane finds its nibble
+// and the rank of its first element with two cross-lane reads.
+// Needs E % 4 == 0 and a 16-byte aligned destination (every chunk then starts
+// on a 16-byte boundary); the caller checks.
+constexpr int kRowsInFlight = 8;  // divides the 8 rows one refill covers
+
+__global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand4_kernel(
+    const float* __restrict__ values, const uint32_t* __restrict__ mask, const int* __restrict__ begin,
+    Geometry g, float* __restrict__ out)
+{
+  const int c = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
+  if (c >= g.active) return;
+  const unsigned lane = lane_id();
+  const long long b = (long long)g.E * c;
+  const int len = (int)min((long long)g.E, (long long)g.n - b);
+  const uint32_t* mrow = mask + (size_t)c * g.W;
+  float* q = out + b;
+  unsigned off = (unsigned)begin[c];
+  const int rows = (len + 255) >> 8;
+  const unsigned sub = lane & 7u;  // my nibble inside the word I read
+  const uint32_t below = (1u << (4u * sub)) - 1u;
+  uint32_t held = 0, pre = 0;  // pre: low half = set bits before my word in its row, high half = through it
+  for (int r0 = 0; r0 < rows; r0 += kRowsInFlight) {
+    {  // refill: 64 words = 8 rows
+      const int w = (r0 >> 3) * 64 + (int)lane;
+      held = w < g.W ? mrow[w] : 0u;
+      const int first = w * 32;  // bits past the end of the chunk carry no data
+      if (first + 32 > len) held = first >= len ? 0u : (held & ((1u << (len - first)) - 1u));
+      const uint32_t cnt = (uint32_t)__popc(held);
+      uint32_t s = cnt;
+#pragma unroll
+      for (int o = 1; o < 8; o <<= 1) {
+        const uint32_t t = (uint32_t)__shfl_up((int)s, o, 64);
+        if (sub >= (unsigned)o) s += t;
+      }
+      pre = (s - cnt) | (s << 16);
+    }
+    float4 x[kRowsInFlight];
+#pragma unroll
+    for (int j = 0; j < kRowsInFlight; j++) {
+      const int src = (j << 3) + (int)(lane >> 3);
+      const uint32_t w = (uint32_t)__shfl((int)held, src, 64);
+      const uint32_t p = (uint32_t)__shfl((int)pre, src, 64);
+      const uint32_t row_total = (uint32_t)__builtin_amdgcn_readlane((int)pre, (j << 3) + 7) >> 16;
+      const uint32_t nib = (w >> (4u * sub)) & 15u;
+      unsigned rk = off + (p & 0xffffu) + (unsigned)__popc(w & below);
+      float4 v;
+      v.x = (nib & 1u) ? values[rk] : 0.0f;
+      rk += nib & 1u;
+      v.y = (nib & 2u) ? values[rk] : 0.0f;
+      rk += (nib >> 1) & 1u;
+      v.z = (nib & 4u) ? values[rk] : 0.0f;
+      rk += (nib >> 2) & 1u;
+      v.w = (nib & 8u) ? values[rk] : 0.0f;
+      x[j] = v;
+      off += row_total;
+    }
+#pragma unroll
+    for (int j = 0; j < kRowsInFlight; j++) {
+      const int k = (r0 + j) * 256 + 4 * (int)lane;
+      if (k + 4 <= len) {
+        *reinterpret_cast<float4*>(q + k) = x[j];
+      } else {  // ragged end of the last chunk
+        if (k < len) q[k] = x[j].x;
+        if (k + 1 < len) q[k + 1] = x[j].y;
+        if (k + 2 < len) q[k + 2] = x[j].z;
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------------ fused
 // count + scan + compact in ONE pass over the tensor: a wavefront keeps its whole
 // chunk in registers (IT values per lane) and counts it; the WAVES chunks of a
@@ -499,8 +574,12 @@ extern "C" int cswap_zvc_expand(const float* d_values, const uint32_t* d_mask, c
   int rc = make_geometry(g, n, process);
   if (rc) return rc;
   unsigned grid = (g.active + kWavesPerGroup - 1) / kWavesPerGroup;
-  hipLaunchKernelGGL(zvc_expand_kernel, dim3(grid), dim3(64 * kWavesPerGroup), 0, (hipStream_t)stream,
-                     d_values, d_mask, d_begin, g, d_out);
+  if (g.E % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out) & 15u) == 0)
+    hipLaunchKernelGGL(zvc_expand4_kernel, dim3(grid), dim3(64 * kWavesPerGroup), 0, (hipStream_t)stream,
+                       d_values, d_mask, d_begin, g, d_out);
+  else
+    hipLaunchKernelGGL(zvc_expand_kernel, dim3(grid), dim3(64 * kWavesPerGroup), 0, (hipStream_t)stream,
+                       d_values, d_mask, d_begin, g, d_out);
   return check_launch();
 }
 

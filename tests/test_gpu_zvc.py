@@ -68,6 +68,33 @@ def test_other_chunk_counts(torch_cuda, process):
     check_against_oracle(x, run_gpu(torch_cuda, x, process), process)
 
 
+@pytest.mark.parametrize("n,process", [(P * 8 - 3, P), (P * 260 - 1, P), (P * 512 - 2, P), (P * 2052 - 7, P),
+                                        (P * 4096 - 254, P), (28, 7), (5000, 1), (299_992, 7), (64 * 2048, 64)])
+def test_expand_four_per_lane(torch_cuda, n, process):
+    """Chunk lengths that are multiples of four take the 16-byte-store expansion;
+    the sizes end the last chunk inside a quad, inside a row and inside a refill
+    group.  The same data is then expanded into a destination that is only
+    4-byte aligned, which takes the per-element kernel: both must agree."""
+    import oracle
+    from cswap_amd import api
+
+    torch = torch_cuda
+    E, W, K = oracle.zvc_geometry(n, process)
+    assert E % 4 == 0
+    rng = np.random.default_rng(n + process)
+    x = (rng.standard_normal(n) * (rng.random(n) < rng.uniform(0.1, 0.9))).astype(np.float32)
+    print("n", n, "process", process, "E", E, flush=True)
+    got = run_gpu(torch, x, process)
+    check_against_oracle(x, got, process)
+    t = torch.from_numpy(x).cuda()
+    values, mask, begin, nnz = api.zvc_compress(t, process)
+    buf = torch.full((n + 1,), -1.0, device="cuda")
+    api.GPUdecompression(values, buf[1:], mask, begin, process)
+    torch.cuda.synchronize()
+    assert float(buf[0]) == -1.0
+    assert np.array_equal(buf[1:].cpu().numpy().view(np.uint32), got[4].view(np.uint32))
+
+
 @pytest.mark.parametrize("pct", [30, 50, 70, 90])
 def test_fused_single_pass_config2(torch_cuda, pct):
     from cswap_amd.workloads import config2_tensor
