@@ -233,6 +233,17 @@ CSWAP_HD unsigned dword_of(unsigned bitpos)
 #endif
 }
 
+// Makes the compiler finish computing v at this point instead of sinking part of
+// it into a later branch (used where one LDS round trip should cover two uses).
+CSWAP_HD void settle(uint64_t& v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" : "+v"(v));
+#else
+  (void)v;
+#endif
+}
+
 CSWAP_HD uint32_t funnel_shr(uint32_t hi, uint32_t lo, unsigned s)  // ({hi,lo} >> (s & 31)) low word
 {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -386,6 +397,7 @@ struct BlockDecoder {
     pos += m;
     while (n < SIZE && pos < limit) {
       uint64_t w = window(pos);
+      settle(w);
       pos++;
       if (!(w & 1)) break;  // negative group test: plane done
       w >>= 1;              // 63 valid bits
