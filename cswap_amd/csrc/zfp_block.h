@@ -63,6 +63,7 @@ struct Perm3 {
 constexpr Perm3 kPerm3 = {{CSWAP_PERM3_LIST}};
 
 // ---------------------------------------------------------------- small helpers
+constexpr uint32_t kNegabinary = 0xaaaaaaaau;
 CSWAP_HD uint32_t int2nb(int32_t x) { return ((uint32_t)x + 0xaaaaaaaau) ^ 0xaaaaaaaau; }
 CSWAP_HD int32_t nb2int(uint32_t u) { return (int32_t)((u ^ 0xaaaaaaaau) - 0xaaaaaaaau); }
 
@@ -78,6 +79,15 @@ CSWAP_HD int ctz64(uint64_t v)  // 64 for v == 0
 CSWAP_HD uint64_t low_mask(unsigned n)  // n in 0..64
 {
   return n >= 64 ? ~(uint64_t)0 : (((uint64_t)1 << n) - 1);
+}
+
+CSWAP_HD unsigned sub_sat(unsigned a, unsigned b)  // max(a - b, 0)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_elementwise_sub_sat(a, b);
+#else
+  return a > b ? a - b : 0u;
+#endif
 }
 
 CSWAP_HD float f32_from_bits(uint32_t b)
@@ -167,28 +177,94 @@ CSWAP_HD void inv_xform3(int32_t (&b)[64])
 // commute (each exchanges one row-index bit with one column-index bit), and
 // after stage 16 the rows 16..31 hold only the high 16 bit-columns of the input,
 // so the top 16 planes can be finished without touching rows 0..15.
-template <int J, int R0, int R1>
+//
+// On the device every output word of a stage is one instruction after at most
+// one shift: a byte permute for J = 16 and 8, a three-input bitwise function for
+// J = 4, 2, 1.  They are written as builtins because the generic and/or/shift
+// form gets re-associated across stages into longer sequences.
+//
+// Negabinary (encode.cuh:203-212, shared.h:176-181) is u = (x + c) ^ c with
+// c = 0xaaaaaaaa.  The xor with c complements the odd bit planes, and J = 1 is
+// the stage that pairs plane 2j with plane 2j+1, so it can complement for free:
+// kNotOut complements the odd rows it writes (values -> planes, J = 1 last),
+// kNotIn complements the odd rows it reads (planes -> values, J = 1 first).
+enum { kPlain = 0, kNotOut = 1, kNotIn = 2 };
+
+CSWAP_HD uint32_t bit_select(uint32_t m, uint32_t a, uint32_t b)  // m ? a : b
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_bitop3_b32(m, a, b, 0xca);
+#else
+  return (a & m) | (b & ~m);
+#endif
+}
+CSWAP_HD uint32_t bit_select_nb(uint32_t m, uint32_t a, uint32_t b)  // m ? a : ~b
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_bitop3_b32(m, a, b, 0xc5);
+#else
+  return (a & m) | (~b & ~m);
+#endif
+}
+CSWAP_HD uint32_t bit_select_nn(uint32_t m, uint32_t a, uint32_t b)  // ~(m ? a : b)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_bitop3_b32(m, a, b, 0x35);
+#else
+  return ~((a & m) | (b & ~m));
+#endif
+}
+
+template <int J, int R0, int R1, int NB = kPlain>
 CSWAP_HD void tr_stage(uint32_t (&a)[32])
 {
+  static_assert(NB == kPlain || J == 1, "only the stage that pairs neighbouring planes can complement them");
   constexpr uint32_t m = J == 16 ? 0x0000ffffu : J == 8 ? 0x00ff00ffu : J == 4 ? 0x0f0f0f0fu
                          : J == 2 ? 0x33333333u : 0x55555555u;
 #pragma unroll
   for (int r = R0; r < R1; r++) {
     if (r & J) continue;
-    uint32_t lo = a[r], hi = a[r + J];
-    a[r] = (lo & m) | ((hi << J) & ~m);
-    a[r + J] = ((lo >> J) & m) | (hi & ~m);
+    const uint32_t lo = a[r], hi = a[r + J];
+#if defined(__HIP_DEVICE_COMPILE__)
+    if (J == 16) {  // bytes, low to high: lo0 lo1 hi0 hi1 / lo2 lo3 hi2 hi3
+      a[r] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+      a[r + J] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
+      continue;
+    }
+    if (J == 8) {  // lo0 hi0 lo2 hi2 / lo1 hi1 lo3 hi3
+      a[r] = __builtin_amdgcn_perm(hi, lo, 0x06020400u);
+      a[r + J] = __builtin_amdgcn_perm(hi, lo, 0x07030501u);
+      continue;
+    }
+#endif
+    if (NB == kNotIn) {  // hi is an odd plane: use its complement (the bit shifted in lands where m selects lo)
+      a[r] = bit_select_nb(m, lo, hi << J);
+      a[r + J] = bit_select_nb(m, lo >> J, hi);
+    } else if (NB == kNotOut) {  // a[r + J] is an odd plane: store its complement
+      a[r] = bit_select(m, lo, hi << J);
+      a[r + J] = bit_select_nn(m, lo >> J, hi);
+    } else {
+      a[r] = bit_select(m, lo, hi << J);
+      a[r + J] = bit_select(m, lo >> J, hi);
+    }
   }
 }
 
-// stages 8,4,2,1 on rows [R0, R0+16)
-template <int R0>
+// stages 8,4,2,1 on rows [R0, R0+16); with kNotIn the order is 1,2,4,8
+template <int R0, int NB = kPlain>
 CSWAP_HD void tr_half(uint32_t (&a)[32])
 {
-  tr_stage<8, R0, R0 + 16>(a);
-  tr_stage<4, R0, R0 + 16>(a);
-  tr_stage<2, R0, R0 + 16>(a);
-  tr_stage<1, R0, R0 + 16>(a);
+  if (NB == kNotIn) {
+    tr_stage<1, R0, R0 + 16, kNotIn>(a);
+    tr_stage<2, R0, R0 + 16>(a);
+    tr_stage<4, R0, R0 + 16>(a);
+    tr_stage<8, R0, R0 + 16>(a);
+  } else {
+    tr_stage<8, R0, R0 + 16>(a);
+    tr_stage<4, R0, R0 + 16>(a);
+    tr_stage<2, R0, R0 + 16>(a);
+    tr_stage<1, R0, R0 + 16, NB>(a);
+  }
 }
 
 CSWAP_HD void transpose32(uint32_t (&a)[32])
@@ -336,21 +412,21 @@ CSWAP_HD void encode_block(const float (&f)[64], unsigned pos0, unsigned maxbits
 
   uint32_t lo[32], hi[32];
 #pragma unroll
-  for (int i = 0; i < 32; i++) {
-    lo[i] = int2nb(ib[kPerm3.v[i]]);
-    hi[i] = int2nb(ib[kPerm3.v[32 + i]]);
+  for (int i = 0; i < 32; i++) {  // negabinary: the add here, the xor inside the transpose
+    lo[i] = (uint32_t)ib[kPerm3.v[i]] + kNegabinary;
+    hi[i] = (uint32_t)ib[kPerm3.v[32 + i]] + kNegabinary;
   }
   // top 16 planes first; the low 16 are only transposed if some block of the
   // wavefront still has bit budget left after them
   tr_stage<16, 0, 32>(lo);
   tr_stage<16, 0, 32>(hi);
-  tr_half<16>(lo);
-  tr_half<16>(hi);
+  tr_half<16, kNotOut>(lo);
+  tr_half<16, kNotOut>(hi);
 #pragma unroll
   for (int k = 31; k >= 16; k--) enc.plane(((uint64_t)hi[k] << 32) | lo[k]);
   if (CSWAP_ANY(enc.active())) {
-    tr_half<0>(lo);
-    tr_half<0>(hi);
+    tr_half<0, kNotOut>(lo);
+    tr_half<0, kNotOut>(hi);
 #pragma unroll
     for (int k = 15; k >= 0; k--) enc.plane(((uint64_t)hi[k] << 32) | lo[k]);
   }
@@ -377,23 +453,15 @@ struct BlockDecoder {
     return ((uint64_t)funnel_shr(w2, w1, p) << 32) | funnel_shr(w1, w0, p);
   }
 
-  // mirror of BlockEncoder::plane (decode.cuh:141-173)
+  // mirror of BlockEncoder::plane (decode.cuh:141-173).  Written without early
+  // exits: a block that is out of budget reads zero verbatim bits and never
+  // enters the step loop, and when every coefficient is already significant the
+  // plane is one 64-bit read.
   CSWAP_HD uint64_t plane()
   {
-    uint64_t x = 0;
-    if (!CSWAP_ANY(active() && n < SIZE)) {  // every block of the wavefront is past discovery
-      if (active()) {
-        unsigned left = limit - pos;
-        unsigned m = left < (unsigned)SIZE ? left : (unsigned)SIZE;
-        x = window(pos) & low_mask(m);
-        pos += m;
-      }
-      return x;
-    }
-    if (!active()) return x;
-    unsigned left = limit - pos;
+    unsigned left = sub_sat(limit, pos);
     unsigned m = n < left ? n : left;
-    x = window(pos) & low_mask(m);
+    uint64_t x = window(pos) & low_mask(m);
     pos += m;
     while (n < SIZE && pos < limit) {
       uint64_t w = window(pos);
@@ -436,8 +504,12 @@ CSWAP_HD void decode_block(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)
     lo[k] = (uint32_t)x;
     hi[k] = (uint32_t)(x >> 32);
   }
-  tr_half<16>(lo);
-  tr_half<16>(hi);
+  tr_half<16, kNotIn>(lo);
+  tr_half<16, kNotIn>(hi);
+  // negabinary: the xor inside the transpose, the subtraction here.  When the low
+  // 16 planes are all zero they are not transposed, so their complemented odd
+  // planes (0xaaaa in every value) are missing from the minuend as well.
+  uint32_t c = kNegabinary;
   if (CSWAP_ANY(dec.active())) {
 #pragma unroll
     for (int k = 15; k >= 0; k--) {
@@ -445,11 +517,12 @@ CSWAP_HD void decode_block(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)
       lo[k] = (uint32_t)x;
       hi[k] = (uint32_t)(x >> 32);
     }
-    tr_half<0>(lo);
-    tr_half<0>(hi);
+    tr_half<0, kNotIn>(lo);
+    tr_half<0, kNotIn>(hi);
   } else {
 #pragma unroll
-    for (int k = 0; k < 16; k++) lo[k] = hi[k] = 0;  // transposing zeros gives zeros
+    for (int k = 0; k < 16; k++) lo[k] = hi[k] = 0;
+    c = kNegabinary & 0xffff0000u;
   }
   tr_stage<16, 0, 32>(lo);
   tr_stage<16, 0, 32>(hi);
@@ -457,8 +530,8 @@ CSWAP_HD void decode_block(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)
   int32_t ib[64];
 #pragma unroll
   for (int i = 0; i < 32; i++) {
-    ib[kPerm3.v[i]] = nb2int(lo[i]);
-    ib[kPerm3.v[32 + i]] = nb2int(hi[i]);
+    ib[kPerm3.v[i]] = (int32_t)(lo[i] - c);
+    ib[kPerm3.v[32 + i]] = (int32_t)(hi[i] - c);
   }
   inv_xform3(ib);
 
