@@ -81,6 +81,24 @@ CSWAP_HD uint64_t low_mask(unsigned n)  // n in 0..64
   return n >= 64 ? ~(uint64_t)0 : (((uint64_t)1 << n) - 1);
 }
 
+// Division of a 31-bit number by a fixed divisor d >= 1 as a multiply and a
+// shift: with l = ceil(log2 d) and mul = ceil(2^(31+l) / d) (which fits 32 bits),
+// floor(b / d) = (b * mul) >> (31 + l) for every b < 2^31 (Granlund & Montgomery,
+// "Division by invariant integers using multiplication", theorem 4.2 with N = 31).
+struct Div31 {
+  uint32_t mul, shift;  // shift = 31 + l
+};
+inline Div31 make_div31(uint32_t d)
+{
+  uint32_t l = 0;
+  while (((uint64_t)1 << l) < d) l++;
+  Div31 r;
+  r.mul = (uint32_t)((((uint64_t)1 << (31 + l)) + d - 1) / d);
+  r.shift = 31 + l;
+  return r;
+}
+CSWAP_HD uint32_t div31(uint32_t b, Div31 d) { return (uint32_t)(((uint64_t)b * d.mul) >> d.shift); }
+
 CSWAP_HD unsigned sub_sat(unsigned a, unsigned b)  // max(a - b, 0)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -436,7 +454,10 @@ CSWAP_HD void encode_block(const float (&f)[64], unsigned pos0, unsigned maxbits
 // mem.ld32(dword_index) reads the bit region; positions are absolute within it
 // and the block owns [pos0, pos0 + maxbits).  Reads may run up to 96 bits past
 // the end of the block (the values are never used).
-template <class Mem, int SIZE = 64>
+// FENCED: the caller guarantees that the bit right after the block reads as one.
+// A run of zeros that the bit budget cuts short then ends at that bit by itself,
+// and the step loop does not have to clamp the run to the bits that are left.
+template <class Mem, int SIZE = 64, bool FENCED = false>
 struct BlockDecoder {
   Mem& mem;
   unsigned pos, limit;
@@ -469,12 +490,15 @@ struct BlockDecoder {
       pos++;
       if (!(w & 1)) break;  // negative group test: plane done
       w >>= 1;              // 63 valid bits
-      unsigned avail = limit - pos;
-      unsigned maxrun = SIZE - 1 - n < avail ? SIZE - 1 - n : avail;
+      unsigned maxrun = SIZE - 1 - n;
+      if (!FENCED) {
+        unsigned avail = limit - pos;
+        maxrun = maxrun < avail ? maxrun : avail;
+      }
       unsigned t = (unsigned)ctz64(w);
       bool found = t < maxrun;  // t zeros then a one; else ran into position 63 or the budget
       unsigned r = found ? t : maxrun;
-      pos += r + (found ? 1u : 0u);
+      pos += r + (found ? 1u : 0u);  // FENCED and out of budget: "finds" the fence, pos = limit + 1
       n += r;
       x |= (uint64_t)1 << n;
       n++;
@@ -484,10 +508,10 @@ struct BlockDecoder {
 };
 
 // Full block decode into f[x + 4y + 16z]; an empty block gives +0.0 everywhere.
-template <class Mem>
+template <bool FENCED = false, class Mem>
 CSWAP_HD void decode_block(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)[64])
 {
-  BlockDecoder<Mem> dec(mem, pos0, maxbits);
+  BlockDecoder<Mem, 64, FENCED> dec(mem, pos0, maxbits);
   uint32_t h = (uint32_t)dec.window(pos0);
   if (!(h & 1)) {
 #pragma unroll

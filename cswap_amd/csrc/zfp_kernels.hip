@@ -22,8 +22,10 @@ struct Field3 {
   uint32_t mx, my;         // blocks along x and y
   uint32_t nblocks;
   long long sx, sy, sz;    // strides in elements
-  int rows16;              // 1: x-rows of every block are contiguous, 16-byte aligned
+  int rows16;              // 1: x-rows of every block are contiguous and 16-byte aligned, rows nest inside
+                           //    planes inside the volume, and any 64 consecutive blocks lie within 4 GiB
   int stream16;            // 1: the stream pointer is 16-byte aligned
+  Div31 by_mx, by_my;      // block index -> block coordinates without a hardware divide
 };
 
 // ------------------------------------------------------------- LDS adapter
@@ -58,32 +60,57 @@ __host__ __device__ inline unsigned region_dwords(unsigned maxbits)
 __device__ __forceinline__ void block_origin(const Field3& fd, uint32_t b, uint32_t& x0, uint32_t& y0,
                                              uint32_t& z0)
 {
-  uint32_t q = b / fd.mx;
+  uint32_t q = div31(b, fd.by_mx);
   x0 = (b - q * fd.mx) * 4;
-  uint32_t r = q / fd.my;
+  uint32_t r = div31(q, fd.by_my);
   y0 = (q - r * fd.my) * 4;
   z0 = r * 4;
 }
 
-__device__ __forceinline__ void load_block(const float* __restrict__ in, const Field3& fd, uint32_t b,
-                                           float (&f)[64])
+// Addressing of the fast path (Field3::rows16): the wavefront's first block gives
+// a wave-uniform 64-bit base, every lane adds a 32-bit byte offset to it.  Block
+// order is x, then y, then z and the strides nest, so offsets grow with the block
+// index; the host only sets rows16 when 64 consecutive blocks span less than 4 GiB.
+struct WaveBase {
+  long long origin;  // element offset of the first block's corner
+  uint32_t fx, fy, fz;
+};
+__device__ __forceinline__ WaveBase wave_base(const Field3& fd, uint32_t first)
+{
+  WaveBase w;
+  block_origin(fd, first, w.fx, w.fy, w.fz);
+  w.origin = (long long)w.fx + (long long)w.fy * fd.sy + (long long)w.fz * fd.sz;
+  return w;
+}
+__device__ __forceinline__ uint32_t lane_bytes(const Field3& fd, const WaveBase& w, uint32_t x0, uint32_t y0,
+                                               uint32_t z0)
+{
+  return ((x0 - w.fx) + (y0 - w.fy) * (uint32_t)fd.sy + (z0 - w.fz) * (uint32_t)fd.sz) * 4u;  // mod 2^32
+}
+
+__device__ __forceinline__ void load_block(const float* __restrict__ in, const Field3& fd, uint32_t first,
+                                           uint32_t b, float (&f)[64])
 {
   uint32_t x0, y0, z0;
   block_origin(fd, b, x0, y0, z0);
-  const float* p = in + (long long)x0 * fd.sx + (long long)y0 * fd.sy + (long long)z0 * fd.sz;
   uint32_t bx = min(4u, fd.nx - x0), by = min(4u, fd.ny - y0), bz = min(4u, fd.nz - z0);
   if (fd.rows16 && bx == 4 && by == 4 && bz == 4) {
+    const WaveBase w = wave_base(fd, first);
+    const char* base = reinterpret_cast<const char*>(in + w.origin);
+    const uint32_t mine = lane_bytes(fd, w, x0, y0, z0);
+    const uint32_t sy4 = (uint32_t)fd.sy * 4u, sz4 = (uint32_t)fd.sz * 4u;
 #pragma unroll
     for (int z = 0; z < 4; z++)
 #pragma unroll
       for (int y = 0; y < 4; y++) {
-        float4 v = *reinterpret_cast<const float4*>(p + y * fd.sy + z * fd.sz);
+        float4 v = *reinterpret_cast<const float4*>(base + (size_t)(mine + (y * sy4 + z * sz4)));
         f[16 * z + 4 * y + 0] = v.x;
         f[16 * z + 4 * y + 1] = v.y;
         f[16 * z + 4 * y + 2] = v.z;
         f[16 * z + 4 * y + 3] = v.w;
       }
   } else {
+    const float* p = in + (long long)x0 * fd.sx + (long long)y0 * fd.sy + (long long)z0 * fd.sz;
 #pragma unroll
     for (int z = 0; z < 4; z++)
 #pragma unroll
@@ -97,23 +124,27 @@ __device__ __forceinline__ void load_block(const float* __restrict__ in, const F
   }
 }
 
-__device__ __forceinline__ void store_block(float* __restrict__ out, const Field3& fd, uint32_t b,
-                                            const float (&f)[64])
+__device__ __forceinline__ void store_block(float* __restrict__ out, const Field3& fd, uint32_t first,
+                                            uint32_t b, const float (&f)[64])
 {
   uint32_t x0, y0, z0;
   block_origin(fd, b, x0, y0, z0);
-  float* p = out + (long long)x0 * fd.sx + (long long)y0 * fd.sy + (long long)z0 * fd.sz;
   uint32_t bx = min(4u, fd.nx - x0), by = min(4u, fd.ny - y0), bz = min(4u, fd.nz - z0);
   if (fd.rows16 && bx == 4 && by == 4 && bz == 4) {
+    const WaveBase w = wave_base(fd, first);
+    char* base = reinterpret_cast<char*>(out + w.origin);
+    const uint32_t mine = lane_bytes(fd, w, x0, y0, z0);
+    const uint32_t sy4 = (uint32_t)fd.sy * 4u, sz4 = (uint32_t)fd.sz * 4u;
 #pragma unroll
     for (int z = 0; z < 4; z++)
 #pragma unroll
       for (int y = 0; y < 4; y++) {
         float4 v = make_float4(f[16 * z + 4 * y], f[16 * z + 4 * y + 1], f[16 * z + 4 * y + 2],
                                f[16 * z + 4 * y + 3]);
-        *reinterpret_cast<float4*>(p + y * fd.sy + z * fd.sz) = v;
+        *reinterpret_cast<float4*>(base + (size_t)(mine + (y * sy4 + z * sz4))) = v;
       }
   } else {
+    float* p = out + (long long)x0 * fd.sx + (long long)y0 * fd.sy + (long long)z0 * fd.sz;
 #pragma unroll
     for (int z = 0; z < 4; z++)
 #pragma unroll
@@ -149,7 +180,7 @@ __global__ __launch_bounds__(64) void zfp_encode3_f32_kernel(const float* __rest
 
   if (lane < valid) {
     float f[64];
-    load_block(in, fd, first + lane, f);
+    load_block(in, fd, first, first + lane, f);
     LdsBits mem{lds};
     encode_block<!WHOLE>(f, lane * slot, maxbits, mem);
   }
@@ -198,6 +229,7 @@ __global__ __launch_bounds__(64) void zfp_decode3_f32_kernel(const uint64_t* __r
       } else {
         for (unsigned j = 0; j < W; j++) dst[j] = src[j];
       }
+      dst[W] = ~0ull;  // the fence the decoder relies on: ones right after the block
     }
   } else {
     const unsigned nwords = (valid * maxbits + 63u) >> 6;
@@ -210,8 +242,8 @@ __global__ __launch_bounds__(64) void zfp_decode3_f32_kernel(const uint64_t* __r
   if (lane < valid) {
     float f[64];
     LdsBits mem{lds};
-    decode_block(mem, lane * slot, maxbits, f);
-    store_block(out, fd, first + lane, f);
+    decode_block<WHOLE>(mem, lane * slot, maxbits, f);
+    store_block(out, fd, first, first + lane, f);
   }
 }
 
@@ -338,14 +370,23 @@ static int make_field(Field3& fd, const void* base, const void* stream, size_t n
   if (nx > 0x7fffffffu || ny > 0x7fffffffu || nz > 0x7fffffffu) return CSWAP_E_ARG;
   size_t mx = (nx + 3) / 4, my = (ny + 3) / 4, mz = (nz + 3) / 4;
   size_t nb = mx * my * mz;
-  if (nb / mz != mx * my || nb > 0xfffffff0ull) return CSWAP_E_ARG;
+  if (nb / mz != mx * my || nb > 0x7fffffffull) return CSWAP_E_ARG;  // block indices stay below 2^31
   fd.nx = (uint32_t)nx; fd.ny = (uint32_t)ny; fd.nz = (uint32_t)nz;
   fd.mx = (uint32_t)mx; fd.my = (uint32_t)my;
   fd.nblocks = (uint32_t)nb;
   fd.sx = sx ? sx : 1;
   fd.sy = sy ? sy : (ptrdiff_t)nx;
   fd.sz = sz ? sz : (ptrdiff_t)(nx * ny);
-  fd.rows16 = fd.sx == 1 && (fd.sy % 4) == 0 && (fd.sz % 4) == 0 && ((uintptr_t)base % 16) == 0;
+  fd.by_mx = make_div31(fd.mx);
+  fd.by_my = make_div31(fd.my);
+  // fast path: aligned contiguous rows; rows inside planes inside the volume (so
+  // element offsets grow with the block index); and the slabs of four planes that
+  // 64 consecutive blocks can touch (one more than they fill) stay below 4 GiB, so
+  // every block of a wavefront is within a 32-bit byte offset of its first block
+  const size_t slabs = (64 + mx * my - 1) / (mx * my) + 1;
+  fd.rows16 = fd.sx == 1 && (fd.sy % 4) == 0 && (fd.sz % 4) == 0 && ((uintptr_t)base % 16) == 0 &&
+              fd.sy >= (ptrdiff_t)nx && fd.sz >= fd.sy * (ptrdiff_t)ny &&
+              (unsigned long long)fd.sz * 16ull * slabs < 0xfff00000ull;
   fd.stream16 = ((uintptr_t)stream % 16) == 0;
   return CSWAP_OK;
 }

@@ -47,6 +47,27 @@ void host_zfp_decode3(const uint64_t* stream, size_t nx, size_t ny, size_t nz, u
   }
 }
 
+// Same decode through the fenced variant: every block is copied into a private
+// slot that is followed by one bits, as the device does for whole-word rates.
+void host_zfp_decode3_fenced(const uint64_t* stream, size_t nx, size_t ny, size_t nz, unsigned maxbits, float* out)
+{
+  size_t mx = (nx + 3) / 4, my = (ny + 3) / 4, mz = (nz + 3) / 4;
+  const unsigned W = maxbits / 64;  // maxbits % 64 == 0
+  uint32_t* slot = new uint32_t[2 * W + 8];
+  for (size_t b = 0; b < mx * my * mz; b++) {
+    size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
+    unsigned bx = nx - x0 < 4 ? nx - x0 : 4, by = ny - y0 < 4 ? ny - y0 : 4, bz = nz - z0 < 4 ? nz - z0 : 4;
+    memcpy(slot, stream + b * W, 8 * (size_t)W);
+    memset(slot + 2 * W, 0xff, 32);
+    float f[64];
+    ArrayBits mem{slot};
+    cswap::decode_block<true>(mem, 0u, maxbits, f);
+    for (unsigned z = 0; z < bz; z++) for (unsigned y = 0; y < by; y++) for (unsigned x = 0; x < bx; x++)
+      out[(x0 + x) + nx * ((y0 + y) + ny * (z0 + z))] = f[x + 4 * y + 16 * z];
+  }
+  delete[] slot;
+}
+
 // 2-D field a[ny][nx] (ny = 0: 1-D field a[nx])
 void host_zfp_encode_low(const float* in, size_t nx, size_t ny, unsigned maxbits, uint64_t* stream)
 {
@@ -81,6 +102,7 @@ void host_zfp_decode_low(const uint64_t* stream, size_t nx, size_t ny, unsigned 
   }
 }
 
+uint32_t host_div31(uint32_t b, uint32_t d) { return cswap::div31(b, cswap::make_div31(d)); }
 void host_transpose32(uint32_t* a) { uint32_t t[32]; memcpy(t, a, sizeof t); cswap::transpose32(t); memcpy(a, t, sizeof t); }
 
 }

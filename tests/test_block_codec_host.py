@@ -22,10 +22,30 @@ def host():
     L = C.CDLL(SO)
     L.host_zfp_encode3.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     L.host_zfp_decode3.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
+    L.host_zfp_decode3_fenced.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     L.host_transpose32.argtypes = [C.c_void_p]
     L.host_zfp_encode_low.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     L.host_zfp_decode_low.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     return L
+
+
+def test_multiply_shift_division_matches_integer_division(host):
+    """Block coordinates come from floor(b / d) computed as (b * mul) >> shift;
+    exact for every b < 2^31, checked at the edges of each quotient step."""
+    host.host_div31.restype = C.c_uint32
+    host.host_div31.argtypes = [C.c_uint32, C.c_uint32]
+    rng = np.random.default_rng(7)
+    divisors = [1, 2, 3, 5, 7, 8, 9, 127, 128, 129, 1000, 65535, 65536, 65537, 2**24 + 1, 2**31 - 1, 2**31,
+                2**32 - 1] + [int(v) for v in rng.integers(1, 2**31, 40)]
+    for d in divisors:
+        bs = {0, 1, d - 1, d, d + 1, 2**31 - 1, 2**31 - 2}
+        top = (2**31 - 1) // d
+        for q in {1, 2, top // 2, top - 1, top} | {int(v) for v in rng.integers(0, top + 1, 20)}:
+            bs |= {q * d - 1, q * d, q * d + d - 1}
+        bs |= {int(v) for v in rng.integers(0, 2**31, 50)}
+        for b in bs:
+            if 0 <= b < 2**31:
+                assert host.host_div31(b, d) == b // d, (b, d)
 
 
 def test_transpose32_is_a_bit_matrix_transpose(host):
@@ -54,6 +74,10 @@ def test_block_codec_matches_golden_vectors(host, golden):
         o = np.zeros_like(f)
         host.host_zfp_decode3(g.ctypes.data, nx, ny, nz, maxbits, o.ctypes.data)
         assert np.array_equal(o.view(np.uint32), dec.view(np.uint32)), (name, rate)
+        if maxbits % 64 == 0:  # the variant the device uses for whole-word rates
+            o2 = np.zeros_like(f)
+            host.host_zfp_decode3_fenced(g.ctypes.data, nx, ny, nz, maxbits, o2.ctypes.data)
+            assert np.array_equal(o2.view(np.uint32), dec.view(np.uint32)), (name, rate, "fenced")
         n += 1
     assert n >= 100
 
