@@ -523,8 +523,8 @@ CSWAP_HD void decode_block(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)
 
   uint32_t lo[32], hi[32];
 #pragma unroll
-  for (int k = 31; k >= 16; k--) {
-    uint64_t x = dec.plane();
+  for (int k = 31; k >= 16; k--) {  // planes that no block of the wavefront can reach are zero without a read
+    uint64_t x = CSWAP_ANY(dec.active()) ? dec.plane() : 0;
     lo[k] = (uint32_t)x;
     hi[k] = (uint32_t)(x >> 32);
   }
