@@ -175,7 +175,7 @@ CSWAP_HD void fwd_xform3(int32_t (&b)[64])
   for (int i = 0; i < 16; i++) fwd_lift4(b[i], b[i + 16], b[i + 32], b[i + 48]);
 }
 
-CSWAP_HD void inv_xform3(int32_t (&b)[64])
+CSWAP_HD void inv_xform3_zy(int32_t (&b)[64])  // the z and y passes; the x pass is one inv_lift4 per row
 {
 #pragma unroll
   for (int i = 0; i < 16; i++) inv_lift4(b[i], b[i + 16], b[i + 32], b[i + 48]);
@@ -184,6 +184,11 @@ CSWAP_HD void inv_xform3(int32_t (&b)[64])
 #pragma unroll
     for (int x = 0; x < 4; x++)
       inv_lift4(b[16 * z + x], b[16 * z + x + 4], b[16 * z + x + 8], b[16 * z + x + 12]);
+}
+
+CSWAP_HD void inv_xform3(int32_t (&b)[64])
+{
+  inv_xform3_zy(b);
 #pragma unroll
   for (int i = 0; i < 16; i++) inv_lift4(b[4 * i], b[4 * i + 1], b[4 * i + 2], b[4 * i + 3]);
 }
@@ -507,15 +512,21 @@ struct BlockDecoder {
   }
 };
 
-// Full block decode into f[x + 4y + 16z]; an empty block gives +0.0 everywhere.
+// Block decode in two parts, so that a caller can finish, convert and store one
+// x-row at a time instead of holding 64 finished values:
+//   decode_block_zy  everything up to and including the inverse lifting along z
+//                    and y; leaves ib[x + 4y + 16z] and the scale w
+//   decode_row       inverse lifting along x of one row and the cast to float
+// An empty block gives ib = 0 and w = 0, i.e. +0.0 everywhere.
 template <bool FENCED = false, class Mem>
-CSWAP_HD void decode_block(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)[64])
+CSWAP_HD void decode_block_zy(Mem& mem, unsigned pos0, unsigned maxbits, int32_t (&ib)[64], float& w)
 {
   BlockDecoder<Mem, 64, FENCED> dec(mem, pos0, maxbits);
   uint32_t h = (uint32_t)dec.window(pos0);
   if (!(h & 1)) {
 #pragma unroll
-    for (int i = 0; i < 64; i++) f[i] = 0.0f;
+    for (int i = 0; i < 64; i++) ib[i] = 0;
+    w = 0.0f;
     return;
   }
   int emax = (int)((h >> 1) & 0xff) - 127;
@@ -551,17 +562,37 @@ CSWAP_HD void decode_block(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)
   tr_stage<16, 0, 32>(lo);
   tr_stage<16, 0, 32>(hi);
 
-  int32_t ib[64];
 #pragma unroll
   for (int i = 0; i < 32; i++) {
     ib[kPerm3.v[i]] = (int32_t)(lo[i] - c);
     ib[kPerm3.v[32 + i]] = (int32_t)(hi[i] - c);
   }
-  inv_xform3(ib);
+  inv_xform3_zy(ib);
+  w = pow2f(emax - 30);
+}
 
-  float w = pow2f(emax - 30);
+// row = y + 4z; f receives the four values of that x-row
+CSWAP_HD void decode_row(int32_t (&ib)[64], int row, float w, float (&f)[4])
+{
+  inv_lift4(ib[4 * row], ib[4 * row + 1], ib[4 * row + 2], ib[4 * row + 3]);
 #pragma unroll
-  for (int i = 0; i < 64; i++) f[i] = w * (float)ib[i];
+  for (int x = 0; x < 4; x++) f[x] = w * (float)ib[4 * row + x];
+}
+
+// Full block decode into f[x + 4y + 16z]
+template <bool FENCED = false, class Mem>
+CSWAP_HD void decode_block(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)[64])
+{
+  int32_t ib[64];
+  float w;
+  decode_block_zy<FENCED>(mem, pos0, maxbits, ib, w);
+#pragma unroll
+  for (int row = 0; row < 16; row++) {
+    float r[4];
+    decode_row(ib, row, w, r);
+#pragma unroll
+    for (int x = 0; x < 4; x++) f[4 * row + x] = r[x];
+  }
 }
 
 // ---------------------------------------------------------------- 2-D and 1-D blocks

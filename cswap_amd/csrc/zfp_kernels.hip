@@ -124,35 +124,40 @@ __device__ __forceinline__ void load_block(const float* __restrict__ in, const F
   }
 }
 
-__device__ __forceinline__ void store_block(float* __restrict__ out, const Field3& fd, uint32_t first,
-                                            uint32_t b, const float (&f)[64])
+// Finishes the block (inverse lifting along x, cast) and stores it.  On the
+// fast path every x-row is finished and stored on its own, so the finished
+// values never all sit in registers at once.
+__device__ __forceinline__ void finish_and_store_block(float* __restrict__ out, const Field3& fd, uint32_t first,
+                                                       uint32_t b, int32_t (&ib)[64], float w)
 {
   uint32_t x0, y0, z0;
   block_origin(fd, b, x0, y0, z0);
   uint32_t bx = min(4u, fd.nx - x0), by = min(4u, fd.ny - y0), bz = min(4u, fd.nz - z0);
   if (fd.rows16 && bx == 4 && by == 4 && bz == 4) {
-    const WaveBase w = wave_base(fd, first);
-    char* base = reinterpret_cast<char*>(out + w.origin);
-    const uint32_t mine = lane_bytes(fd, w, x0, y0, z0);
+    const WaveBase wb = wave_base(fd, first);
+    char* base = reinterpret_cast<char*>(out + wb.origin);
+    const uint32_t mine = lane_bytes(fd, wb, x0, y0, z0);
     const uint32_t sy4 = (uint32_t)fd.sy * 4u, sz4 = (uint32_t)fd.sz * 4u;
 #pragma unroll
     for (int z = 0; z < 4; z++)
 #pragma unroll
       for (int y = 0; y < 4; y++) {
-        float4 v = make_float4(f[16 * z + 4 * y], f[16 * z + 4 * y + 1], f[16 * z + 4 * y + 2],
-                               f[16 * z + 4 * y + 3]);
-        *reinterpret_cast<float4*>(base + (size_t)(mine + (y * sy4 + z * sz4))) = v;
+        float r[4];
+        decode_row(ib, y + 4 * z, w, r);
+        *reinterpret_cast<float4*>(base + (size_t)(mine + (y * sy4 + z * sz4))) = make_float4(r[0], r[1], r[2], r[3]);
       }
   } else {
     float* p = out + (long long)x0 * fd.sx + (long long)y0 * fd.sy + (long long)z0 * fd.sz;
 #pragma unroll
     for (int z = 0; z < 4; z++)
 #pragma unroll
-      for (int y = 0; y < 4; y++)
+      for (int y = 0; y < 4; y++) {
+        float r[4];
+        decode_row(ib, y + 4 * z, w, r);
 #pragma unroll
         for (int x = 0; x < 4; x++)
-          if ((uint32_t)x < bx && (uint32_t)y < by && (uint32_t)z < bz)
-            p[x * fd.sx + y * fd.sy + z * fd.sz] = f[16 * z + 4 * y + x];
+          if ((uint32_t)x < bx && (uint32_t)y < by && (uint32_t)z < bz) p[x * fd.sx + y * fd.sy + z * fd.sz] = r[x];
+      }
   }
 }
 
@@ -243,10 +248,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void
   __syncthreads();
 
   if (lane < valid) {
-    float f[64];
+    int32_t ib[64];
+    float w;
     LdsBits mem{lds};
-    decode_block<WHOLE>(mem, lane * slot, maxbits, f);
-    store_block(out, fd, first, first + lane, f);
+    decode_block_zy<WHOLE>(mem, lane * slot, maxbits, ib, w);
+    // block coordinates and addresses are worked out only now, from a lane id
+    // that is recomputed here and tied to a decoded value: otherwise they (or
+    // the thread index they come from) are held in registers through the whole
+    // decode, or spilled
+    uint32_t zero = 0;
+    asm volatile("" : "+v"(zero) : "v"(ib[0]));
+    const uint32_t b = first + __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));  // lane id again
+    finish_and_store_block(out, fd, first, b, ib, w);
   }
 }
 
