@@ -279,6 +279,7 @@ def extras(torch, api, dev):
     try:
         from cswap_amd import swap
         ex["swap"] = swap.bench_schedule(dev)
+        ex["swap_backward"] = swap.bench_backward(dev)
     except ImportError:
         pass
     return ex

@@ -100,6 +100,7 @@ _SIGNATURES = {
     "cswap_swap_out": (i32, [vp, vp, sz, sz, sz, i32, vp, C.POINTER(i32)]),
     "cswap_swap_wait": (i32, [vp, i32]),
     "cswap_swap_in": (i32, [vp, i32, vp, vp]),
+    "cswap_swap_prefetch": (i32, [vp, i32]),
     "cswap_swap_release": (i32, [vp, i32]),
     "cswap_swap_info": (i32, [vp, i32, C.POINTER(TicketInfo)]),
     "cswap_engine_calibrate": (i32, [vp, C.POINTER(Costs)]),

@@ -86,7 +86,7 @@ class Pool {
   size_t size_ = 0;
 };
 
-enum TicketState { kFree = 0, kOutInFlight = 1, kOnHost = 2, kInInFlight = 3 };
+enum TicketState { kFree = 0, kOutInFlight = 1, kOnHost = 2, kInInFlight = 3, kPrefetched = 4 };
 
 struct Ticket {
   int state = kFree;
@@ -364,6 +364,42 @@ extern "C" int cswap_swap_wait(cswap_engine* e, int ticket)
   return CSWAP_OK;
 }
 
+// Finish an outbound copy that is still in flight (swap-in or prefetch right after swap-out).
+static int settle_outbound(cswap_engine* e, Ticket& t)
+{
+  if (t.state != kOutInFlight) return CSWAP_OK;
+  CSWAP_HIP_TRY(hipEventSynchronize(t.ev_copy));
+  drop_device(e, t);
+  t.state = kOnHost;
+  return CSWAP_OK;
+}
+
+extern "C" int cswap_swap_prefetch(cswap_engine* e, int ticket)
+{
+  if (!e) return CSWAP_E_ARG;
+  std::lock_guard<std::mutex> lock(e->mu);
+  Ticket* t = get_ticket(e, ticket);
+  if (!t) return CSWAP_E_ARG;
+  if (t->state == kPrefetched) return CSWAP_OK;
+  int rc = settle_outbound(e, *t);
+  if (rc) return rc;
+  if (t->state != kOnHost) return CSWAP_E_STATE;
+  size_t off;
+  if (!e->dpool.alloc(t->bytes_out, &off)) return CSWAP_E_NOMEM;
+  t->dev_off = off; t->dev_bytes = t->bytes_out; t->dev_held = true;
+  // the staging region was released only after the events of its last user were waited for,
+  // so the copy stream has nothing to order against
+  hipError_t err = hipMemcpyAsync(e->d_base + off, e->h_base + t->host_off, t->bytes_out, hipMemcpyHostToDevice, e->copy);
+  if (err == hipSuccess) err = hipEventRecord(t->ev_copy, e->copy);
+  if (err != hipSuccess) {
+    (void)hipStreamSynchronize(e->copy);
+    drop_device(e, *t);
+    return hip_fail(err);
+  }
+  t->state = kPrefetched;
+  return CSWAP_OK;
+}
+
 extern "C" int cswap_swap_in(cswap_engine* e, int ticket, float* d_out, cswap_stream_t compute_)
 {
   if (!e || !d_out) return CSWAP_E_ARG;
@@ -371,39 +407,46 @@ extern "C" int cswap_swap_in(cswap_engine* e, int ticket, float* d_out, cswap_st
   std::lock_guard<std::mutex> lock(e->mu);
   Ticket* t = get_ticket(e, ticket);
   if (!t) return CSWAP_E_ARG;
-  if (t->state == kOutInFlight) {  // swap-in right after swap-out: finish the outbound copy first
-    CSWAP_HIP_TRY(hipEventSynchronize(t->ev_copy));
-    drop_device(e, *t);
-    t->state = kOnHost;
-  }
-  if (t->state != kOnHost) return CSWAP_E_STATE;
+  int rc = settle_outbound(e, *t);
+  if (rc) return rc;
+  if (t->state != kOnHost && t->state != kPrefetched) return CSWAP_E_STATE;
 
-  void* dst = d_out;
-  if (t->policy != CSWAP_POLICY_NONE) {
-    size_t off;
-    if (!e->dpool.alloc(t->bytes_out, &off)) return CSWAP_E_NOMEM;
-    t->dev_off = off; t->dev_bytes = t->bytes_out; t->dev_held = true;
-    dst = e->d_base + off;
+  hipError_t err = hipSuccess;
+  void* src = nullptr;  // device address of the payload once ev_copy has fired
+  if (t->state == kPrefetched) {
+    src = e->d_base + t->dev_off;
+    err = hipStreamWaitEvent(compute, t->ev_copy, 0);
+    if (err == hipSuccess && t->policy == CSWAP_POLICY_NONE)
+      err = hipMemcpyAsync(d_out, src, t->bytes_out, hipMemcpyDeviceToDevice, compute);
+  } else {
+    src = d_out;
+    if (t->policy != CSWAP_POLICY_NONE) {
+      size_t off;
+      if (!e->dpool.alloc(t->bytes_out, &off)) return CSWAP_E_NOMEM;
+      t->dev_off = off; t->dev_bytes = t->bytes_out; t->dev_held = true;
+      src = e->d_base + off;
+    }
+    // the copy may not overtake earlier work of the compute stream on d_out
+    err = hipEventRecord(t->ev_ready, compute);
+    if (err == hipSuccess) err = hipStreamWaitEvent(e->copy, t->ev_ready, 0);
+    if (err == hipSuccess) err = hipMemcpyAsync(src, e->h_base + t->host_off, t->bytes_out, hipMemcpyHostToDevice, e->copy);
+    if (err == hipSuccess) err = hipEventRecord(t->ev_copy, e->copy);
+    if (err == hipSuccess) err = hipStreamWaitEvent(compute, t->ev_copy, 0);
   }
-  // the copy may not overtake earlier work of the compute stream on d_out
-  hipError_t err = hipEventRecord(t->ev_ready, compute);
-  if (err == hipSuccess) err = hipStreamWaitEvent(e->copy, t->ev_ready, 0);
-  if (err == hipSuccess) err = hipMemcpyAsync(dst, e->h_base + t->host_off, t->bytes_out, hipMemcpyHostToDevice, e->copy);
-  if (err == hipSuccess) err = hipEventRecord(t->ev_copy, e->copy);
-  if (err == hipSuccess) err = hipStreamWaitEvent(compute, t->ev_copy, 0);
   if (err != hipSuccess) {
     (void)hipStreamSynchronize(e->copy);
+    (void)hipStreamSynchronize(compute);
     drop_device(e, *t);
+    t->state = kOnHost;
     return hip_fail(err);
   }
-  int rc = CSWAP_OK;
   if (t->policy == CSWAP_POLICY_SPARSE) {
     const size_t hdr = zvc_header_bytes((int)t->n, e->process);
-    char* base = (char*)dst;
+    char* base = (char*)src;
     rc = cswap_zvc_expand((const float*)(base + hdr), (const uint32_t*)(base + 4 * (size_t)e->process),
                           (const int*)base, (int)t->n, e->process, d_out, compute);
   } else if (t->policy == CSWAP_POLICY_ZFP) {
-    rc = cswap_zfp_decompress_f32((const uint64_t*)dst, t->nx, t->ny, t->nz, 0, 0, 0, e->maxbits, d_out, compute);
+    rc = cswap_zfp_decompress_f32((const uint64_t*)src, t->nx, t->ny, t->nz, 0, 0, 0, e->maxbits, d_out, compute);
   }
   err = hipEventRecord(t->ev_done, compute);
   t->state = kInInFlight;
@@ -420,7 +463,7 @@ extern "C" int cswap_swap_release(cswap_engine* e, int ticket)
   if (!t) return CSWAP_E_ARG;
   if (t->state == kFree) return CSWAP_E_STATE;
   hipError_t err = hipSuccess;
-  if (t->state == kOutInFlight) err = hipEventSynchronize(t->ev_copy);
+  if (t->state == kOutInFlight || t->state == kPrefetched) err = hipEventSynchronize(t->ev_copy);
   if (t->state == kInInFlight) err = hipEventSynchronize(t->ev_done);
   drop_device(e, *t);
   e->hpool.free(t->host_off, t->host_bytes);

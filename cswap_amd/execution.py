@@ -23,7 +23,7 @@ class Execution:
         self.policy: list[int] = []
         self.begin_stage: list[int] = []
         self._tickets: dict[int, tuple[int, tuple]] = {}
-        self._pending = -1
+        self._pending: list[int] = []
 
     def init_(self, n: int) -> None:
         self.policy = [0] * n
@@ -38,24 +38,30 @@ class Execution:
     def postforward(self) -> None:
         pass
 
-    def pre(self, tensor: torch.Tensor, tensor_id: int, layer_type: int = ACT) -> None:
+    def pre(self, tensor, tensor_id=None, layer_type: int = ACT) -> None:
+        """``pre(tensor, tensor_id)`` for an op with one input, or
+        ``pre([(tensor, tensor_id), ...])`` for an op with several (concatenation,
+        residual add; Execution.h:135-212): the op index advances once and every
+        input whose ``begin_stage`` is this op goes out under its own policy."""
+        inputs = [(tensor, tensor_id)] if isinstance(tensor, torch.Tensor) else list(tensor)
         self.index += 1
-        self._pending = -1
-        if tensor_id < 0 or tensor_id >= len(self.policy):
-            return
-        pol = self.policy[tensor_id]
-        if self.index != self.begin_stage[tensor_id] or pol in (0, 1):
-            return
-        ticket = self.engine.pre(tensor, pol)
-        self._tickets[tensor_id] = (ticket, tuple(tensor.shape))
-        self._pending = tensor_id
+        self._pending = []
+        for t, tid in inputs:
+            if tid is None or tid < 0 or tid >= len(self.policy):
+                continue
+            pol = self.policy[tid]
+            if self.index != self.begin_stage[tid] or pol in (0, 1) or tid in self._tickets:
+                continue
+            ticket = self.engine.pre(t, pol)
+            self._tickets[tid] = (ticket, tuple(t.shape))
+            self._pending.append(tid)
 
     def post(self) -> int:
-        """Wait for the copy the matching ``pre`` started; returns the id of the
+        """Wait for the copies the matching ``pre`` started; returns the id of the
         op's output tensor (``x.tensor_id = index``, Execution.h:219)."""
-        if self._pending >= 0:
-            self.engine.post(self._tickets[self._pending][0])
-            self._pending = -1
+        for tid in self._pending:
+            self.engine.post(self._tickets[tid][0])
+        self._pending = []
         return self.index
 
     def swapped(self, tensor_id: int) -> bool:
@@ -65,6 +71,10 @@ class Execution:
         if tensor_id not in self._tickets:
             return 0
         return self.engine.info(self._tickets[tensor_id][0]).policy
+
+    def prefetch(self, tensor_id: int) -> None:
+        """Start the inbound copy of a tensor that a later fetch() will ask for."""
+        self.engine.prefetch(self._tickets[tensor_id][0])
 
     def fetch(self, tensor_id: int, out: torch.Tensor | None = None) -> torch.Tensor:
         ticket, shape = self._tickets.pop(tensor_id)

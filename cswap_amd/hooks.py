@@ -17,6 +17,9 @@ from __future__ import annotations
 import torch
 
 from . import swap
+from ._lib import CswapError
+
+E_NOMEM = -4   # CSWAP_E_NOMEM
 
 
 class _Handle:
@@ -33,12 +36,22 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
     The outbound copy of tensor i overlaps with whatever the compute stream does
     until tensor i+1 is packed, at which point its completion is awaited and the
     device copy is let go (the reference does the same one layer later,
-    CSWAP+/vgg16-cifar10.cpp:221-228)."""
+    CSWAP+/vgg16-cifar10.cpp:221-228).
 
-    def __init__(self, engine: "swap.SwapEngine", policy: int = swap.AUTO, min_bytes: int = 1 << 20):
+    Backward asks for the tensors in roughly the reverse of the order they were
+    packed in, so each unpack also starts the inbound copy of the ``prefetch``
+    tensors packed just before the one it returns: their transfer then runs on
+    the copy stream under the backward kernels of the current layer."""
+
+    def __init__(self, engine: "swap.SwapEngine", policy: int = swap.AUTO, min_bytes: int = 1 << 20,
+                 prefetch: int = 1):
         self.engine = engine
         self.policy = policy
         self.min_bytes = min_bytes
+        self.prefetch = prefetch
+        self._order = []           # handles in pack order
+        self._fetched = set()      # tickets already swapped in or being prefetched
+        self._released = set()
         self._pending = None       # handle whose outbound copy may still be in flight
         self._to_release = []      # tickets whose swap-in has been launched
         self.stats = {"swapped": 0, "bytes_in": 0, "bytes_out": 0, "kept": 0}
@@ -68,12 +81,14 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         self.stats["bytes_out"] += info.bytes_out
         h = _Handle(ticket, tuple(t.shape), t)   # keep the device copy alive until the copy finished
         self._pending = h
+        self._order.append(h)
         return h
 
     # -- backward side
     def _drain(self):
         for tk in self._to_release:
             self.engine.release(tk)
+            self._released.add(tk)
         self._to_release.clear()
 
     def _unpack(self, h):
@@ -84,11 +99,41 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         self._drain()
         out = torch.empty(h.shape, dtype=torch.float32, device="cuda")
         self.engine.swap_in(h.ticket, out)
+        self._fetched.add(h.ticket)
         self._to_release.append(h.ticket)   # released once the next swap-in is issued (or at close)
+        self._prefetch_before(h)
         return out
+
+    def _prefetch_before(self, h):
+        """Start the inbound copies of the tensors packed just before ``h``."""
+        if self.prefetch <= 0 or h not in self._order:
+            return
+        i = self._order.index(h)
+        started = 0
+        for g in reversed(self._order[:i]):
+            if started >= self.prefetch:
+                break
+            if g.ticket in self._fetched:
+                continue
+            if self._pending is g:
+                self._settle()
+            try:
+                self.engine.prefetch(g.ticket)
+            except CswapError as err:
+                if err.code != E_NOMEM:
+                    raise
+                break                      # staging pool full: the swap-in will fetch it on demand
+            self._fetched.add(g.ticket)
+            self.stats["prefetched"] = self.stats.get("prefetched", 0) + 1
+            started += 1
 
     def close(self):
         """Wait for and release everything still held; call after backward."""
         self._settle()
         torch.cuda.synchronize()
         self._drain()
+        for h in self._order:              # saved but never asked for by backward
+            if h.ticket not in self._released:
+                self.engine.release(h.ticket)
+                self._released.add(h.ticket)
+        self._order.clear()

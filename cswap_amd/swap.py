@@ -90,6 +90,10 @@ class SwapEngine:
               "cswap_swap_in")
         return out
 
+    def prefetch(self, ticket: int) -> None:
+        """Start the host-to-device copy of a swapped tensor ahead of its swap_in."""
+        check(lib().cswap_swap_prefetch(self._h, ticket), "cswap_swap_prefetch")
+
     def release(self, ticket: int) -> None:
         check(lib().cswap_swap_release(self._h, ticket), "cswap_swap_release")
 
@@ -158,3 +162,60 @@ def bench_schedule(dev, batch: int = 128, seed: int = 0) -> dict:
     return {"costs": {k: round(getattr(costs, k), 2) for k, _ in Costs._fields_ if k.endswith(("gbs", "us"))},
             "total_none_ms": round(tot["none"], 2), "total_auto_ms": round(tot["auto"], 2),
             "worst_compressed_over_raw": round(worst, 3), "tensors": rows}
+
+
+def bench_backward(dev, batch: int = 128, seed: int = 0, compute_reps: int = 2) -> dict:
+    """Configuration 4, backward side: every swapped tensor of the schedule is
+    already on the host; walk them in reverse (the order backward asks for them),
+    each followed by a dummy layer backward on the compute stream.  Compared:
+    raw tensors fetched on demand, compressed tensors fetched on demand, and
+    compressed tensors with the next one prefetched under the current layer."""
+    from .workloads import config4_schedule, config4_tensor
+
+    sched = [e for e in config4_schedule(batch) if e["kind"] != "dense"]   # the swapped ones: ReLU and pool outputs
+    total = sum(int(torch.tensor(e["shape"]).prod()) * 4 for e in sched)
+    biggest = max(int(torch.tensor(e["shape"]).prod()) for e in sched) * 4
+    eng = SwapEngine(pinned_bytes=total + (64 << 20), device_bytes=4 * biggest + (64 << 20))
+    eng.calibrate()
+    a = torch.randn(2048, 2048, device=dev)
+    b = torch.randn(2048, 2048, device=dev)
+    xs = [torch.from_numpy(config4_tensor(e, seed)).to(dev) for e in sched]
+    outs = [torch.empty_like(x) for x in xs]
+    res = {}
+    for label, pol, ahead in (("raw_on_demand", NONE, 0), ("compressed_on_demand", AUTO, 0),
+                              ("compressed_prefetch_1", AUTO, 1), ("raw_prefetch_1", NONE, 1)):
+        best = None
+        for _ in range(3):
+            tks = []
+            for x in xs:
+                tk = eng.pre(x, pol)
+                eng.post(tk)
+                tks.append(tk)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            order = list(range(len(xs)))[::-1]
+            if ahead:
+                eng.prefetch(tks[order[0]])
+            for k, i in enumerate(order):
+                if k >= 2:
+                    eng.release(tks[order[k - 2]])      # its decompression finished a layer ago
+                for j in order[k + 1:k + 1 + ahead]:
+                    eng.prefetch(tks[j])
+                eng.swap_in(tks[i], outs[i])
+                _dummy_compute(a, b, compute_reps)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            for i in order[-2:]:
+                eng.release(tks[i])
+            best = dt if best is None else min(best, dt)
+        res[label + "_ms"] = round(best * 1e3, 2)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in xs:
+        _dummy_compute(a, b, compute_reps)
+    torch.cuda.synchronize()
+    res["compute_only_ms"] = round((time.perf_counter() - t0) * 1e3, 2)
+    res["tensors"] = len(xs)
+    res["MB"] = round(total / 1e6, 1)
+    eng.close()
+    return res

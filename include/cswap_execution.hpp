@@ -37,34 +37,57 @@ class Execution {
   void preforward() { init(); }
   void postforward() {}
 
+  // One input of an op: its tensor id (-1: not a tracked tensor), device pointer and field extents.
+  struct Input {
+    int tensor_id;
+    const float* d_tensor;
+    size_t nx, ny, nz;
+  };
+
   // Call before op `index+1` runs on `compute`.  `tensor_id` is the id of the
   // op's input (-1: not a tracked tensor).  Returns a CSWAP_* status.
   int pre(int tensor_id, const float* d_tensor, size_t nx, size_t ny, size_t nz, cswap_stream_t compute,
-          Layer_type = ACT)
+          Layer_type layer_type = ACT)
+  {
+    const Input one = {tensor_id, d_tensor, nx, ny, nz};
+    return pre(std::vector<Input>(1, one), compute, layer_type);
+  }
+
+  // The same for an op with several inputs (concatenation, residual add;
+  // Execution.h:135-212): the op index advances once, every input whose
+  // begin_stage is this op goes out under its own policy, and the copies queue
+  // on the engine's copy stream in input order (the reference opens one stream
+  // per input, Execution.h:165,195,200; one link carries them either way).
+  // On an error the inputs already started stay pending for post().
+  int pre(const std::vector<Input>& inputs, cswap_stream_t compute, Layer_type = ACT)
   {
     index++;
-    pending_ = -1;
-    if (tensor_id < 0 || (size_t)tensor_id >= policy.size()) return CSWAP_OK;
-    const int pol = policy[(size_t)tensor_id];
-    if (index != begin_stage[(size_t)tensor_id] || pol == 0 || pol == 1) return CSWAP_OK;
-    int ticket = -1;
-    int rc = cswap_swap_out(engine_, d_tensor, nx, ny, nz, pol, compute, &ticket);
-    if (rc) return rc;
-    tickets_[tensor_id] = ticket;
-    pending_ = tensor_id;
+    pending_.clear();
+    for (const Input& in : inputs) {
+      if (in.tensor_id < 0 || (size_t)in.tensor_id >= policy.size()) continue;
+      const int pol = policy[(size_t)in.tensor_id];
+      if (index != begin_stage[(size_t)in.tensor_id] || pol == 0 || pol == 1) continue;
+      if (tickets_.count(in.tensor_id)) continue;  // the same tensor fed twice to one op
+      int ticket = -1;
+      int rc = cswap_swap_out(engine_, in.d_tensor, in.nx, in.ny, in.nz, pol, compute, &ticket);
+      if (rc) return rc;
+      tickets_[in.tensor_id] = ticket;
+      pending_.push_back(in.tensor_id);
+    }
     return CSWAP_OK;
   }
 
-  // Call after the op has been launched: waits for the copy started by the
-  // matching pre() (Execution.h:248-299); afterwards the caller may release the
-  // device storage of the input.  Returns the id of the op's output tensor.
+  // Call after the op has been launched: waits for the copies started by the
+  // matching pre() (Execution.h:248-299, 311-401); afterwards the caller may
+  // release the device storage of the inputs.  Returns the id of the op's output tensor.
   int post(int* status = nullptr)
   {
     int rc = CSWAP_OK;
-    if (pending_ >= 0) {
-      rc = cswap_swap_wait(engine_, tickets_[pending_]);
-      pending_ = -1;
+    for (int id : pending_) {
+      int r = cswap_swap_wait(engine_, tickets_[id]);
+      if (r && !rc) rc = r;
     }
+    pending_.clear();
     if (status) *status = rc;
     return index;
   }
@@ -78,6 +101,15 @@ class Execution {
     if (it == tickets_.end()) return 0;
     cswap_ticket_info info;
     return cswap_swap_info(engine_, it->second, &info) == CSWAP_OK ? info.policy : 0;
+  }
+
+  // Backward side, ahead of time: start the inbound copy of a tensor that a later
+  // fetch() will ask for, so that it overlaps the backward kernels before it.
+  int prefetch(int tensor_id)
+  {
+    auto it = tickets_.find(tensor_id);
+    if (it == tickets_.end()) return CSWAP_E_STATE;
+    return cswap_swap_prefetch(engine_, it->second);
   }
 
   // Backward side: bring the tensor back into d_out on `compute` and forget it.
@@ -99,7 +131,7 @@ class Execution {
  private:
   cswap_engine* engine_;
   std::map<int, int> tickets_;
-  int pending_ = -1;
+  std::vector<int> pending_;
 };
 
 }  // namespace cswap

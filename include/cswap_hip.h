@@ -214,7 +214,7 @@ typedef struct {
   int    policy;              /* what was actually done */
   size_t n, nnz;              /* elements; non-zeros (valid when probed) */
   size_t bytes_in, bytes_out; /* 4*n; bytes that crossed the link */
-  int    state;               /* 0 free, 1 out in flight, 2 resident on host, 3 in in flight */
+  int    state;               /* 0 free, 1 out in flight, 2 resident on host, 3 in in flight, 4 prefetched */
 } cswap_ticket_info;
 
 void cswap_engine_config_default(cswap_engine_config* cfg);
@@ -234,6 +234,14 @@ int cswap_swap_wait(cswap_engine* e, int ticket);
  * `compute` (ordered by an event).  Returns at once; the data is ready when
  * `compute` reaches this point. */
 int cswap_swap_in(cswap_engine* e, int ticket, float* d_out, cswap_stream_t compute);
+/* Backward side, ahead of time: start the host-to-device copy of the payload
+ * into the engine's device staging pool on the copy stream, before a
+ * destination exists, so that it overlaps the backward compute of the layers
+ * that run first.  A later cswap_swap_in then only waits for that copy and
+ * decompresses (policy NONE: one device-to-device copy).  Idempotent; the
+ * reference's counterpart lives in its patched autograd engine, which it does
+ * not ship (fields read at Execution.h:260-262,278-282). */
+int cswap_swap_prefetch(cswap_engine* e, int ticket);
 /* Return the ticket's host (and any device) memory to the pools.  Waits for the
  * work of the ticket that is still in flight. */
 int cswap_swap_release(cswap_engine* e, int ticket);

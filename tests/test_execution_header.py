@@ -18,9 +18,13 @@ int main() {
   int id = exe.post();
   rc |= exe.pre(0, nullptr, 1, 1, 1, nullptr);            // policy 0: kept
   exe.post();
+  std::vector<cswap::Execution::Input> two = {{0, nullptr, 1, 1, 1}, {-1, nullptr, 1, 1, 1}};
+  rc |= exe.pre(two, nullptr, cswap::CONV);               // an op with two inputs, neither swapped
+  int id2 = exe.post();
+  rc |= (exe.prefetch(7) == CSWAP_E_STATE) ? 0 : 1;       // nothing was swapped under id 7
   exe.postforward();
-  printf("%d %d %d %d\n", rc, id, exe.index, (int)exe.swapped(0));
-  return (rc == 0 && id == 0 && exe.index == 1 && !exe.swapped(0) && exe.com_and_tran(5) == 0) ? 0 : 1;
+  printf("%d %d %d %d %d\n", rc, id, id2, exe.index, (int)exe.swapped(0));
+  return (rc == 0 && id == 0 && id2 == 2 && exe.index == 2 && !exe.swapped(0) && exe.com_and_tran(5) == 0) ? 0 : 1;
 }
 """
 

@@ -62,8 +62,11 @@ def test_vgg_walk_with_reference_policy_vector():
     assert exe.com_and_tran(2) == 3 and exe.com_and_tran(6) == 6 and exe.com_and_tran(5) == 2
     assert exe.com_and_tran(12) in (2, 3, 6) and exe.com_and_tran(0) == 0
 
-    for tid in sorted(kept, reverse=True):       # backward order
+    order = sorted(kept, reverse=True)           # backward order
+    for k, tid in enumerate(order):
         tag = exe.com_and_tran(tid)
+        if k + 1 < len(order):
+            exe.prefetch(order[k + 1])           # the next one comes in under this layer's backward
         back = exe.fetch(tid)
         torch.cuda.synchronize()
         ref = kept[tid]
@@ -74,4 +77,45 @@ def test_vgg_walk_with_reference_policy_vector():
         else:
             assert torch.equal(back, ref)
         assert not exe.swapped(tid)
+    eng.close()
+
+
+def test_op_with_several_inputs_swaps_each_under_its_own_policy():
+    """Vector form of pre/post (Execution.h:135-212,311-401): a residual add whose
+    two inputs are both consumed by that op, one as ZVC and one as ZFP, plus an
+    untracked third input."""
+    import torch
+
+    import oracle
+    from cswap_amd import swap
+    from cswap_amd.execution import ACT, Execution
+
+    torch.manual_seed(1)
+    eng = swap.SwapEngine(pinned_bytes=256 << 20, device_bytes=256 << 20)
+    exe = Execution(eng)
+    exe.init_(8)
+    exe.policy[0] = 3
+    exe.policy[1] = 6
+    exe.begin_stage[0] = 2            # both are consumed by op 2, the add
+    exe.begin_stage[1] = 2
+    a = torch.relu(torch.randn(16, 64, 32, 32, device="cuda"))      # output of op 0
+    b = torch.randn(16, 64, 32, 32, device="cuda")                  # output of op 1
+    c = torch.randn(16, 64, 32, 32, device="cuda")                  # not tracked
+    exe.preforward()
+    exe.pre(a, -1); exe.post()        # op 0
+    exe.pre(a, -1); exe.post()        # op 1
+    exe.pre([(a, 0), (b, 1), (c, -1)], layer_type=ACT)              # op 2
+    s = a + b + c
+    assert exe.post() == 2
+    exe.postforward()
+    assert exe.swapped(0) and exe.swapped(1) and exe.com_and_tran(0) == 3 and exe.com_and_tran(1) == 6
+    exe.prefetch(0)
+    back_b = exe.fetch(1)
+    back_a = exe.fetch(0)
+    torch.cuda.synchronize()
+    assert torch.equal(back_a, a)
+    f = b.cpu().numpy().reshape(-1, 32, 32)
+    want = oracle.zfp_decode3(oracle.zfp_encode3(f, 512, omp=True), f.shape, 512, omp=True)
+    assert np.array_equal(back_b.cpu().numpy().reshape(f.shape).view(np.uint32), want.view(np.uint32))
+    assert torch.equal(s, a + b + c)
     eng.close()

@@ -62,11 +62,18 @@ def test_lossless_policies_keep_gradients_bit_identical(torch_cuda, policy_name)
     ctx = swap_saved_tensors(eng, policy=pol, min_bytes=1 << 16)
     loss1, g1 = grads(torch, net, x, ctx)
     assert ctx.stats["swapped"] >= 3
+    assert ctx.stats["prefetched"] >= 2          # backward pulled the earlier tensors in ahead of time
     assert loss1 == loss0
     for a, b in zip(g0, g1):
         assert torch.equal(a, b)
     if policy_name == "sparse":
         assert ctx.stats["bytes_out"] < ctx.stats["bytes_in"]
+    # same result with on-demand swap-in only, and with a deeper look-ahead
+    for depth in (0, 3):
+        ctx = swap_saved_tensors(eng, policy=pol, min_bytes=1 << 16, prefetch=depth)
+        loss2, g2 = grads(torch, net, x, ctx)
+        assert loss2 == loss0 and all(torch.equal(a, b) for a, b in zip(g0, g2)), depth
+        assert ctx.stats.get("prefetched", 0) == 0 if depth == 0 else ctx.stats["prefetched"] >= 2
     eng.close()
 
 

@@ -144,6 +144,55 @@ def test_copies_are_ordered_against_compute_by_events(torch_cuda, engine):
             assert float(total) == float(want.sum())
 
 
+@pytest.mark.parametrize("policy_name", ["none", "sparse", "zfp", "auto"])
+def test_prefetch_then_swap_in_equals_plain_swap_in(torch_cuda, engine, policy_name):
+    """cswap_swap_prefetch moves the payload to device staging ahead of time; the
+    swap-in that follows must give bit for bit what an on-demand swap-in gives,
+    also when the prefetch is issued while the outbound copy is still in flight."""
+    torch = torch_cuda
+    from cswap_amd import swap
+
+    pol = {"none": swap.NONE, "sparse": swap.SPARSE, "zfp": swap.ZFP, "auto": swap.AUTO}[policy_name]
+    x = relu_tensor(torch, (8, 64, 32, 32), 0.7, 11)
+    plain = torch.full_like(x, -5.0)
+    tk = engine.pre(x, pol)
+    engine.post(tk)
+    engine.swap_in(tk, plain)
+    torch.cuda.synchronize()
+    engine.release(tk)
+
+    for settle_first in (True, False):
+        out = torch.full_like(x, -7.0)
+        tk = engine.pre(x, pol)
+        if settle_first:
+            engine.post(tk)
+        engine.prefetch(tk)
+        assert engine.info(tk).state == 4
+        engine.prefetch(tk)                      # idempotent
+        busy = torch.randn(1024, 1024, device="cuda")
+        for _ in range(4):                       # compute that the copy can hide under
+            busy = busy @ busy * 1e-3
+        engine.swap_in(tk, out)
+        assert engine.info(tk).state == 3
+        torch.cuda.synchronize()
+        engine.release(tk)
+        assert torch.equal(out.view(torch.int32), plain.view(torch.int32)), (policy_name, settle_first)
+
+
+def test_prefetched_ticket_can_be_released_unused(torch_cuda, engine):
+    torch = torch_cuda
+    from cswap_amd import swap
+
+    x = relu_tensor(torch, (4, 64, 32, 32), 0.5, 12)
+    tk = engine.pre(x, swap.ZFP)
+    engine.prefetch(tk)
+    engine.release(tk)
+    assert engine.info(tk).state == 0
+    L = __import__("cswap_amd._lib", fromlist=["lib"]).lib()
+    assert L.cswap_swap_prefetch(engine._h, tk) == -5       # released ticket
+    assert L.cswap_swap_prefetch(engine._h, 10 ** 6) == -1  # no such ticket
+
+
 def test_state_machine_errors(torch_cuda, engine):
     torch = torch_cuda
     from cswap_amd._lib import lib
