@@ -49,6 +49,12 @@ class TicketInfo(C.Structure):
                 ("bytes_out", C.c_size_t), ("state", C.c_int)]
 
 
+class PlanSummary(C.Structure):
+    _fields_ = [("time_us", C.c_double), ("base_time_us", C.c_double), ("bytes_total", C.c_size_t),
+                ("bytes_target", C.c_size_t), ("bytes_moved", C.c_size_t), ("bytes_on_link", C.c_size_t),
+                ("n_selected", C.c_int), ("target_met", C.c_int)]
+
+
 class ZfpBitstream(C.Structure):
     _fields_ = [("bits", C.c_uint), ("buffer", C.c_uint64), ("ptr", C.c_void_p), ("begin", C.c_void_p),
                 ("end", C.c_void_p)]
@@ -105,6 +111,19 @@ _SIGNATURES = {
     "cswap_swap_info": (i32, [vp, i32, C.POINTER(TicketInfo)]),
     "cswap_engine_calibrate": (i32, [vp, C.POINTER(Costs)]),
     "cswap_engine_copy_stream": (vp, [vp]),
+    "cswap_planner_create": (vp, [C.POINTER(Costs), u]),
+    "cswap_planner_destroy": (None, [vp]),
+    "cswap_planner_reset": (i32, [vp]),
+    "cswap_planner_set_backward_factor": (i32, [vp, C.c_double]),
+    "cswap_planner_add_comptime": (i32, [vp, C.c_double]),
+    "cswap_planner_add_tensor": (i32, [vp, i32, sz]),
+    "cswap_planner_add_stepdep": (i32, [vp, i32, i32]),
+    "cswap_planner_add_omitid": (i32, [vp, i32]),
+    "cswap_planner_set_field": (i32, [vp, i32, sz, sz, sz]),
+    "cswap_planner_set_nnz": (i32, [vp, i32, sz]),
+    "cswap_planner_init": (i32, [vp, C.c_double]),
+    "cswap_planner_make_policy": (i32, [vp, C.POINTER(i32), C.POINTER(i32), i32, C.POINTER(PlanSummary)]),
+    "cswap_planner_capuchin": (i32, [vp, C.POINTER(i32), C.POINTER(i32), i32, C.POINTER(PlanSummary)]),
     # the reference's own entry-point names (include/cswap_compat.h)
     "PreGPUcompression": (None, [i32, i32, vp, vp, i32, i32, vp]),
     "PreAcc": (None, [vp, i32, vp, i32, i32, vp]),

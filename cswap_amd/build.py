@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libcswap_hip.so")
 
-SOURCES = ["common.cpp", "zfp_kernels.hip", "zvc_kernels.hip", "select.cpp", "swap_engine.cpp",
+SOURCES = ["common.cpp", "zfp_kernels.hip", "zvc_kernels.hip", "select.cpp", "planner.cpp", "swap_engine.cpp",
            "compat.cpp"]
 
 HIPCC_FLAGS = [

@@ -251,6 +251,56 @@ int cswap_swap_info(cswap_engine* e, int ticket, cswap_ticket_info* info);
 int cswap_engine_calibrate(cswap_engine* e, cswap_costs* out_costs);
 cswap_stream_t cswap_engine_copy_stream(cswap_engine* e);
 
+/* --------------------------------------------------------------- planner -----
+ * Which activations to move off the device, and with which action, so that a
+ * given share of the activation bytes leaves the device at the least predicted
+ * cost.  Stands in for c10::PolicyMaker of the reference's patched PyTorch
+ * (definitions not in its tree; driven as at inception-v3-cifar100.cpp:207-214
+ * and vgg16-cifar10.cpp:474-497).  Pure host code.  Tensor id = index of the op
+ * that produced it; ops are numbered in the order of cswap_planner_add_comptime.
+ */
+typedef struct cswap_planner cswap_planner;
+
+typedef struct {
+  double time_us;        /* predicted iteration time with the plan */
+  double base_time_us;   /* predicted iteration time with nothing swapped */
+  size_t bytes_total;    /* bytes of all recorded tensors */
+  size_t bytes_target;   /* ratio * bytes_total */
+  size_t bytes_moved;    /* device bytes the plan moves to the host */
+  size_t bytes_on_link;  /* bytes that cross the link one way under the plan */
+  int    n_selected;
+  int    target_met;     /* 0: every eligible tensor is selected and it is still not enough */
+} cswap_plan_summary;
+
+/* costs NULL (or without link bandwidth) = cswap_costs_default; zfp_maxbits 0 = 512 */
+cswap_planner* cswap_planner_create(const cswap_costs* costs, unsigned zfp_maxbits);
+void cswap_planner_destroy(cswap_planner* p);
+int  cswap_planner_reset(cswap_planner* p);
+/* backward time of an op = factor * its forward time (default 2) */
+int  cswap_planner_set_backward_factor(cswap_planner* p, double factor);
+/* PolicyMaker::add_comptime(timeuse): forward time of the next op */
+int  cswap_planner_add_comptime(cswap_planner* p, double microseconds);
+/* PolicyMaker::add_tensor(index, x.nbytes()) */
+int  cswap_planner_add_tensor(cswap_planner* p, int id, size_t nbytes);
+/* PolicyMaker::add_stepdep({pre.tensor_id, index}): op to_id consumes tensor from_id (-1: untracked input) */
+int  cswap_planner_add_stepdep(cswap_planner* p, int from_id, int to_id);
+/* PolicyMaker::add_omitid(id): never touch this tensor */
+int  cswap_planner_add_omitid(cswap_planner* p, int id);
+/* What the reference's profile cannot know: the field extents (exact ZFP size)
+ * and the non-zero count of the profiled iteration (enables ZVC for the tensor). */
+int  cswap_planner_set_field(cswap_planner* p, int id, size_t nx, size_t ny, size_t nz);
+int  cswap_planner_set_nnz(cswap_planner* p, int id, size_t nnz);
+/* PolicyMaker::init(ratio): share of the recorded bytes to move off the device, 0..1 */
+int  cswap_planner_init(cswap_planner* p, double ratio);
+/* PolicyMaker::make_policy(time_): policy[id] in {0 keep, 2 raw, 3 ZVC, 6 ZFP}
+ * (Execution.h:70,86,107) and begin_stage[id] = op of the last forward use
+ * (what read_lastvisit fills, resnet-cifar10.cpp:330); both arrays have n entries,
+ * begin_stage may be NULL. */
+int  cswap_planner_make_policy(cswap_planner* p, int* policy, int* begin_stage, int n, cswap_plan_summary* summary);
+/* PolicyMaker::capuchin(time_): the raw-swap baseline (action 2 only, tensors
+ * that stay away longest first). */
+int  cswap_planner_capuchin(cswap_planner* p, int* policy, int* begin_stage, int n, cswap_plan_summary* summary);
+
 #ifdef __cplusplus
 }
 #endif
