@@ -280,6 +280,8 @@ def extras(torch, api, dev):
         from cswap_amd import swap
         ex["swap"] = swap.bench_schedule(dev)
         ex["swap_backward"] = swap.bench_backward(dev)
+        from cswap_amd import planner
+        ex["planner"] = planner.bench_planner(dev)
     except ImportError:
         pass
     return ex

@@ -119,3 +119,44 @@ def test_op_with_several_inputs_swaps_each_under_its_own_policy():
     assert np.array_equal(back_b.cpu().numpy().reshape(f.shape).view(np.uint32), want.view(np.uint32))
     assert torch.equal(s, a + b + c)
     eng.close()
+
+
+def test_planned_iteration_restores_every_swapped_tensor():
+    """Profile -> make_policy -> Execution walk with prefetch: every tensor the plan
+    moved comes back as its codec round trip (lossless actions: bit-identical)."""
+    import torch
+
+    from cswap_amd import api, swap
+    from cswap_amd.planner import PolicyMaker, _vgg_modules, run_planned_iteration
+
+    torch.manual_seed(0)
+    dev = torch.device("cuda")
+    mods = [m.eval() for m in _vgg_modules(torch, dev)][:17]
+    x = torch.randn(16, 3, 64, 64, device=dev)
+    costs = swap.default_costs()
+    costs.allow_lossy = 0
+    costs.size_floor_bytes = 0
+    pm = PolicyMaker(costs)
+    with torch.no_grad():
+        t, tid = x, -1
+        for i, m in enumerate(mods):
+            out = m(t)
+            pm.add_comptime(100.0)
+            pm.add_tensor(i, out.numel() * 4)
+            pm.add_stepdep([tid, i])
+            pm.set_nnz(i, int(api.probe_nnz(out).item()))
+            t, tid = out, i
+    pm.init(0.6)
+    pol, _ = pm.make_policy(len(mods))
+    assert 3 in pol and 2 in pol and 6 not in pol
+    eng = swap.SwapEngine(pinned_bytes=1 << 30, device_bytes=512 << 20)
+    seen, kept = [], {}
+
+    def check(tid, back):
+        seen.append(tid)
+        assert torch.equal(back, kept[tid]), tid
+
+    run_planned_iteration(eng, mods, x, pol, pm.begin_stage, check=check, keep=kept)
+    assert sorted(seen) == [i for i, p in enumerate(pol) if p]
+    eng.close()
+    pm.close()
