@@ -273,6 +273,31 @@ def extras(torch, api, dev):
 
     for pct in (30, 50, 70, 90):
         zvc_case(f"config2_s{pct}", torch.from_numpy(config2_tensor(pct)).to(dev))
+
+    # ---- ZVC chunk count: the reference's 512*32 against the size rule the engine uses
+    def geometry_case(mib):
+        from cswap_amd._lib import lib
+        L = lib()
+        n = mib * 1024 * 1024 // 4
+        t = torch.relu(torch.randn(n, device=dev))
+        o = torch.empty_like(t)
+        st = torch.cuda.current_stream().cuda_stream
+        row = {}
+        for label, process in (("reference_16384", api.PROCESS), ("size_rule", L.cswap_zvc_pick_process(n))):
+            _, W, _ = api.zvc_geometry(n, process)
+            values = torch.empty(n, device=dev)
+            mask = torch.empty(W * process, dtype=torch.int32, device=dev)
+            begin = torch.zeros(process, dtype=torch.int32, device=dev)
+            nnz = torch.zeros(1, dtype=torch.int32, device=dev)
+            c = ev_ms(torch, lambda: L.cswap_zvc_compress(t.data_ptr(), n, process, begin.data_ptr(), nnz.data_ptr(),
+                                                          values.data_ptr(), mask.data_ptr(), st), 30)
+            e = ev_ms(torch, lambda: L.cswap_zvc_expand(values.data_ptr(), mask.data_ptr(), begin.data_ptr(), n,
+                                                        process, o.data_ptr(), st), 30)
+            row[label] = {"process": process, "compress_ms": round(c, 4), "expand_ms": round(e, 4)}
+        ex[f"zvc_geometry_{mib}MiB"] = row
+
+    for mib in (1, 4, 16, 32, 128):
+        geometry_case(mib)
     g = torch.Generator(device=dev); g.manual_seed(1)
     zvc_case("relu_256MiB", torch.relu(torch.randn(64 * 1024 * 1024, generator=g, device=dev)))
 

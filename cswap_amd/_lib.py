@@ -88,6 +88,7 @@ _SIGNATURES = {
     "cswap_zvc_chunk_words": (i32, [i32, i32]),
     "cswap_zvc_active_chunks": (i32, [i32, i32]),
     "cswap_zvc_mask_bytes": (sz, [i32, i32]),
+    "cswap_zvc_pick_process": (i32, [sz]),
     "cswap_zvc_count": (i32, [vp, i32, i32, vp, vp]),
     "cswap_zvc_scan": (i32, [vp, i32, vp, vp]),
     "cswap_zvc_compact": (i32, [vp, i32, i32, vp, vp, vp, vp]),
@@ -111,6 +112,8 @@ _SIGNATURES = {
     "cswap_swap_info": (i32, [vp, i32, C.POINTER(TicketInfo)]),
     "cswap_engine_calibrate": (i32, [vp, C.POINTER(Costs)]),
     "cswap_engine_copy_stream": (vp, [vp]),
+    "cswap_engine_tune": (i32, [vp, sz, C.POINTER(i32)]),
+    "cswap_engine_process_for": (i32, [vp, sz]),
     "cswap_planner_create": (vp, [C.POINTER(Costs), u]),
     "cswap_planner_destroy": (None, [vp]),
     "cswap_planner_reset": (i32, [vp]),

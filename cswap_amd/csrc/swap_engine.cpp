@@ -91,6 +91,7 @@ enum TicketState { kFree = 0, kOutInFlight = 1, kOnHost = 2, kInInFlight = 3, kP
 struct Ticket {
   int state = kFree;
   int policy = CSWAP_POLICY_NONE;
+  int process = 0;  // ZVC chunk count this tensor was compacted with
   size_t n = 0, nnz = 0, nx = 0, ny = 0, nz = 0;
   size_t bytes_out = 0;
   size_t host_off = 0, host_bytes = 0;
@@ -111,7 +112,8 @@ struct cswap_engine {
   Pool hpool, dpool;
   std::vector<Ticket> tickets;
   cswap_costs costs;
-  int process = 512 * 32;
+  int process = 0;       // fixed ZVC chunk count; 0 = per tensor size
+  int tuned[40] = {0};   // measured best chunk count per size class (index = bit length of n), 0 = not measured
   unsigned maxbits = 512;
   int* h_nnz = nullptr;  // pinned, 1 int
   int* d_nnz = nullptr;
@@ -127,7 +129,7 @@ extern "C" void cswap_engine_config_default(cswap_engine_config* cfg)
   if (!cfg) return;
   cfg->pinned_pool_bytes = (size_t)1 << 30;
   cfg->device_pool_bytes = (size_t)1 << 30;
-  cfg->process = 512 * 32;
+  cfg->process = 0;
   cfg->zfp_maxbits = 512;
   cfg->max_tickets = 256;
   cswap_costs_default(&cfg->costs);
@@ -157,13 +159,12 @@ extern "C" int cswap_engine_create(cswap_engine** out, const cswap_engine_config
   cswap_engine_config cfg;
   if (cfg_in) cfg = *cfg_in; else cswap_engine_config_default(&cfg);
   if (!cfg.pinned_pool_bytes || !cfg.device_pool_bytes) return CSWAP_E_ARG;
-  if (cfg.process == 0) cfg.process = 512 * 32;
   if (cfg.zfp_maxbits == 0) cfg.zfp_maxbits = 512;
   if (cfg.max_tickets <= 0) cfg.max_tickets = 256;
   if (cfg.process < 0 || cfg.process > (1 << 20) || cfg.zfp_maxbits < 16 || cfg.zfp_maxbits > 4096)
     return CSWAP_E_ARG;
   if (cfg.costs.bw_d2h_gbs <= 0 || cfg.costs.bw_h2d_gbs <= 0) cswap_costs_default(&cfg.costs);
-  cfg.costs.process = cfg.process;
+  cfg.costs.process = cfg.process ? cfg.process : 512 * 32;
 
   cswap_engine* e = new (std::nothrow) cswap_engine;
   if (!e) return CSWAP_E_NOMEM;
@@ -199,6 +200,22 @@ extern "C" int cswap_engine_create(cswap_engine** out, const cswap_engine_config
 
 extern "C" cswap_stream_t cswap_engine_copy_stream(cswap_engine* e) { return e ? (cswap_stream_t)e->copy : nullptr; }
 
+static int size_class(size_t n)
+{
+  int b = 0;
+  while (n) { b++; n >>= 1; }
+  return b < 40 ? b : 39;
+}
+
+// Chunk count for a tensor of n elements: the configured one, else what
+// cswap_engine_tune measured for tensors of this size class, else the rule.
+static int process_for(const cswap_engine* e, size_t n)
+{
+  if (e->process > 0) return e->process;
+  const int t = e->tuned[size_class(n)];
+  return t > 0 ? t : cswap_zvc_pick_process(n);
+}
+
 static void drop_device(cswap_engine* e, Ticket& t)
 {
   if (t.dev_held) {
@@ -228,6 +245,9 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   Ticket& t = e->tickets[(size_t)id];
   t.policy = policy; t.n = n; t.nnz = 0; t.nx = nx; t.ny = ny; t.nz = nz;
   t.dev_held = false;
+  t.process = zvc_ok ? process_for(e, n) : 0;
+  cswap_costs costs = e->costs;  // the selector prices the ZVC header with this tensor's chunk count
+  if (t.process) costs.process = t.process;
 
   int rc;
   bool want_probe = (policy == CSWAP_POLICY_AUTO && zvc_ok) || policy == CSWAP_POLICY_SPARSE;
@@ -236,7 +256,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     // best conceivable ZVC outcome (all zeros) is modelled to beat the raw swap,
     // the raw swap it is.
     cswap_choice best_case;
-    if ((rc = cswap_select_field(nx, ny, nz, 0, e->maxbits, &e->costs, &best_case))) return rc;
+    if ((rc = cswap_select_field(nx, ny, nz, 0, e->maxbits, &costs, &best_case))) return rc;
     if (best_case.policy == CSWAP_POLICY_NONE) {
       policy = t.policy = CSWAP_POLICY_NONE;
       want_probe = false;
@@ -245,14 +265,14 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   if (want_probe) {
     // Worst-case ZVC staging; the chunk counts go straight into its header so
     // that a later compaction needs no second counting pass.
-    const size_t hdr = zvc_header_bytes((int)n, e->process);
+    const size_t hdr = zvc_header_bytes((int)n, t.process);
     const size_t worst = hdr + 4 * n;
     size_t off;
     if (e->dpool.alloc(worst, &off)) {
       t.dev_off = off; t.dev_bytes = worst; t.dev_held = true;
       int* d_begin = (int*)(e->d_base + off);
-      if ((rc = cswap_zvc_count(d_in, (int)n, e->process, d_begin, compute))) { drop_device(e, t); return rc; }
-      if ((rc = cswap_zvc_scan(d_begin, cswap_zvc_active_chunks((int)n, e->process), e->d_nnz, compute))) {
+      if ((rc = cswap_zvc_count(d_in, (int)n, t.process, d_begin, compute))) { drop_device(e, t); return rc; }
+      if ((rc = cswap_zvc_scan(d_begin, cswap_zvc_active_chunks((int)n, t.process), e->d_nnz, compute))) {
         drop_device(e, t); return rc;
       }
       hipError_t err = hipMemcpyAsync(e->h_nnz, e->d_nnz, sizeof(int), hipMemcpyDeviceToHost, compute);
@@ -271,7 +291,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
 
   if (policy == CSWAP_POLICY_AUTO) {
     cswap_choice ch;
-    cswap_costs c = e->costs;
+    cswap_costs c = costs;
     if (!t.dev_held) c.sparse_max_ratio = 0.0;  // not probed: ZVC is not an option
     if ((rc = cswap_select_field(nx, ny, nz, t.nnz, e->maxbits, &c, &ch))) { drop_device(e, t); return rc; }
     t.policy = ch.policy;
@@ -280,12 +300,12 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   // ---- compress on the compute stream
   const void* src = nullptr;
   if (t.policy == CSWAP_POLICY_SPARSE) {
-    const size_t hdr = zvc_header_bytes((int)n, e->process);
+    const size_t hdr = zvc_header_bytes((int)n, t.process);
     char* base = e->d_base + t.dev_off;
     int* d_begin = (int*)base;
-    uint32_t* d_mask = (uint32_t*)(base + 4 * (size_t)e->process);
+    uint32_t* d_mask = (uint32_t*)(base + 4 * (size_t)t.process);
     float* d_values = (float*)(base + hdr);
-    if ((rc = cswap_zvc_compact(d_in, (int)n, e->process, d_begin, d_values, d_mask, compute))) {
+    if ((rc = cswap_zvc_compact(d_in, (int)n, t.process, d_begin, d_values, d_mask, compute))) {
       drop_device(e, t); return rc;
     }
     t.bytes_out = hdr + 4 * t.nnz;
@@ -441,10 +461,10 @@ extern "C" int cswap_swap_in(cswap_engine* e, int ticket, float* d_out, cswap_st
     return hip_fail(err);
   }
   if (t->policy == CSWAP_POLICY_SPARSE) {
-    const size_t hdr = zvc_header_bytes((int)t->n, e->process);
+    const size_t hdr = zvc_header_bytes((int)t->n, t->process);
     char* base = (char*)src;
-    rc = cswap_zvc_expand((const float*)(base + hdr), (const uint32_t*)(base + 4 * (size_t)e->process),
-                          (const int*)base, (int)t->n, e->process, d_out, compute);
+    rc = cswap_zvc_expand((const float*)(base + hdr), (const uint32_t*)(base + 4 * (size_t)t->process),
+                          (const int*)base, (int)t->n, t->process, d_out, compute);
   } else if (t->policy == CSWAP_POLICY_ZFP) {
     rc = cswap_zfp_decompress_f32((const uint64_t*)src, t->nx, t->ny, t->nz, 0, 0, 0, e->maxbits, d_out, compute);
   }
@@ -532,7 +552,8 @@ extern "C" int cswap_engine_calibrate(cswap_engine* e, cswap_costs* out_costs)
     if (4 * n > hfree) { rc = CSWAP_E_NOMEM; break; }
     if (!e->hpool.alloc(4 * n, &hoff)) { rc = CSWAP_E_NOMEM; break; }
     hheld = true;
-    const size_t hdr = zvc_header_bytes((int)n, e->process);
+    const int proc = process_for(e, n);
+    const size_t hdr = zvc_header_bytes((int)n, proc);
     hipError_t er;
     if ((er = hipMalloc((void**)&d_x, 4 * n)) != hipSuccess || (er = hipMalloc((void**)&d_y, 4 * n)) != hipSuccess ||
         (er = hipMalloc((void**)&d_tmp, hdr + 4 * n)) != hipSuccess ||
@@ -556,10 +577,10 @@ extern "C" int cswap_engine_calibrate(cswap_engine* e, cswap_costs* out_costs)
     if ((rc = ms(small, 20, &t))) break;
     c.copy_latency_us = t * 1e3;
     int* d_begin = (int*)d_tmp;
-    uint32_t* d_mask = (uint32_t*)(d_tmp + 4 * (size_t)e->process);
+    uint32_t* d_mask = (uint32_t*)(d_tmp + 4 * (size_t)proc);
     float* d_vals = (float*)(d_tmp + hdr);
-    auto zc = [&]() { return cswap_zvc_compress(d_x, (int)n, e->process, d_begin, e->d_nnz, d_vals, d_mask, s); };
-    auto ze = [&]() { return cswap_zvc_expand(d_vals, d_mask, d_begin, (int)n, e->process, d_y, s); };
+    auto zc = [&]() { return cswap_zvc_compress(d_x, (int)n, proc, d_begin, e->d_nnz, d_vals, d_mask, s); };
+    auto ze = [&]() { return cswap_zvc_expand(d_vals, d_mask, d_begin, (int)n, proc, d_y, s); };
     if ((rc = ms(zc, 2, &t))) break;
     if ((rc = ms(zc, 10, &t))) break;
     c.zvc_compress_gbs = gb / (t * 1e-3);
@@ -577,17 +598,18 @@ extern "C" int cswap_engine_calibrate(cswap_engine* e, cswap_costs* out_costs)
     c.zfp_decompress_gbs = gb / (t * 1e-3);
     // the probe: counting pass throughput, and the fixed cost of count + scan +
     // 4-byte copy + host wait measured on a tensor too small to matter
-    auto cnt = [&]() { return cswap_zvc_count(d_x, (int)n, e->process, d_begin, s); };
+    auto cnt = [&]() { return cswap_zvc_count(d_x, (int)n, proc, d_begin, s); };
     if ((rc = ms(cnt, 2, &t))) break;
     if ((rc = ms(cnt, 10, &t))) break;
     c.probe_gbs = gb / (t * 1e-3);
     {
       const int small_n = 1 << 16, reps = 10;
+      const int small_proc = process_for(e, (size_t)small_n);
       hipError_t er2 = hipStreamSynchronize(s);
       auto t0 = std::chrono::steady_clock::now();
       for (int i = 0; i < reps && er2 == hipSuccess && !rc; i++) {
-        rc = cswap_zvc_count(d_x, small_n, e->process, d_begin, s);
-        if (!rc) rc = cswap_zvc_scan(d_begin, cswap_zvc_active_chunks(small_n, e->process), e->d_nnz, s);
+        rc = cswap_zvc_count(d_x, small_n, small_proc, d_begin, s);
+        if (!rc) rc = cswap_zvc_scan(d_begin, cswap_zvc_active_chunks(small_n, small_proc), e->d_nnz, s);
         if (!rc) er2 = hipMemcpyAsync(e->h_nnz, e->d_nnz, sizeof(int), hipMemcpyDeviceToHost, s);
         if (!rc && er2 == hipSuccess) er2 = hipEventRecord(e->ev_probe, s);
         if (!rc && er2 == hipSuccess) er2 = hipEventSynchronize(e->ev_probe);
@@ -608,4 +630,74 @@ extern "C" int cswap_engine_calibrate(cswap_engine* e, cswap_costs* out_costs)
   if (d_tmp) (void)hipFree(d_tmp);
   if (!rc && out_costs) *out_costs = e->costs;
   return rc;
+}
+
+// ----------------------------------------------------------------- geometry tuning
+// The reference passes its launch geometry (dimsize x blocksize = chunk count)
+// through every ZVC entry point (CSWAP+/zfp/compression.cu:334-374) and always
+// uses 512 x 32.  Here the chunk count is a free parameter of the engine's own
+// payload layout, and the fastest one depends on the tensor size: this measures
+// count + scan + compact + expand for power-of-two chunk counts on a synthetic
+// half-zero tensor of n elements and remembers the winner for that size class.
+extern "C" int cswap_engine_tune(cswap_engine* e, size_t n, int* best_process)
+{
+  if (!e || n < 64 || n > 0x7fffffffull) return CSWAP_E_ARG;
+  std::lock_guard<std::mutex> lock(e->mu);
+  int rc = CSWAP_OK;
+  hipStream_t s = nullptr;
+  float *d_x = nullptr, *d_y = nullptr;
+  char* d_tmp = nullptr;
+  hipEvent_t a = nullptr, b = nullptr;
+  const int lo = 1024, hi = 65536;
+  int best = 0;
+  double best_ms = 0;
+  do {
+    hipError_t er;
+    const size_t hdr_max = zvc_header_bytes((int)n, hi) + zvc_header_bytes((int)n, lo);  // either extreme fits
+    if ((er = hipMalloc((void**)&d_x, 4 * n)) != hipSuccess || (er = hipMalloc((void**)&d_y, 4 * n)) != hipSuccess ||
+        (er = hipMalloc((void**)&d_tmp, hdr_max + 4 * n)) != hipSuccess ||
+        (er = hipEventCreate(&a)) != hipSuccess || (er = hipEventCreate(&b)) != hipSuccess) {
+      rc = hip_fail(er); break;
+    }
+    hipLaunchKernelGGL(fill_relu_like_kernel, dim3(1024), dim3(256), 0, s, d_x, n);
+    for (int proc = lo; proc <= hi && !rc; proc *= 2) {
+      if ((size_t)proc * 16 > n && proc > lo) break;  // fewer than 16 elements per chunk is never the answer
+      const size_t hdr = zvc_header_bytes((int)n, proc);
+      int* d_begin = (int*)d_tmp;
+      uint32_t* d_mask = (uint32_t*)(d_tmp + 4 * (size_t)proc);
+      float* d_vals = (float*)(d_tmp + hdr);
+      auto once = [&]() {
+        int r = cswap_zvc_compress(d_x, (int)n, proc, d_begin, e->d_nnz, d_vals, d_mask, s);
+        return r ? r : cswap_zvc_expand(d_vals, d_mask, d_begin, (int)n, proc, d_y, s);
+      };
+      if ((rc = once())) break;  // warm-up
+      const int reps = 5;
+      er = hipEventRecord(a, s);
+      for (int i = 0; i < reps && er == hipSuccess && !rc; i++) rc = once();
+      if (rc) break;
+      if (er == hipSuccess) er = hipEventRecord(b, s);
+      if (er == hipSuccess) er = hipEventSynchronize(b);
+      float t = 0;
+      if (er == hipSuccess) er = hipEventElapsedTime(&t, a, b);
+      if (er != hipSuccess) { rc = hip_fail(er); break; }
+      if (!best || t < best_ms) { best = proc; best_ms = t; }
+    }
+  } while (0);
+  (void)hipStreamSynchronize(s);
+  if (a) (void)hipEventDestroy(a);
+  if (b) (void)hipEventDestroy(b);
+  if (d_x) (void)hipFree(d_x);
+  if (d_y) (void)hipFree(d_y);
+  if (d_tmp) (void)hipFree(d_tmp);
+  if (rc) return rc;
+  e->tuned[size_class(n)] = best;
+  if (best_process) *best_process = best;
+  return CSWAP_OK;
+}
+
+extern "C" int cswap_engine_process_for(cswap_engine* e, size_t n)
+{
+  if (!e || !n) return 0;
+  std::lock_guard<std::mutex> lock(e->mu);
+  return process_for(e, n);
 }

@@ -42,7 +42,7 @@ def select_field(nx: int, ny: int, nz: int, nnz: int, maxbits: int = 512, costs:
 
 class SwapEngine:
     def __init__(self, pinned_bytes: int = 1 << 30, device_bytes: int = 1 << 30, maxbits: int = 512,
-                 process: int = 512 * 32, max_tickets: int = 256, costs: Costs | None = None):
+                 process: int = 0, max_tickets: int = 256, costs: Costs | None = None):
         cfg = EngineConfig()
         lib().cswap_engine_config_default(C.byref(cfg))
         cfg.pinned_pool_bytes = pinned_bytes
@@ -89,6 +89,16 @@ class SwapEngine:
         check(lib().cswap_swap_in(self._h, ticket, out.data_ptr(), torch.cuda.current_stream().cuda_stream),
               "cswap_swap_in")
         return out
+
+    def tune(self, numel: int) -> int:
+        """Measure the best ZVC chunk count for tensors of about ``numel`` elements
+        (used from then on when the engine was created with ``process=0``)."""
+        best = C.c_int(0)
+        check(lib().cswap_engine_tune(self._h, numel, C.byref(best)), "cswap_engine_tune")
+        return best.value
+
+    def process_for(self, numel: int) -> int:
+        return lib().cswap_engine_process_for(self._h, numel)
 
     def prefetch(self, ticket: int) -> None:
         """Start the host-to-device copy of a swapped tensor ahead of its swap_in."""

@@ -90,6 +90,10 @@ int    cswap_zvc_chunk_elems(int n, int process);   /* E */
 int    cswap_zvc_chunk_words(int n, int process);   /* W */
 int    cswap_zvc_active_chunks(int n, int process); /* chunks that hold data = ceil(n/E) */
 size_t cswap_zvc_mask_bytes(int n, int process);    /* W*process*4, Execution.h:88 */
+/* A good chunk count for n elements when the caller may choose (the reference
+ * always passes 512*32): about 1024 elements per chunk, a power of two in
+ * [1024, 16384].  Both directions must use the same value. */
+int    cswap_zvc_pick_process(size_t n);
 
 /* Replaces PreGPUcompression (zfp/compression.cu:134-165, launcher :334-341):
  * d_count[i] = number of elements != 0 in chunk i, for the active chunks. */
@@ -204,7 +208,7 @@ typedef struct cswap_engine cswap_engine;
 typedef struct {
   size_t pinned_pool_bytes;   /* host side: compressed tensors live here while swapped out */
   size_t device_pool_bytes;   /* device staging for compressed data in flight */
-  int    process;             /* ZVC chunk count; 0 = 16384 */
+  int    process;             /* ZVC chunk count; 0 = per tensor size (cswap_engine_tune result, else cswap_zvc_pick_process) */
   unsigned zfp_maxbits;       /* bits per 4x4x4 block for policy ZFP; 0 = 512 (8 bits/value) */
   int    max_tickets;         /* tensors that may be swapped out at once; 0 = 256 */
   cswap_costs costs;          /* used by CSWAP_POLICY_AUTO; zero bw fields = defaults */
@@ -249,6 +253,17 @@ int cswap_swap_info(cswap_engine* e, int ticket, cswap_ticket_info* info);
 /* Measure link bandwidth and kernel throughput on this box and store them in
  * the engine's cost model (allocates temporaries; call once after create). */
 int cswap_engine_calibrate(cswap_engine* e, cswap_costs* out_costs);
+/* Launch-geometry self-tuning.  The reference hands dimsize x blocksize (the
+ * chunk count) to every ZVC entry point and always uses 512 x 32
+ * (zfp/compression.cu:334-374).  With config.process == 0 the engine picks the
+ * chunk count per tensor: cswap_engine_tune(e, n, &best) times count + scan +
+ * compact + expand for power-of-two chunk counts on a synthetic tensor of n
+ * elements (allocates temporaries) and remembers the winner for tensors of that
+ * size class (same bit length of n); sizes never tuned use
+ * cswap_zvc_pick_process.  cswap_engine_process_for reports the chunk count the
+ * engine would use for a tensor of n elements. */
+int cswap_engine_tune(cswap_engine* e, size_t n, int* best_process);
+int cswap_engine_process_for(cswap_engine* e, size_t n);
 cswap_stream_t cswap_engine_copy_stream(cswap_engine* e);
 
 /* --------------------------------------------------------------- planner -----

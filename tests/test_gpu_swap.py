@@ -60,7 +60,7 @@ def test_round_trip_equals_codec_round_trip(torch_cuda, engine, policy_name):
         if pol == swap.SPARSE:
             nnz = np.count_nonzero(xn)
             assert info.nnz == nnz
-            assert info.bytes_out == 4 * nnz + xn.size // 8 + 4 * 16384
+            assert info.bytes_out == 4 * nnz + xn.size // 8 + 4 * engine.process_for(xn.size)
 
 
 def test_auto_policy_follows_selector(torch_cuda, engine):
@@ -191,6 +191,38 @@ def test_prefetched_ticket_can_be_released_unused(torch_cuda, engine):
     L = __import__("cswap_amd._lib", fromlist=["lib"]).lib()
     assert L.cswap_swap_prefetch(engine._h, tk) == -5       # released ticket
     assert L.cswap_swap_prefetch(engine._h, 10 ** 6) == -1  # no such ticket
+
+
+def test_chunk_count_follows_size_rule_tuning_and_configuration(torch_cuda):
+    """With process=0 the engine picks the ZVC chunk count per tensor: the size
+    rule first, the measured winner once cswap_engine_tune has run for that size
+    class; a configured chunk count overrides both.  Results stay bit-exact."""
+    torch = torch_cuda
+    from cswap_amd import swap
+    from cswap_amd._lib import lib
+
+    L = lib()
+    eng = swap.SwapEngine(pinned_bytes=256 << 20, device_bytes=256 << 20)
+    n = 3 * 1024 * 1024 + 17
+    x = relu_tensor(torch, (n,), 0.6, 5)
+    assert eng.process_for(n) == L.cswap_zvc_pick_process(n) == 2048
+    best = eng.tune(n)
+    assert best in (1024, 2048, 4096, 8192, 16384, 32768, 65536)
+    assert eng.process_for(n) == best and eng.process_for(n // 8) == L.cswap_zvc_pick_process(n // 8)
+    for e, want in ((eng, best), (swap.SwapEngine(pinned_bytes=64 << 20, device_bytes=64 << 20, process=16384), 16384)):
+        out = torch.full_like(x, -1.0)
+        tk = e.pre(x, swap.SPARSE)
+        e.post(tk)
+        info = e.info(tk)
+        E = -(-n // want)
+        assert info.bytes_out == 4 * int((x != 0).sum()) + 4 * want + 4 * want * (-(-E // 32))
+        e.swap_in(tk, out)
+        torch.cuda.synchronize()
+        e.release(tk)
+        assert torch.equal(out, x)
+        if e is not eng:
+            e.close()
+    eng.close()
 
 
 def test_state_machine_errors(torch_cuda, engine):

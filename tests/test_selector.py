@@ -119,3 +119,21 @@ def test_bad_arguments():
     assert lib().cswap_select(0, 0, 512, None, C.byref(ch)) == -1
     assert lib().cswap_select(10, 11, 512, None, C.byref(ch)) == -1
     assert lib().cswap_select(10, 1, 512, None, None) == -1
+
+
+def test_chunk_count_rule():
+    """About 1024 elements per chunk, a power of two between 1024 and 16384."""
+    from cswap_amd._lib import lib
+
+    L = lib()
+    assert L.cswap_zvc_pick_process(1) == 1024
+    assert L.cswap_zvc_pick_process(262144) == 1024          # 1 MiB
+    assert L.cswap_zvc_pick_process(4 << 20) == 4096         # 16 MiB
+    assert L.cswap_zvc_pick_process(8 << 20) == 8192         # 32 MiB
+    assert L.cswap_zvc_pick_process(64 << 20) == 16384       # 256 MiB
+    assert L.cswap_zvc_pick_process(2**31 - 1) == 16384
+    prev = 0
+    for k in range(10, 31):
+        p = L.cswap_zvc_pick_process(1 << k)
+        assert p >= prev and p & (p - 1) == 0 and 1024 <= p <= 16384
+        prev = p
