@@ -135,6 +135,65 @@ def test_strided_field(torch_cuda):
     assert np.all(o == -7.0)   # nothing outside the field was touched
 
 
+@pytest.mark.parametrize("case", ["padded_rows_and_planes", "one_block_per_slab", "slab_crossing", "planes_before_rows",
+                                  "big_offsets"])
+def test_aligned_strided_fields(torch_cuda, case):
+    """Fields embedded in larger allocations with 16-byte aligned rows: these take
+    the 16-byte row path with a wave-uniform base and 32-bit lane offsets (a
+    wavefront's 64 blocks may span many slabs of four planes), except when the
+    strides do not nest (planes closer together than rows), which must fall back
+    to the element path.  Either way the stream equals that of the contiguous copy
+    and nothing outside the field is written."""
+    torch = torch_cuda
+    import oracle
+    from cswap_amd._lib import check, lib
+
+    rng = np.random.default_rng(abs(hash(case)) % 2**32)
+    if case == "padded_rows_and_planes":
+        alloc, sl = (14, 12, 24), (slice(1, 13), slice(4, 12), slice(4, 20))       # (12, 8, 16) inside
+    elif case == "one_block_per_slab":
+        alloc, sl = (400, 4, 8), (slice(0, 400), slice(0, 4), slice(4, 8))         # nx = ny = 4: 64 blocks = 64 slabs
+    elif case == "slab_crossing":
+        alloc, sl = (24, 20, 28), (slice(0, 24), slice(0, 20), slice(0, 28))       # 35 blocks per slab, contiguous
+    elif case == "big_offsets":
+        alloc, sl = (40, 260, 1028), (slice(4, 36), slice(0, 256), slice(4, 1028))  # 40 MB allocation
+    else:
+        alloc, sl = None, None
+    if case == "planes_before_rows":
+        # memory order (y, z, x): sy = 8*16, sz = 16  -> planes are closer together than rows
+        big = rng.standard_normal((8, 8, 16)).astype(np.float32)                   # [y][z][x]
+        sub = np.ascontiguousarray(big.transpose(1, 0, 2))                         # field [z][y][x]
+        nz, ny, nx = sub.shape
+        sx, sy, sz, off = 1, 8 * 16, 16, 0
+    else:
+        big = rng.standard_normal(alloc).astype(np.float32)
+        sub = np.ascontiguousarray(big[sl])
+        nz, ny, nx = sub.shape
+        sx, sy, sz = 1, alloc[2], alloc[1] * alloc[2]
+        off = sl[0].start * sz + sl[1].start * sy + sl[2].start
+    tb = torch.from_numpy(big).cuda()
+    assert (tb.data_ptr() + 4 * off) % 16 == 0
+    cap = lib().cswap_zfp_stream_capacity(nx, ny, nz, 512)
+    s = torch.zeros(cap, dtype=torch.uint8, device="cuda")
+    check(lib().cswap_zfp_compress_f32(tb.data_ptr() + 4 * off, nx, ny, nz, sx, sy, sz, 512, s.data_ptr(), None),
+          "compress")
+    torch.cuda.synchronize()
+    want = oracle.zfp_encode3(sub, 512, omp=True)
+    assert np.array_equal(s.cpu().numpy().view(np.uint64), want)
+    out = torch.full(big.shape, -7.0, dtype=torch.float32, device="cuda")
+    check(lib().cswap_zfp_decompress_f32(s.data_ptr(), nx, ny, nz, sx, sy, sz, 512, out.data_ptr() + 4 * off, None),
+          "decompress")
+    torch.cuda.synchronize()
+    o = out.cpu().numpy()
+    dec = oracle.zfp_decode3(want, sub.shape, 512, omp=True)
+    if case == "planes_before_rows":
+        assert np.array_equal(o.transpose(1, 0, 2).view(np.uint32), dec.view(np.uint32))
+    else:
+        assert np.array_equal(o[sl].view(np.uint32), dec.view(np.uint32))
+        o[sl] = -7.0
+        assert np.all(o == -7.0)   # nothing outside the field was touched
+
+
 def test_large_tensor_properties(torch_cuda):
     """At full size (402 MB softmax-shaped tensor) the checker is too slow, so
     use properties that hold at any size: (a) a sampled slab equals the checker,
