@@ -95,7 +95,7 @@ def test_ragged_shapes_and_odd_rates(torch_cuda, shape, maxbits):
     import oracle
     from cswap_amd import api
 
-    rng = np.random.default_rng(hash((shape, maxbits)) % 2**32)
+    rng = np.random.default_rng(sum(shape) * 4099 + maxbits)
     f = (rng.standard_normal(shape) * 10.0 ** rng.integers(-3, 4)).astype(np.float32)
     s = gpu_encode(torch, f, maxbits)
     want = oracle.zfp_encode3(f, maxbits)
@@ -148,7 +148,7 @@ def test_aligned_strided_fields(torch_cuda, case):
     import oracle
     from cswap_amd._lib import check, lib
 
-    rng = np.random.default_rng(abs(hash(case)) % 2**32)
+    rng = np.random.default_rng(sum(map(ord, case)))
     if case == "padded_rows_and_planes":
         alloc, sl = (14, 12, 24), (slice(1, 13), slice(4, 12), slice(4, 20))       # (12, 8, 16) inside
     elif case == "one_block_per_slab":
