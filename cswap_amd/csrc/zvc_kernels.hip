@@ -41,6 +41,7 @@ struct Geometry {
   int W;        // mask words per chunk
   int process;  // chunks in the layout
   int active;   // chunks that hold data
+  int backwards;  // compaction order, see zvc_compact_kernel
 };
 
 // ------------------------------------------------------------------ count
@@ -141,8 +142,14 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_compact_kernel(
     const float* __restrict__ in, Geometry g, const int* __restrict__ begin, float* __restrict__ values,
     uint32_t* __restrict__ mask)
 {
-  const int c = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
+  // Tensors larger than the memory-side cache are walked from the last chunk
+  // to the first: the counting pass that ran just before went first to last, so
+  // the chunks it touched last are the ones still cached (measured: count + scan
+  // + compact 6-7 % faster at 256 and 512 MiB; smaller tensors stay cached
+  // either way and are walked forwards).
+  int c = (int)(blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6));
   if (c >= g.process) return;
+  if (g.backwards) c = g.process - 1 - c;
   const unsigned lane = lane_id();
   uint32_t* mrow = mask + (size_t)c * g.W;
   if (c >= g.active) {  // chunk without data: the reference leaves these words untouched; define them
@@ -506,6 +513,7 @@ static int make_geometry(Geometry& g, int n, int process)
   g.E = n / process + (n % process != 0);
   g.W = g.E / 32 + (g.E % 32 != 0);
   g.active = n / g.E + (n % g.E != 0);
+  g.backwards = n > (48 << 20);  // more than 192 MB of fp32
   return CSWAP_OK;
 }
 
