@@ -393,3 +393,34 @@ def test_simple_c_harness(torch_cuda):
     want = oracle.zfp_encode3(ori, maxbits, omp=True)
     assert np.array_equal(buf.view(np.uint64), want)
     assert np.array_equal(a.view(np.uint32), oracle.zfp_decode3(want, ori.shape, maxbits, omp=True).view(np.uint32))
+
+
+def test_reference_harness_binary_runs_against_this_library(torch_cuda):
+    """oracle/_ref/simple_harness is the reference's own command-line harness
+    (CSWAP+/simple.c with CSWAP+/zfp/zfp.c), compiled unmodified and linked
+    against libcswap_hip.so in place of the reference's CUDA library: host arrays
+    of 2560 x 512 x 50 floats through zfp_stream_set_accuracy + cuda_compress +
+    cuda_decompress.  The binary is built where the reference tree is present
+    and travels with the tree; without it there is nothing to run."""
+    import os
+    import re
+    import subprocess
+
+    from conftest import ROOT
+
+    exe = os.path.join(ROOT, "oracle", "_ref", "simple_harness")
+    if not os.path.exists(exe):
+        pytest.skip("oracle/_ref/simple_harness was not built (no reference tree at build time)")
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=110)
+    print(out.stdout, out.stderr, flush=True)
+    assert out.returncode == 0
+    n = 2560 * 512 * 50
+    assert "All tensor size =  250 MB" in out.stdout
+    size_mb = float(re.search(r"zfpsize : ([0-9.]+) MB", out.stdout).group(1))
+    # the harness asks for accuracy mode; the reference's CUDA path only reads maxbits from the stream
+    # (cuZFP.cu:105-151), so the size is blocks x maxbits
+    assert 0 < size_mb < 4.0 * n / 2**20 * 1.1
+    cnt = int(re.search(r"error cnt:(\d+)", out.stdout).group(1))
+    assert 0 <= cnt <= n
+    loss = float(re.search(r"Final accuray loss is -> ([0-9.eE+-]+)", out.stdout).group(1))
+    assert loss < 0.05
