@@ -26,7 +26,7 @@ vp, sz, pd, u, i32 = C.c_void_p, C.c_size_t, C.c_ssize_t, C.c_uint, C.c_int
 
 class Costs(C.Structure):
     _fields_ = [("bw_d2h_gbs", C.c_double), ("bw_h2d_gbs", C.c_double), ("copy_latency_us", C.c_double),
-                ("kernel_latency_us", C.c_double), ("zvc_compress_gbs", C.c_double),
+                ("kernel_latency_us", C.c_double), ("zfp_latency_us", C.c_double), ("zvc_compress_gbs", C.c_double),
                 ("zvc_expand_gbs", C.c_double), ("zfp_compress_gbs", C.c_double),
                 ("zfp_decompress_gbs", C.c_double), ("sparse_max_ratio", C.c_double), ("lossy_min_gain", C.c_double),
                 ("probe_latency_us", C.c_double), ("probe_gbs", C.c_double), ("min_gain", C.c_double),

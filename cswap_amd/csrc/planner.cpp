@@ -82,8 +82,8 @@ static Option price(const cswap_planner* p, const TensorRec& r, int policy)
   } else {
     o.bytes_out = r.nx ? cswap_zfp_stream_capacity(r.nx, r.ny, r.nz, p->maxbits)
                        : cswap_policy_bytes(CSWAP_POLICY_ZFP, n, 0, p->maxbits, 0, 0, 0, 0);
-    t_comp = c.kernel_latency_us + in_bytes / (c.zfp_compress_gbs * 1e3);
-    t_decomp = c.kernel_latency_us + in_bytes / (c.zfp_decompress_gbs * 1e3);
+    t_comp = c.zfp_latency_us + in_bytes / (c.zfp_compress_gbs * 1e3);
+    t_decomp = c.zfp_latency_us + in_bytes / (c.zfp_decompress_gbs * 1e3);
   }
   const double t_out = c.copy_latency_us + (double)o.bytes_out / (c.bw_d2h_gbs * 1e3);
   const double t_in = c.copy_latency_us + (double)o.bytes_out / (c.bw_h2d_gbs * 1e3);

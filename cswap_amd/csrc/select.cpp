@@ -17,6 +17,7 @@ extern "C" void cswap_costs_default(cswap_costs* c)
   c->bw_h2d_gbs = 50.0;
   c->copy_latency_us = 10.0;
   c->kernel_latency_us = 4.0;
+  c->zfp_latency_us = 11.0;
   c->zvc_compress_gbs = 1400.0;   // fp32 bytes in / (count + scan + compact)
   c->zvc_expand_gbs = 1500.0;
   c->zfp_compress_gbs = 2100.0;
@@ -82,7 +83,7 @@ static int select_core(size_t n, size_t nnz, size_t b_zfp, const cswap_costs* co
   }
   if (c.allow_lossy && b_zfp && c.zfp_compress_gbs > 0 && c.zfp_decompress_gbs > 0) {
     if ((double)b_zfp < in_bytes)
-      t_zfp = t_probe + 2.0 * c.kernel_latency_us + in_bytes / (c.zfp_compress_gbs * 1e3) +
+      t_zfp = t_probe + 2.0 * c.zfp_latency_us + in_bytes / (c.zfp_compress_gbs * 1e3) +
               in_bytes / (c.zfp_decompress_gbs * 1e3) + link_us((double)b_zfp);
   }
 

@@ -596,6 +596,16 @@ extern "C" int cswap_engine_calibrate(cswap_engine* e, cswap_costs* out_costs)
     if ((rc = ms(fdc, 2, &t))) break;
     if ((rc = ms(fdc, 10, &t))) break;
     c.zfp_decompress_gbs = gb / (t * 1e-3);
+    {  // fixed cost of a ZFP kernel: a field of one wavefront per SIMD at most (64 x 64 x 16 = 1024 blocks)
+      double tc = 0, td = 0;
+      auto sc = [&]() { return cswap_zfp_compress_f32(d_x, 64, 64, 16, 0, 0, 0, e->maxbits, (uint64_t*)d_tmp, s); };
+      auto sd = [&]() { return cswap_zfp_decompress_f32((const uint64_t*)d_tmp, 64, 64, 16, 0, 0, 0, e->maxbits, d_y, s); };
+      if ((rc = ms(sc, 2, &tc))) break;
+      if ((rc = ms(sc, 20, &tc))) break;
+      if ((rc = ms(sd, 2, &td))) break;
+      if ((rc = ms(sd, 20, &td))) break;
+      c.zfp_latency_us = 0.5 * (tc + td) * 1e3;
+    }
     // the probe: counting pass throughput, and the fixed cost of count + scan +
     // 4-byte copy + host wait measured on a tensor too small to matter
     auto cnt = [&]() { return cswap_zvc_count(d_x, (int)n, proc, d_begin, s); };

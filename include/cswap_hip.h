@@ -160,7 +160,9 @@ typedef enum { CSWAP_POLICY_AUTO = -1, CSWAP_POLICY_NONE = 2, CSWAP_POLICY_SPARS
 typedef struct {
   double bw_d2h_gbs, bw_h2d_gbs;         /* pinned host link, GB/s */
   double copy_latency_us;                /* fixed cost of one async copy */
-  double kernel_latency_us;              /* fixed cost of one kernel */
+  double kernel_latency_us;              /* fixed cost of one ZVC kernel */
+  double zfp_latency_us;                 /* fixed cost of one ZFP kernel: a lone wavefront's serial work, which a
+                                            tensor too small to fill the chip cannot go below */
   double zvc_compress_gbs, zvc_expand_gbs; /* GB/s of fp32 in / out */
   double zfp_compress_gbs, zfp_decompress_gbs;
   double sparse_max_ratio;               /* ZVC eligible only below this size ratio */

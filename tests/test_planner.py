@@ -18,6 +18,7 @@ def costs(**kw):
     c.bw_d2h_gbs = c.bw_h2d_gbs = 50.0
     c.copy_latency_us = 10.0
     c.kernel_latency_us = 4.0
+    c.zfp_latency_us = 4.0
     c.size_floor_bytes = 0
     for k, v in kw.items():
         setattr(c, k, v)
