@@ -37,27 +37,44 @@ def zfp_stream_capacity(nx: int, ny: int, nz: int, maxbits: int) -> int:
 def cuda_compress(t: torch.Tensor, maxbits: int, out: torch.Tensor | None = None) -> torch.Tensor:
     """Fixed-rate ZFP of ``t`` viewed as the field (nx=last dim, ny=second to
     last, nz=rest).  Returns the stream as a uint8 device tensor."""
-    _need_f32_cuda(t)
+    is_int = t.dtype == torch.int32          # zfp_type_int32; every other dtype but fp32 is refused
+    if not is_int:
+        _need_f32_cuda(t)
+    elif not (t.is_cuda and t.is_contiguous()):
+        raise TypeError("expected a contiguous int32 CUDA tensor")
     nx, ny, nz = field_dims(t.shape)
     cap = zfp_stream_capacity(nx, ny, nz, maxbits)
     if out is None:
         out = torch.empty(cap, dtype=torch.uint8, device=t.device)
     elif out.numel() * out.element_size() < cap:
         raise ValueError("stream buffer too small")
-    check(lib().cswap_zfp_compress_f32(t.data_ptr(), nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(), _stream()),
-          "cswap_zfp_compress_f32")
+    if is_int:
+        check(lib().cswap_zfp_compress_i32_nd(t.data_ptr(), 3, nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(),
+                                              _stream()), "cswap_zfp_compress_i32_nd")
+    else:
+        check(lib().cswap_zfp_compress_f32(t.data_ptr(), nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(), _stream()),
+              "cswap_zfp_compress_f32")
     return out
 
 
-def cuda_decompress(stream: torch.Tensor, shape, maxbits: int, out: torch.Tensor | None = None) -> torch.Tensor:
+def cuda_decompress(stream: torch.Tensor, shape, maxbits: int, out: torch.Tensor | None = None,
+                    dtype=torch.float32) -> torch.Tensor:
     nx, ny, nz = field_dims(shape)
     if out is None:
-        out = torch.empty(tuple(shape), dtype=torch.float32, device=stream.device)
-    _need_f32_cuda(out)
+        out = torch.empty(tuple(shape), dtype=dtype, device=stream.device)
+    is_int = out.dtype == torch.int32
+    if not is_int:
+        _need_f32_cuda(out)
+    elif not (out.is_cuda and out.is_contiguous()):
+        raise TypeError("expected a contiguous int32 CUDA tensor")
     if stream.numel() * stream.element_size() < zfp_stream_capacity(nx, ny, nz, maxbits):
         raise ValueError("stream buffer too small")
-    check(lib().cswap_zfp_decompress_f32(stream.data_ptr(), nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(),
-                                         _stream()), "cswap_zfp_decompress_f32")
+    if is_int:
+        check(lib().cswap_zfp_decompress_i32_nd(stream.data_ptr(), 3, nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(),
+                                                _stream()), "cswap_zfp_decompress_i32_nd")
+    else:
+        check(lib().cswap_zfp_decompress_f32(stream.data_ptr(), nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(),
+                                             _stream()), "cswap_zfp_decompress_f32")
     return out
 
 

@@ -104,7 +104,10 @@ size_t cuda_compress(cswap_zfp_stream* zs, const cswap_zfp_field* f)
 {
   if (!zs || !f || !zs->stream || !f->data || !zs->stream->begin) return 0;
   const int dims = field_dims_of(f);
-  if (f->type != 3 || !dims) return 0;  // float fields of 1, 2 or 3 dimensions
+  // fields of 1, 2 or 3 dimensions of float (zfp_type_float = 3) or int32 (zfp_type_int32 = 1);
+  // the 64-bit scalar types the reference also dispatches on (cuZFP.cu:400-422) are not implemented
+  if ((f->type != 3 && f->type != 1) || !dims) return 0;
+  const bool is_int = f->type == 1;
   const unsigned maxbits = zs->maxbits;
   const size_t cap = cswap_zfp_stream_capacity_nd(dims, f->nx, f->ny, f->nz, maxbits);
   const size_t bytes = cswap_zfp_stream_bytes_nd(dims, f->nx, f->ny, f->nz, maxbits);
@@ -125,8 +128,10 @@ size_t cuda_compress(cswap_zfp_stream* zs, const cswap_zfp_field* f)
       if (hipMalloc(&tmp_s, cap) != hipSuccess) break;
       d_stream = (uint64_t*)tmp_s;
     }
-    if (cswap_zfp_compress_f32_nd(d_in, dims, f->nx, f->ny, f->nz, field_dev ? f->sx : 0, field_dev ? f->sy : 0,
-                                  field_dev ? f->sz : 0, maxbits, d_stream, nullptr))
+    const ptrdiff_t sx = field_dev ? f->sx : 0, sy = field_dev ? f->sy : 0, sz = field_dev ? f->sz : 0;
+    if (is_int ? cswap_zfp_compress_i32_nd((const int32_t*)d_in, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits,
+                                           d_stream, nullptr)
+               : cswap_zfp_compress_f32_nd(d_in, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits, d_stream, nullptr))
       break;
     if (!stream_dev) {
       if (hipMemcpy(zs->stream->begin, tmp_s, cap, hipMemcpyDeviceToHost) != hipSuccess) break;
@@ -148,7 +153,8 @@ void cuda_decompress(cswap_zfp_stream* zs, cswap_zfp_field* f)
 {
   if (!zs || !f || !zs->stream || !f->data || !zs->stream->begin) return;
   const int dims = field_dims_of(f);
-  if (f->type != 3 || !dims) return;
+  if ((f->type != 3 && f->type != 1) || !dims) return;
+  const bool is_int = f->type == 1;
   const unsigned maxbits = zs->maxbits;
   const size_t cap = cswap_zfp_stream_capacity_nd(dims, f->nx, f->ny, f->nz, maxbits);
   const size_t bytes = cswap_zfp_stream_bytes_nd(dims, f->nx, f->ny, f->nz, maxbits);
@@ -169,8 +175,10 @@ void cuda_decompress(cswap_zfp_stream* zs, cswap_zfp_field* f)
       if (hipMemcpy(tmp_s, zs->stream->begin, cap, hipMemcpyHostToDevice) != hipSuccess) break;
       d_stream = (const uint64_t*)tmp_s;
     }
-    if (cswap_zfp_decompress_f32_nd(d_stream, dims, f->nx, f->ny, f->nz, field_dev ? f->sx : 0,
-                                    field_dev ? f->sy : 0, field_dev ? f->sz : 0, maxbits, d_out, nullptr))
+    const ptrdiff_t sx = field_dev ? f->sx : 0, sy = field_dev ? f->sy : 0, sz = field_dev ? f->sz : 0;
+    if (is_int ? cswap_zfp_decompress_i32_nd(d_stream, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits,
+                                             (int32_t*)d_out, nullptr)
+               : cswap_zfp_decompress_f32_nd(d_stream, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits, d_out, nullptr))
       break;
     if (!field_dev) {
       if (hipMemcpy(f->data, tmp_out, fb, hipMemcpyDeviceToHost) != hipSuccess) break;

@@ -416,21 +416,11 @@ struct BlockEncoder {
   }
 };
 
-// Full block encode: f[x + 4y + 16z] (already padded for partial blocks).
-template <bool GUARD, class Mem>
-CSWAP_HD void encode_block(const float (&f)[64], unsigned pos0, unsigned maxbits, Mem& mem)
+// Integer back end of a 4x4x4 block: transform, reorder, bit planes, coder
+// (encode.cuh:306-345 with the callers at :347-380).  ib is overwritten.
+template <class Enc>
+CSWAP_HD void encode_ints3(int32_t (&ib)[64], Enc& enc)
 {
-  uint32_t e = block_header_e(f);
-  if (e == 0) return;  // all-zero block: every bit stays 0 (encode.cuh:357-358)
-  BlockEncoder<Mem, GUARD> enc(mem, pos0, maxbits);
-  enc.put(2 * e + 1, 9);
-
-  // block-floating-point cast: scale 2^(30-emax) as a float, truncate
-  float s = pow2f(30 - ((int)e - 127));
-  int32_t ib[64];
-#pragma unroll
-  for (int i = 0; i < 64; i++) ib[i] = (int32_t)(s * f[i]);
-
   fwd_xform3(ib);
 
   uint32_t lo[32], hi[32];
@@ -453,6 +443,32 @@ CSWAP_HD void encode_block(const float (&f)[64], unsigned pos0, unsigned maxbits
 #pragma unroll
     for (int k = 15; k >= 0; k--) enc.plane(((uint64_t)hi[k] << 32) | lo[k]);
   }
+}
+
+// Full block encode: f[x + 4y + 16z] (already padded for partial blocks).
+template <bool GUARD, class Mem>
+CSWAP_HD void encode_block(const float (&f)[64], unsigned pos0, unsigned maxbits, Mem& mem)
+{
+  uint32_t e = block_header_e(f);
+  if (e == 0) return;  // all-zero block: every bit stays 0 (encode.cuh:357-358)
+  BlockEncoder<Mem, GUARD> enc(mem, pos0, maxbits);
+  enc.put(2 * e + 1, 9);
+
+  // block-floating-point cast: scale 2^(30-emax) as a float, truncate
+  float s = pow2f(30 - ((int)e - 127));
+  int32_t ib[64];
+#pragma unroll
+  for (int i = 0; i < 64; i++) ib[i] = (int32_t)(s * f[i]);
+  encode_ints3(ib, enc);
+}
+
+// int32 block (zfp_type_int32): no header, no cast, the whole budget for the
+// coder (encode.cuh:371-380).  ib is overwritten.
+template <bool GUARD, class Mem>
+CSWAP_HD void encode_block_i32(int32_t (&ib)[64], unsigned pos0, unsigned maxbits, Mem& mem)
+{
+  BlockEncoder<Mem, GUARD> enc(mem, pos0, maxbits);
+  encode_ints3(ib, enc);
 }
 
 // ---------------------------------------------------------------- decoder
@@ -518,20 +534,11 @@ struct BlockDecoder {
 //                    and y; leaves ib[x + 4y + 16z] and the scale w
 //   decode_row       inverse lifting along x of one row and the cast to float
 // An empty block gives ib = 0 and w = 0, i.e. +0.0 everywhere.
-template <bool FENCED = false, class Mem>
-CSWAP_HD void decode_block_zy(Mem& mem, unsigned pos0, unsigned maxbits, int32_t (&ib)[64], float& w)
+// Integer back end of a 4x4x4 block up to and including the inverse lifting
+// along z and y (decode.cuh:127-179 and the first two passes of :181-226).
+template <class Dec>
+CSWAP_HD void decode_ints3_zy(Dec& dec, int32_t (&ib)[64])
 {
-  BlockDecoder<Mem, 64, FENCED> dec(mem, pos0, maxbits);
-  uint32_t h = (uint32_t)dec.window(pos0);
-  if (!(h & 1)) {
-#pragma unroll
-    for (int i = 0; i < 64; i++) ib[i] = 0;
-    w = 0.0f;
-    return;
-  }
-  int emax = (int)((h >> 1) & 0xff) - 127;
-  dec.pos = pos0 + 9;
-
   uint32_t lo[32], hi[32];
 #pragma unroll
   for (int k = 31; k >= 16; k--) {  // planes that no block of the wavefront can reach are zero without a read
@@ -568,7 +575,39 @@ CSWAP_HD void decode_block_zy(Mem& mem, unsigned pos0, unsigned maxbits, int32_t
     ib[kPerm3.v[32 + i]] = (int32_t)(hi[i] - c);
   }
   inv_xform3_zy(ib);
+}
+
+template <bool FENCED = false, class Mem>
+CSWAP_HD void decode_block_zy(Mem& mem, unsigned pos0, unsigned maxbits, int32_t (&ib)[64], float& w)
+{
+  BlockDecoder<Mem, 64, FENCED> dec(mem, pos0, maxbits);
+  uint32_t h = (uint32_t)dec.window(pos0);
+  if (!(h & 1)) {
+#pragma unroll
+    for (int i = 0; i < 64; i++) ib[i] = 0;
+    w = 0.0f;
+    return;
+  }
+  int emax = (int)((h >> 1) & 0xff) - 127;
+  dec.pos = pos0 + 9;
+  decode_ints3_zy(dec, ib);
   w = pow2f(emax - 30);
+}
+
+// int32 block (zfp_type_int32): no header; finish each x-row with inv_lift4
+template <bool FENCED = false, class Mem>
+CSWAP_HD void decode_block_i32_zy(Mem& mem, unsigned pos0, unsigned maxbits, int32_t (&ib)[64])
+{
+  BlockDecoder<Mem, 64, FENCED> dec(mem, pos0, maxbits);
+  decode_ints3_zy(dec, ib);
+}
+
+template <bool FENCED = false, class Mem>
+CSWAP_HD void decode_block_i32(Mem& mem, unsigned pos0, unsigned maxbits, int32_t (&ib)[64])
+{
+  decode_block_i32_zy<FENCED>(mem, pos0, maxbits, ib);
+#pragma unroll
+  for (int row = 0; row < 16; row++) inv_lift4(ib[4 * row], ib[4 * row + 1], ib[4 * row + 2], ib[4 * row + 3]);
 }
 
 // row = y + 4z; f receives the four values of that x-row
@@ -609,22 +648,28 @@ constexpr Perm2 kPerm2 = {{CSWAP_P2(0,0), CSWAP_P2(1,0), CSWAP_P2(0,1), CSWAP_P2
                            CSWAP_P2(2,1), CSWAP_P2(1,2), CSWAP_P2(3,0), CSWAP_P2(0,3), CSWAP_P2(2,2), CSWAP_P2(3,1),
                            CSWAP_P2(1,3), CSWAP_P2(3,2), CSWAP_P2(2,3), CSWAP_P2(3,3)}};
 
-template <int DIMS, bool GUARD, class Mem>
+// INT: f holds the bit patterns of int32 values (zfp_type_int32: no header, no cast)
+template <int DIMS, bool GUARD, bool INT = false, class Mem>
 CSWAP_HD void encode_block_low(const float (&f)[16], unsigned pos0, unsigned maxbits, Mem& mem)
 {
   constexpr int SIZE = DIMS == 2 ? 16 : 4;
-  float m = 0.0f;
-#pragma unroll
-  for (int i = 0; i < SIZE; i++) m = fmaxf(m, fabsf(f[i]));
-  uint32_t mb = f32_bits(m);
-  uint32_t e = mb ? (mb >> 23) + 1 : 0;
-  if (e == 0) return;
   BlockEncoder<Mem, GUARD, SIZE> enc(mem, pos0, maxbits);
-  enc.put(2 * e + 1, 9);
-  float s = pow2f(30 - ((int)e - 127));
   int32_t ib[16];
+  if (INT) {
 #pragma unroll
-  for (int i = 0; i < SIZE; i++) ib[i] = (int32_t)(s * f[i]);
+    for (int i = 0; i < SIZE; i++) ib[i] = (int32_t)f32_bits(f[i]);
+  } else {
+    float m = 0.0f;
+#pragma unroll
+    for (int i = 0; i < SIZE; i++) m = fmaxf(m, fabsf(f[i]));
+    uint32_t mb = f32_bits(m);
+    uint32_t e = mb ? (mb >> 23) + 1 : 0;
+    if (e == 0) return;
+    enc.put(2 * e + 1, 9);
+    float s = pow2f(30 - ((int)e - 127));
+#pragma unroll
+    for (int i = 0; i < SIZE; i++) ib[i] = (int32_t)(s * f[i]);
+  }
   uint32_t a[32];
 #pragma unroll
   for (int i = 0; i < 32; i++) a[i] = 0;
@@ -645,19 +690,22 @@ CSWAP_HD void encode_block_low(const float (&f)[16], unsigned pos0, unsigned max
   for (int k = 31; k >= 0; k--) enc.plane((uint64_t)a[k]);
 }
 
-template <int DIMS, class Mem>
+template <int DIMS, bool INT = false, class Mem>
 CSWAP_HD void decode_block_low(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)[16])
 {
   constexpr int SIZE = DIMS == 2 ? 16 : 4;
   BlockDecoder<Mem, SIZE> dec(mem, pos0, maxbits);
-  uint32_t h = (uint32_t)dec.window(pos0);
-  if (!(h & 1)) {
+  int emax = 0;
+  if (!INT) {
+    uint32_t h = (uint32_t)dec.window(pos0);
+    if (!(h & 1)) {
 #pragma unroll
-    for (int i = 0; i < 16; i++) f[i] = 0.0f;
-    return;
+      for (int i = 0; i < 16; i++) f[i] = 0.0f;
+      return;
+    }
+    emax = (int)((h >> 1) & 0xff) - 127;
+    dec.pos = pos0 + 9;
   }
-  int emax = (int)((h >> 1) & 0xff) - 127;
-  dec.pos = pos0 + 9;
   uint32_t a[32];
 #pragma unroll
   for (int k = 31; k >= 0; k--) a[k] = (uint32_t)dec.plane();
@@ -675,9 +723,14 @@ CSWAP_HD void decode_block_low(Mem& mem, unsigned pos0, unsigned maxbits, float 
     for (int i = 0; i < 4; i++) ib[i] = nb2int(a[i]);
     inv_lift4(ib[0], ib[1], ib[2], ib[3]);
   }
-  float w = pow2f(emax - 30);
+  if (INT) {
 #pragma unroll
-  for (int i = 0; i < SIZE; i++) f[i] = w * (float)ib[i];
+    for (int i = 0; i < SIZE; i++) f[i] = f32_from_bits((uint32_t)ib[i]);
+  } else {
+    float w = pow2f(emax - 30);
+#pragma unroll
+    for (int i = 0; i < SIZE; i++) f[i] = w * (float)ib[i];
+  }
 #pragma unroll
   for (int i = SIZE; i < 16; i++) f[i] = 0.0f;
 }

@@ -127,6 +127,15 @@ __device__ __forceinline__ void load_block(const float* __restrict__ in, const F
 // Finishes the block (inverse lifting along x, cast) and stores it.  On the
 // fast path every x-row is finished and stored on its own, so the finished
 // values never all sit in registers at once.
+// one x-row of an int32 block: last lifting pass, values handed on as bit patterns
+__device__ __forceinline__ void decode_row_i32(int32_t (&ib)[64], int row, float (&f)[4])
+{
+  inv_lift4(ib[4 * row], ib[4 * row + 1], ib[4 * row + 2], ib[4 * row + 3]);
+#pragma unroll
+  for (int x = 0; x < 4; x++) f[x] = __int_as_float(ib[4 * row + x]);
+}
+
+template <bool INT>
 __device__ __forceinline__ void finish_and_store_block(float* __restrict__ out, const Field3& fd, uint32_t first,
                                                        uint32_t b, int32_t (&ib)[64], float w)
 {
@@ -143,7 +152,8 @@ __device__ __forceinline__ void finish_and_store_block(float* __restrict__ out, 
 #pragma unroll
       for (int y = 0; y < 4; y++) {
         float r[4];
-        decode_row(ib, y + 4 * z, w, r);
+        if (INT) decode_row_i32(ib, y + 4 * z, r);
+        else decode_row(ib, y + 4 * z, w, r);
         *reinterpret_cast<float4*>(base + (size_t)(mine + (y * sy4 + z * sz4))) = make_float4(r[0], r[1], r[2], r[3]);
       }
   } else {
@@ -153,7 +163,8 @@ __device__ __forceinline__ void finish_and_store_block(float* __restrict__ out, 
 #pragma unroll
       for (int y = 0; y < 4; y++) {
         float r[4];
-        decode_row(ib, y + 4 * z, w, r);
+        if (INT) decode_row_i32(ib, y + 4 * z, r);
+        else decode_row(ib, y + 4 * z, w, r);
 #pragma unroll
         for (int x = 0; x < 4; x++)
           if ((uint32_t)x < bx && (uint32_t)y < by && (uint32_t)z < bz) p[x * fd.sx + y * fd.sy + z * fd.sz] = r[x];
@@ -164,7 +175,8 @@ __device__ __forceinline__ void finish_and_store_block(float* __restrict__ out, 
 // ------------------------------------------------------------- kernels
 // grid.x = ceil(nblocks/64) workgroups of one wavefront; dynamic LDS =
 // region_dwords(maxbits) dwords.
-template <bool WHOLE>
+// INT: the field holds int32 values (moved as 32-bit patterns through the same loads and stores)
+template <bool WHOLE, bool INT = false>
 __global__ __launch_bounds__(64) void zfp_encode3_f32_kernel(const float* __restrict__ in, Field3 fd,
                                                              unsigned maxbits,
                                                              uint64_t* __restrict__ stream)
@@ -187,7 +199,14 @@ __global__ __launch_bounds__(64) void zfp_encode3_f32_kernel(const float* __rest
     float f[64];
     load_block(in, fd, first, first + lane, f);
     LdsBits mem{lds};
-    encode_block<!WHOLE>(f, lane * slot, maxbits, mem);
+    if (INT) {
+      int32_t v[64];
+#pragma unroll
+      for (int i = 0; i < 64; i++) v[i] = __float_as_int(f[i]);
+      encode_block_i32<!WHOLE>(v, lane * slot, maxbits, mem);
+    } else {
+      encode_block<!WHOLE>(f, lane * slot, maxbits, mem);
+    }
   }
   __syncthreads();
 
@@ -215,7 +234,7 @@ __global__ __launch_bounds__(64) void zfp_encode3_f32_kernel(const float* __rest
 // Five wavefronts per SIMD (96 registers, five of them spilled around the
 // store phase): measured 2.5 % faster than the four that 105 registers allow;
 // six (80 registers, 20 spills) is slower again.
-template <bool WHOLE>
+template <bool WHOLE, bool INT = false>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void zfp_decode3_f32_kernel(const uint64_t* __restrict__ stream, Field3 fd,
                                                              unsigned maxbits, float* __restrict__ out)
 {
@@ -251,7 +270,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void
     int32_t ib[64];
     float w;
     LdsBits mem{lds};
-    decode_block_zy<WHOLE>(mem, lane * slot, maxbits, ib, w);
+    if (INT) {
+      w = 0.0f;
+      decode_block_i32_zy<WHOLE>(mem, lane * slot, maxbits, ib);
+    } else {
+      decode_block_zy<WHOLE>(mem, lane * slot, maxbits, ib, w);
+    }
     // block coordinates and addresses are worked out only now, from a lane id
     // that is recomputed here and tied to a decoded value: otherwise they (or
     // the thread index they come from) are held in registers through the whole
@@ -259,7 +283,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void
     uint32_t zero = 0;
     asm volatile("" : "+v"(zero) : "v"(ib[0]));
     const uint32_t b = first + __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));  // lane id again
-    finish_and_store_block(out, fd, first, b, ib, w);
+    finish_and_store_block<INT>(out, fd, first, b, ib, w);
   }
 }
 
@@ -313,7 +337,7 @@ __device__ __forceinline__ void store_block_low(float* __restrict__ out, const F
 
 // The wave's 64 blocks are packed back to back in LDS exactly as in the stream
 // (64 * maxbits bits = maxbits whole words) and moved cooperatively.
-template <int DIMS>
+template <int DIMS, bool INT = false>
 __global__ __launch_bounds__(64) void zfp_encode_low_f32_kernel(const float* __restrict__ in, FieldLow fd,
                                                                 unsigned maxbits, uint64_t* __restrict__ stream)
 {
@@ -329,7 +353,7 @@ __global__ __launch_bounds__(64) void zfp_encode_low_f32_kernel(const float* __r
     float f[16];
     load_block_low<DIMS>(in, fd, first + lane, f);
     LdsBits mem{lds};
-    encode_block_low<DIMS, true>(f, lane * maxbits, maxbits, mem);
+    encode_block_low<DIMS, true, INT>(f, lane * maxbits, maxbits, mem);
   }
   __syncthreads();
   const unsigned nwords = (valid * maxbits + 63u) >> 6;
@@ -338,7 +362,7 @@ __global__ __launch_bounds__(64) void zfp_encode_low_f32_kernel(const float* __r
   for (unsigned i = lane; i < nwords; i += 64) dst[i] = src[i];
 }
 
-template <int DIMS>
+template <int DIMS, bool INT = false>
 __global__ __launch_bounds__(64) void zfp_decode_low_f32_kernel(const uint64_t* __restrict__ stream, FieldLow fd,
                                                                 unsigned maxbits, float* __restrict__ out)
 {
@@ -355,7 +379,7 @@ __global__ __launch_bounds__(64) void zfp_decode_low_f32_kernel(const uint64_t* 
   if (lane < valid) {
     float f[16];
     LdsBits mem{lds};
-    decode_block_low<DIMS>(mem, lane * maxbits, maxbits, f);
+    decode_block_low<DIMS, INT>(mem, lane * maxbits, maxbits, f);
     store_block_low<DIMS>(out, fd, first + lane, f);
   }
 }
@@ -423,42 +447,65 @@ extern "C" size_t cswap_zfp_stream_capacity(size_t nx, size_t ny, size_t nz, uns
   return ((nb * maxbits + 63) / 64) * 8;
 }
 
-extern "C" int cswap_zfp_compress_f32(const float* d_in, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
-                                      ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream,
-                                      cswap_stream_t stream)
+// d_in / d_out are fields of 32-bit elements: fp32, or int32 when is_int
+static int compress3(const void* d_in, bool is_int, size_t nx, size_t ny, size_t nz, ptrdiff_t sx, ptrdiff_t sy,
+                     ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream, cswap_stream_t stream)
 {
   if (!d_in || !d_stream) return CSWAP_E_ARG;
   Field3 fd;
   int rc = make_field(fd, d_in, d_stream, nx, ny, nz, sx, sy, sz, maxbits);
   if (rc) return rc;
+  const float* in = static_cast<const float*>(d_in);
   unsigned grid = (fd.nblocks + 63) / 64;
   size_t lds_bytes = (size_t)region_dwords(maxbits) * 4;
-  if ((maxbits & 63u) == 0)
-    hipLaunchKernelGGL(zfp_encode3_f32_kernel<true>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
-                       d_in, fd, maxbits, d_stream);
+  hipStream_t st = (hipStream_t)stream;
+  const bool whole = (maxbits & 63u) == 0;
+  if (whole && !is_int)
+    hipLaunchKernelGGL((zfp_encode3_f32_kernel<true, false>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
+  else if (!whole && !is_int)
+    hipLaunchKernelGGL((zfp_encode3_f32_kernel<false, false>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
+  else if (whole)
+    hipLaunchKernelGGL((zfp_encode3_f32_kernel<true, true>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
   else
-    hipLaunchKernelGGL(zfp_encode3_f32_kernel<false>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
-                       d_in, fd, maxbits, d_stream);
+    hipLaunchKernelGGL((zfp_encode3_f32_kernel<false, true>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
   return check_launch();
+}
+
+static int decompress3(const uint64_t* d_stream, bool is_int, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
+                       ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, void* d_out, cswap_stream_t stream)
+{
+  if (!d_out || !d_stream) return CSWAP_E_ARG;
+  Field3 fd;
+  int rc = make_field(fd, d_out, d_stream, nx, ny, nz, sx, sy, sz, maxbits);
+  if (rc) return rc;
+  float* out = static_cast<float*>(d_out);
+  unsigned grid = (fd.nblocks + 63) / 64;
+  size_t lds_bytes = (size_t)region_dwords(maxbits) * 4;
+  hipStream_t st = (hipStream_t)stream;
+  const bool whole = (maxbits & 63u) == 0;
+  if (whole && !is_int)
+    hipLaunchKernelGGL((zfp_decode3_f32_kernel<true, false>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
+  else if (!whole && !is_int)
+    hipLaunchKernelGGL((zfp_decode3_f32_kernel<false, false>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
+  else if (whole)
+    hipLaunchKernelGGL((zfp_decode3_f32_kernel<true, true>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
+  else
+    hipLaunchKernelGGL((zfp_decode3_f32_kernel<false, true>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
+  return check_launch();
+}
+
+extern "C" int cswap_zfp_compress_f32(const float* d_in, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
+                                      ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream,
+                                      cswap_stream_t stream)
+{
+  return compress3(d_in, false, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
 }
 
 extern "C" int cswap_zfp_decompress_f32(const uint64_t* d_stream, size_t nx, size_t ny, size_t nz,
                                         ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
                                         float* d_out, cswap_stream_t stream)
 {
-  if (!d_out || !d_stream) return CSWAP_E_ARG;
-  Field3 fd;
-  int rc = make_field(fd, d_out, d_stream, nx, ny, nz, sx, sy, sz, maxbits);
-  if (rc) return rc;
-  unsigned grid = (fd.nblocks + 63) / 64;
-  size_t lds_bytes = (size_t)region_dwords(maxbits) * 4;
-  if ((maxbits & 63u) == 0)
-    hipLaunchKernelGGL(zfp_decode3_f32_kernel<true>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
-                       d_stream, fd, maxbits, d_out);
-  else
-    hipLaunchKernelGGL(zfp_decode3_f32_kernel<false>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
-                       d_stream, fd, maxbits, d_out);
-  return check_launch();
+  return decompress3(d_stream, false, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
 }
 
 // ------------------------------------------------------------- any dimensionality
@@ -483,42 +530,77 @@ extern "C" size_t cswap_zfp_stream_bytes_nd(int dims, size_t nx, size_t ny, size
   return cswap_zfp_stream_capacity_nd(dims, nx, ny, nz, maxbits);  // 1-D and 2-D round up (zfp/shared.h:42-71)
 }
 
-extern "C" int cswap_zfp_compress_f32_nd(const float* d_in, int dims, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
-                                         ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream,
-                                         cswap_stream_t stream)
+static int compress_nd(const void* d_in, bool is_int, int dims, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
+                       ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream, cswap_stream_t stream)
 {
-  if (dims == 3) return cswap_zfp_compress_f32(d_in, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
+  if (dims == 3) return compress3(d_in, is_int, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
   if (!d_in || !d_stream || (dims != 1 && dims != 2)) return CSWAP_E_ARG;
   FieldLow fd;
   int rc = make_field_low(fd, dims, d_in, d_stream, nx, ny, sx, sy, maxbits);
   if (rc) return rc;
+  const float* in = static_cast<const float*>(d_in);
   unsigned grid = (fd.nblocks + 63) / 64;
   size_t lds_bytes = (size_t)((2u * maxbits + 4u + 3u) / 4u) * 16;
-  if (dims == 2)
-    hipLaunchKernelGGL(zfp_encode_low_f32_kernel<2>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream, d_in,
-                       fd, maxbits, d_stream);
+  hipStream_t st = (hipStream_t)stream;
+  if (dims == 2 && !is_int)
+    hipLaunchKernelGGL((zfp_encode_low_f32_kernel<2, false>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
+  else if (dims == 2)
+    hipLaunchKernelGGL((zfp_encode_low_f32_kernel<2, true>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
+  else if (!is_int)
+    hipLaunchKernelGGL((zfp_encode_low_f32_kernel<1, false>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
   else
-    hipLaunchKernelGGL(zfp_encode_low_f32_kernel<1>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream, d_in,
-                       fd, maxbits, d_stream);
+    hipLaunchKernelGGL((zfp_encode_low_f32_kernel<1, true>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
   return check_launch();
+}
+
+static int decompress_nd(const uint64_t* d_stream, bool is_int, int dims, size_t nx, size_t ny, size_t nz,
+                         ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, void* d_out,
+                         cswap_stream_t stream)
+{
+  if (dims == 3) return decompress3(d_stream, is_int, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
+  if (!d_out || !d_stream || (dims != 1 && dims != 2)) return CSWAP_E_ARG;
+  FieldLow fd;
+  int rc = make_field_low(fd, dims, d_out, d_stream, nx, ny, sx, sy, maxbits);
+  if (rc) return rc;
+  float* out = static_cast<float*>(d_out);
+  unsigned grid = (fd.nblocks + 63) / 64;
+  size_t lds_bytes = (size_t)((2u * maxbits + 4u + 3u) / 4u) * 16;
+  hipStream_t st = (hipStream_t)stream;
+  if (dims == 2 && !is_int)
+    hipLaunchKernelGGL((zfp_decode_low_f32_kernel<2, false>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
+  else if (dims == 2)
+    hipLaunchKernelGGL((zfp_decode_low_f32_kernel<2, true>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
+  else if (!is_int)
+    hipLaunchKernelGGL((zfp_decode_low_f32_kernel<1, false>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
+  else
+    hipLaunchKernelGGL((zfp_decode_low_f32_kernel<1, true>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
+  return check_launch();
+}
+
+extern "C" int cswap_zfp_compress_f32_nd(const float* d_in, int dims, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
+                                         ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream,
+                                         cswap_stream_t stream)
+{
+  return compress_nd(d_in, false, dims, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
 }
 
 extern "C" int cswap_zfp_decompress_f32_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
                                            ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, float* d_out,
                                            cswap_stream_t stream)
 {
-  if (dims == 3) return cswap_zfp_decompress_f32(d_stream, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
-  if (!d_out || !d_stream || (dims != 1 && dims != 2)) return CSWAP_E_ARG;
-  FieldLow fd;
-  int rc = make_field_low(fd, dims, d_out, d_stream, nx, ny, sx, sy, maxbits);
-  if (rc) return rc;
-  unsigned grid = (fd.nblocks + 63) / 64;
-  size_t lds_bytes = (size_t)((2u * maxbits + 4u + 3u) / 4u) * 16;
-  if (dims == 2)
-    hipLaunchKernelGGL(zfp_decode_low_f32_kernel<2>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
-                       d_stream, fd, maxbits, d_out);
-  else
-    hipLaunchKernelGGL(zfp_decode_low_f32_kernel<1>, dim3(grid), dim3(64), lds_bytes, (hipStream_t)stream,
-                       d_stream, fd, maxbits, d_out);
-  return check_launch();
+  return decompress_nd(d_stream, false, dims, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
+}
+
+extern "C" int cswap_zfp_compress_i32_nd(const int32_t* d_in, int dims, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
+                                         ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream,
+                                         cswap_stream_t stream)
+{
+  return compress_nd(d_in, true, dims, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
+}
+
+extern "C" int cswap_zfp_decompress_i32_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
+                                           ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
+                                           int32_t* d_out, cswap_stream_t stream)
+{
+  return decompress_nd(d_stream, true, dims, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
 }

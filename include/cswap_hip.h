@@ -77,6 +77,17 @@ int cswap_zfp_compress_f32_nd(const float* d_in, int dims, size_t nx, size_t ny,
 int cswap_zfp_decompress_f32_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
                                 ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
                                 float* d_out, cswap_stream_t stream);
+/* int32 fields (zfp_type_int32 in cuda_compress / cuda_decompress,
+ * zfp/cuZFP.cu:412-416,513-517): the same transform and coder applied to the
+ * values themselves -- no exponent header, no cast, the whole maxbits is the
+ * coder's budget (zfp/encode.cuh:371-380,393-402,415-424).  Same stream sizes as
+ * above.  64-bit scalar types (double, int64) are not implemented. */
+int cswap_zfp_compress_i32_nd(const int32_t* d_in, int dims, size_t nx, size_t ny, size_t nz,
+                              ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
+                              uint64_t* d_stream, cswap_stream_t stream);
+int cswap_zfp_decompress_i32_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
+                                ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
+                                int32_t* d_out, cswap_stream_t stream);
 
 /* ------------------------------------------------------------------ ZVC -----
  * Zero-value compaction in the reference's format (zfp/compression.cu).  The

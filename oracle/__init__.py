@@ -54,6 +54,10 @@ def _sig(lib: C.CDLL) -> C.CDLL:
     lib.orc_zfp_decode1_f32.restype = None
     lib.orc_zfp_decode1_f32.argtypes = [vp, sz, pd, u, vp]
     lib.orc_perm2.argtypes = [vp]
+    lib.orc_zfp_encode_i32.restype = sz
+    lib.orc_zfp_encode_i32.argtypes = [vp, i, sz, sz, sz, pd, pd, pd, u, vp]
+    lib.orc_zfp_decode_i32.restype = None
+    lib.orc_zfp_decode_i32.argtypes = [vp, i, sz, sz, sz, pd, pd, pd, u, vp]
     lib.orc_zfp_encode_block_f32.restype = None
     lib.orc_zfp_encode_block_f32.argtypes = [vp, u, sz, vp]
     lib.orc_zfp_decode_block_f32.restype = None
@@ -156,6 +160,35 @@ def zfp_decode_nd(stream: np.ndarray, shape, maxbits: int) -> np.ndarray:
         lib().orc_zfp_decode2_f32(_p(s), shape[1], shape[0], 0, 0, maxbits, _p(out))
     else:
         lib().orc_zfp_decode1_f32(_p(s), shape[0], 0, maxbits, _p(out))
+    return out
+
+
+def _dims3(shape):
+    shape = tuple(shape)
+    nx = shape[-1]
+    ny = shape[-2] if len(shape) >= 2 else 1
+    nz = shape[-3] if len(shape) >= 3 else 1
+    return len(shape), nx, ny, nz
+
+
+def zfp_encode_i32(field: np.ndarray, maxbits: int) -> np.ndarray:
+    """1-D, 2-D or 3-D C-contiguous int32 field (x fastest) -> stream words."""
+    assert field.dtype == np.int32 and field.flags.c_contiguous and 1 <= field.ndim <= 3
+    dims, nx, ny, nz = _dims3(field.shape)
+    blocks = int(np.prod([(n + 3) // 4 for n in field.shape]))
+    out = np.zeros((blocks * maxbits + 63) // 64 + 1, dtype=np.uint64)
+    lib().orc_zfp_encode_i32(_p(field), dims, nx, ny, nz, 0, 0, 0, maxbits, _p(out))
+    return out[:-1]
+
+
+def zfp_decode_i32(stream: np.ndarray, shape, maxbits: int) -> np.ndarray:
+    dims, nx, ny, nz = _dims3(shape)
+    blocks = int(np.prod([(n + 3) // 4 for n in shape]))
+    s = np.zeros((blocks * maxbits + 63) // 64 + 1, dtype=np.uint64)
+    w = np.ascontiguousarray(stream).view(np.uint64)
+    s[: w.size] = w
+    out = np.zeros(tuple(shape), dtype=np.int32)
+    lib().orc_zfp_decode_i32(_p(s), dims, nx, ny, nz, 0, 0, 0, maxbits, _p(out))
     return out
 
 

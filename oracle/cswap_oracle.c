@@ -554,6 +554,128 @@ void orc_zfp_decode1_f32(const word_t *stream, size_t nx, ptrdiff_t sx, unsigned
 }
 
 /* ------------------------------------------------------------------------ */
+/* int32 fields (zfp_type_int32, cuZFP.cu:412-416,513-517): the same transform */
+/* and coder applied to the values themselves -- no exponent header, no cast,  */
+/* the whole maxbits is the coder's budget (encode.cuh:371-380,393-402,415-424;*/
+/* decode.cuh:228-288 with the integer specialisations).  Partial blocks are   */
+/* padded by the same rule.  dims = 1, 2 or 3.                                 */
+/* ------------------------------------------------------------------------ */
+
+static void pad_vec_i32(int32_t *p, unsigned n, ptrdiff_t s)
+{
+    switch (n) {
+    case 0: p[0] = 0; /* fall through */
+    case 1: p[s] = p[0]; /* fall through */
+    case 2: p[2 * s] = p[s]; /* fall through */
+    case 3: p[3 * s] = p[0]; /* fall through */
+    default: break;
+    }
+}
+
+static void encode_block_i32(int32_t *ib, int dims, unsigned maxbits, size_t block_idx, word_t *stream)
+{
+    bitcur c = { stream, block_idx * (size_t)maxbits };
+    uint32_t ub[64];
+    if (dims == 3) {
+        orc_fwd_xform3(ib);
+        for (int i = 0; i < 64; i++) ub[i] = orc_int2uint(ib[PERM3[i]]);
+        encode_ints(&c, maxbits, ub, 64);
+    } else if (dims == 2) {
+        for (int y = 0; y < 4; y++) orc_fwd_lift(ib + 4 * y, 1);
+        for (int x = 0; x < 4; x++) orc_fwd_lift(ib + x, 4);
+        for (int i = 0; i < 16; i++) ub[i] = orc_int2uint(ib[PERM2[i]]);
+        encode_ints(&c, maxbits, ub, 16);
+    } else {
+        orc_fwd_lift(ib, 1);
+        for (int i = 0; i < 4; i++) ub[i] = orc_int2uint(ib[i]);
+        encode_ints(&c, maxbits, ub, 4);
+    }
+}
+
+static void decode_block_i32(const word_t *stream, int dims, unsigned maxbits, size_t block_idx, int32_t *ib)
+{
+    bitcur c = { (word_t *)stream, block_idx * (size_t)maxbits };
+    uint32_t ub[64];
+    if (dims == 3) {
+        decode_ints(&c, maxbits, ub, 64);
+        for (int i = 0; i < 64; i++) ib[PERM3[i]] = orc_uint2int(ub[i]);
+        orc_inv_xform3(ib);
+    } else if (dims == 2) {
+        decode_ints(&c, maxbits, ub, 16);
+        for (int i = 0; i < 16; i++) ib[PERM2[i]] = orc_uint2int(ub[i]);
+        for (int x = 0; x < 4; x++) orc_inv_lift(ib + x, 4);
+        for (int y = 0; y < 4; y++) orc_inv_lift(ib + 4 * y, 1);
+    } else {
+        decode_ints(&c, maxbits, ub, 4);
+        for (int i = 0; i < 4; i++) ib[i] = orc_uint2int(ub[i]);
+        orc_inv_lift(ib, 1);
+    }
+}
+
+/* a[nz][ny][nx] (ny, nz ignored below dims); strides 0 = contiguous.  Returns
+ * the stream size in bytes as the reference reports it. */
+size_t orc_zfp_encode_i32(const int32_t *in, int dims, size_t nx, size_t ny, size_t nz,
+                          ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, word_t *stream)
+{
+    if (dims < 2) ny = 1;
+    if (dims < 3) nz = 1;
+    if (!sx) sx = 1;
+    if (!sy) sy = (ptrdiff_t)nx;
+    if (!sz) sz = (ptrdiff_t)(nx * ny);
+    size_t mx = pad4(nx) / 4, my = dims >= 2 ? pad4(ny) / 4 : 1, mz = dims >= 3 ? pad4(nz) / 4 : 1;
+    size_t blocks = mx * my * mz;
+    memset(stream, 0, ((blocks * (size_t)maxbits + 63) / 64) * sizeof(word_t));
+    for (size_t b = 0; b < blocks; b++) {
+        int32_t q[64];
+        size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
+        unsigned bx = (unsigned)(nx - x0 < 4 ? nx - x0 : 4);
+        unsigned by = dims >= 2 ? (unsigned)(ny - y0 < 4 ? ny - y0 : 4) : 1;
+        unsigned bz = dims >= 3 ? (unsigned)(nz - z0 < 4 ? nz - z0 : 4) : 1;
+        const int32_t *p = in + (ptrdiff_t)x0 * sx + (ptrdiff_t)y0 * sy + (ptrdiff_t)z0 * sz;
+        memset(q, 0, sizeof q);
+        for (unsigned z = 0; z < bz; z++) {
+            for (unsigned y = 0; y < by; y++) {
+                for (unsigned x = 0; x < bx; x++) q[16 * z + 4 * y + x] = p[x * sx + y * sy + z * sz];
+                pad_vec_i32(q + 16 * z + 4 * y, bx, 1);
+            }
+            if (dims >= 2)
+                for (unsigned x = 0; x < 4; x++) pad_vec_i32(q + 16 * z + x, by, 4);
+        }
+        if (dims >= 3)
+            for (unsigned y = 0; y < 4; y++)
+                for (unsigned x = 0; x < 4; x++) pad_vec_i32(q + 4 * y + x, bz, 16);
+        encode_block_i32(q, dims, maxbits, b, stream);
+    }
+    if (dims == 3) return orc_zfp_stream_bytes3(nx, ny, nz, maxbits);
+    return ((blocks * (size_t)maxbits + 63) / 64) * sizeof(word_t);
+}
+
+void orc_zfp_decode_i32(const word_t *stream, int dims, size_t nx, size_t ny, size_t nz,
+                        ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, int32_t *out)
+{
+    if (dims < 2) ny = 1;
+    if (dims < 3) nz = 1;
+    if (!sx) sx = 1;
+    if (!sy) sy = (ptrdiff_t)nx;
+    if (!sz) sz = (ptrdiff_t)(nx * ny);
+    size_t mx = pad4(nx) / 4, my = dims >= 2 ? pad4(ny) / 4 : 1, mz = dims >= 3 ? pad4(nz) / 4 : 1;
+    size_t blocks = mx * my * mz;
+    for (size_t b = 0; b < blocks; b++) {
+        int32_t q[64];
+        size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
+        unsigned bx = (unsigned)(nx - x0 < 4 ? nx - x0 : 4);
+        unsigned by = dims >= 2 ? (unsigned)(ny - y0 < 4 ? ny - y0 : 4) : 1;
+        unsigned bz = dims >= 3 ? (unsigned)(nz - z0 < 4 ? nz - z0 : 4) : 1;
+        memset(q, 0, sizeof q);
+        decode_block_i32(stream, dims, maxbits, b, q);
+        int32_t *p = out + (ptrdiff_t)x0 * sx + (ptrdiff_t)y0 * sy + (ptrdiff_t)z0 * sz;
+        for (unsigned z = 0; z < bz; z++)
+            for (unsigned y = 0; y < by; y++)
+                for (unsigned x = 0; x < bx; x++) p[x * sx + y * sy + z * sz] = q[16 * z + 4 * y + x];
+    }
+}
+
+/* ------------------------------------------------------------------------ */
 /* ZVC: zero-value compaction (CSWAP+/zfp/compression.cu)                     */
 /*                                                                           */
 /* The reference runs `process` GPU threads; thread i owns the contiguous    */

@@ -27,6 +27,13 @@ def golden_12d():
 
 
 @pytest.fixture(scope="session")
+def golden_i32():
+    import numpy as np
+
+    return np.load(os.path.join(ROOT, "tests", "golden", "zfp_golden_i32.npz"))
+
+
+@pytest.fixture(scope="session")
 def digests():
     import json
 

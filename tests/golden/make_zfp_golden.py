@@ -13,6 +13,8 @@ Fixture contents
   zfp_golden.npz   small 3-D fields: ``<name>/in`` fp32 (nz,ny,nx), and per rate
                    ``<name>/r<rate>/stream`` (uint8) and ``<name>/r<rate>/dec``.
   zfp_golden_12d.npz  the same for 2-D (ny,nx) and 1-D (nx,) fields.
+  zfp_golden_i32.npz  int32 fields of 1, 2 and 3 dimensions (``-t i32``); written
+                   alone by ``make_zfp_golden.py --i32``.
   zfp_digests.json SHA-256 of input, stream and decoded output for the large
                    seeded configurations (inputs are re-created from the seed).
 """
@@ -35,14 +37,53 @@ from cswap_amd.workloads import config1_field, config3_fields  # noqa: E402
 def run_zfp(field: np.ndarray, rate: float):
     """field: (nz, ny, nx), (ny, nx) or (nx,) -- x is always the fastest axis."""
     dims = [str(n) for n in reversed(field.shape)]
+    is_int = field.dtype == np.int32
+    dt, flag = ("<i4", ["-t", "i32"]) if is_int else ("<f4", ["-f"])
     with tempfile.TemporaryDirectory() as d:
-        fi, fz, fo = (os.path.join(d, n) for n in ("in.f32", "out.zfp", "out.f32"))
-        field.astype("<f4").tofile(fi)
-        subprocess.check_call([ZFP, "-q", "-f", f"-{field.ndim}", *dims, "-r", repr(rate),
+        fi, fz, fo = (os.path.join(d, n) for n in ("in.raw", "out.zfp", "out.raw"))
+        field.astype(dt).tofile(fi)
+        subprocess.check_call([ZFP, "-q", *flag, f"-{field.ndim}", *dims, "-r", repr(rate),
                                "-i", fi, "-z", fz, "-o", fo])
         stream = np.fromfile(fz, dtype=np.uint8)
-        dec = np.fromfile(fo, dtype="<f4").reshape(field.shape)
+        dec = np.fromfile(fo, dtype=dt).reshape(field.shape)
     return stream, dec
+
+
+def int_fields():
+    rng = np.random.default_rng(777)
+    f = {}
+    f["i3_rand_8x8x8"] = rng.integers(-2**20, 2**20, (8, 8, 8)).astype(np.int32)
+    f["i3_partial_7x5x6"] = rng.integers(-1000, 1000, (7, 5, 6)).astype(np.int32)
+    f["i3_wide_4x4x8"] = rng.integers(-2**30, 2**30, (4, 4, 8)).astype(np.int32)
+    z = rng.integers(-500, 500, (8, 8, 8)).astype(np.int32)
+    z[0:4, 0:4, 0:4] = 0
+    z[4:8, 4:8, 4:8] = 12345
+    f["i3_zero_const_blocks"] = z
+    g = np.arange(12)
+    zz, yy, xx = np.meshgrid(g, g, g, indexing="ij")
+    f["i3_smooth_12"] = (1e6 * np.exp(-((xx - 5) ** 2 + (yy - 6) ** 2 + (zz - 4) ** 2) / 30)).astype(np.int32)
+    f["i3_nx2_ny2_8x2x2"] = rng.integers(-2**15, 2**15, (8, 2, 2)).astype(np.int32)
+    f["i3_single"] = np.array([[[-77]]], dtype=np.int32)
+    f["i2_rand_8x12"] = rng.integers(-2**24, 2**24, (8, 12)).astype(np.int32)
+    f["i2_partial_7x9"] = rng.integers(-99, 99, (7, 9)).astype(np.int32)
+    f["i2_smooth_20x20"] = (1e5 * np.exp(-((g[None, :8] - 3) ** 2 + (g[:8, None] - 4) ** 2) / 9)).astype(np.int32)
+    f["i1_rand_64"] = rng.integers(-2**28, 2**28, 64).astype(np.int32)
+    f["i1_partial_13"] = rng.integers(-5, 5, 13).astype(np.int32)
+    f["i1_ramp_100"] = (np.arange(100) * 1000 - 40000).astype(np.int32)
+    return f
+
+
+def main_i32():
+    out = {}
+    for name, fld in int_fields().items():
+        out[f"{name}/in"] = fld
+        rates = RATES_SMALL if fld.ndim == 3 else RATES_2D if fld.ndim == 2 else RATES_1D
+        for r in rates:
+            stream, dec = run_zfp(fld, r)
+            out[f"{name}/r{r}/stream"] = stream
+            out[f"{name}/r{r}/dec"] = dec
+    np.savez_compressed(os.path.join(HERE, "zfp_golden_i32.npz"), **out)
+    print("wrote", len(out), "int32 arrays")
 
 
 def small_fields():
@@ -151,4 +192,8 @@ def main():
 
 
 if __name__ == "__main__":
-    main()
+    if "--i32" in sys.argv:
+        main_i32()
+    else:
+        main()
+        main_i32()

@@ -102,6 +102,76 @@ void host_zfp_decode_low(const uint64_t* stream, size_t nx, size_t ny, unsigned 
   }
 }
 
+// int32 fields through the same header: dims = 1, 2 or 3, contiguous a[nz][ny][nx]
+static void gather_i32(const int32_t* in, int dims, size_t nx, size_t ny, size_t nz, size_t b, float* f, unsigned& bx,
+                       unsigned& by, unsigned& bz, size_t& x0, size_t& y0, size_t& z0)
+{
+  size_t mx = (nx + 3) / 4, my = dims >= 2 ? (ny + 3) / 4 : 1;
+  x0 = (b % mx) * 4; y0 = ((b / mx) % my) * 4; z0 = (b / (mx * my)) * 4;
+  bx = nx - x0 < 4 ? nx - x0 : 4;
+  by = dims >= 2 ? (ny - y0 < 4 ? ny - y0 : 4) : 1;
+  bz = dims >= 3 ? (nz - z0 < 4 ? nz - z0 : 4) : 1;
+  for (int i = 0; i < 64; i++) f[i] = 0.0f;
+  for (unsigned z = 0; z < bz; z++) for (unsigned y = 0; y < by; y++) for (unsigned x = 0; x < bx; x++) {
+    int32_t v = in[(x0 + x) + nx * ((y0 + y) + ny * (z0 + z))];
+    memcpy(&f[x + 4 * y + 16 * z], &v, 4);
+  }
+}
+
+void host_zfp_encode_i32(const int32_t* in, int dims, size_t nx, size_t ny, size_t nz, unsigned maxbits, uint64_t* stream)
+{
+  if (dims < 2) ny = 1;
+  if (dims < 3) nz = 1;
+  size_t blocks = ((nx + 3) / 4) * (dims >= 2 ? (ny + 3) / 4 : 1) * (dims >= 3 ? (nz + 3) / 4 : 1);
+  for (size_t b = 0; b < blocks; b++) {
+    float f[64];
+    unsigned bx, by, bz; size_t x0, y0, z0;
+    gather_i32(in, dims, nx, ny, nz, b, f, bx, by, bz, x0, y0, z0);
+    ArrayBits mem{reinterpret_cast<uint32_t*>(stream)};
+    if (dims == 3) {
+      if (bx < 4 || by < 4 || bz < 4) cswap::pad_block3(f, bx, by, bz);
+      int32_t v[64];
+      memcpy(v, f, sizeof v);
+      cswap::encode_block_i32<true>(v, (unsigned)(b * (size_t)maxbits), maxbits, mem);
+    } else {
+      float g[16];
+      for (int i = 0; i < 16; i++) g[i] = f[i];
+      for (int y = 0; y < (dims == 2 ? 4 : 1); y++) cswap::pad4(g[4 * y], g[4 * y + 1], g[4 * y + 2], g[4 * y + 3], bx);
+      if (dims == 2) {
+        for (int x = 0; x < 4; x++) cswap::pad4(g[x], g[x + 4], g[x + 8], g[x + 12], by);
+        cswap::encode_block_low<2, true, true>(g, (unsigned)(b * (size_t)maxbits), maxbits, mem);
+      } else {
+        cswap::encode_block_low<1, true, true>(g, (unsigned)(b * (size_t)maxbits), maxbits, mem);
+      }
+    }
+  }
+}
+
+void host_zfp_decode_i32(const uint64_t* stream, int dims, size_t nx, size_t ny, size_t nz, unsigned maxbits, int32_t* out)
+{
+  if (dims < 2) ny = 1;
+  if (dims < 3) nz = 1;
+  size_t mx = (nx + 3) / 4, my = dims >= 2 ? (ny + 3) / 4 : 1, mz = dims >= 3 ? (nz + 3) / 4 : 1;
+  for (size_t b = 0; b < mx * my * mz; b++) {
+    size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
+    unsigned bx = nx - x0 < 4 ? nx - x0 : 4, by = dims >= 2 ? (ny - y0 < 4 ? ny - y0 : 4) : 1,
+             bz = dims >= 3 ? (nz - z0 < 4 ? nz - z0 : 4) : 1;
+    int32_t v[64];
+    ArrayBits mem{reinterpret_cast<uint32_t*>(const_cast<uint64_t*>(stream))};
+    if (dims == 3) {
+      cswap::decode_block_i32(mem, (unsigned)(b * (size_t)maxbits), maxbits, v);
+    } else {
+      float g[16];
+      if (dims == 2) cswap::decode_block_low<2, true>(mem, (unsigned)(b * (size_t)maxbits), maxbits, g);
+      else cswap::decode_block_low<1, true>(mem, (unsigned)(b * (size_t)maxbits), maxbits, g);
+      for (int i = 0; i < 64; i++) v[i] = 0;
+      memcpy(v, g, sizeof g);
+    }
+    for (unsigned z = 0; z < bz; z++) for (unsigned y = 0; y < by; y++) for (unsigned x = 0; x < bx; x++)
+      out[(x0 + x) + nx * ((y0 + y) + ny * (z0 + z))] = v[x + 4 * y + 16 * z];
+  }
+}
+
 uint32_t host_div31(uint32_t b, uint32_t d) { return cswap::div31(b, cswap::make_div31(d)); }
 void host_transpose32(uint32_t* a) { uint32_t t[32]; memcpy(t, a, sizeof t); cswap::transpose32(t); memcpy(a, t, sizeof t); }
 

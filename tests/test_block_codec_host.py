@@ -102,3 +102,30 @@ def test_low_dimensional_block_codecs_match_golden_vectors(host, golden_12d):
         assert np.array_equal(o.view(np.uint32), dec.view(np.uint32)), (name, rate)
         n += 1
     assert n >= 60
+
+
+def test_int32_block_codec_matches_golden_vectors(host, golden_i32):
+    """The int32 front ends of the header the GPU lanes run (no exponent header, no
+    cast) against the zfp 0.5.5 vectors for 1-D, 2-D and 3-D fields."""
+    A = [C.c_void_p, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
+    host.host_zfp_encode_i32.argtypes = A
+    host.host_zfp_decode_i32.argtypes = A
+    n = 0
+    for name, rate, maxbits, f, stream, dec in golden_cases(golden_i32):
+        shp = (1,) * (3 - f.ndim) + f.shape
+        nz, ny, nx = shp
+        blocks = int(np.prod([-(-d // 4) for d in f.shape]))
+        words = (blocks * maxbits + 63) // 64
+        s = np.zeros(words + 2, dtype=np.uint64)
+        host.host_zfp_encode_i32(f.ctypes.data, f.ndim, nx, ny, nz, maxbits, s.ctypes.data)
+        sb = s[:words].view(np.uint8)
+        k = min(sb.size, stream.size)
+        assert np.array_equal(sb[:k], stream[:k]), (name, rate)
+        assert not sb[k:].any() and not stream[k:].any()
+        g = np.zeros((words + 2) * 8, dtype=np.uint8)
+        g[:k] = stream[:k]
+        o = np.zeros_like(f)
+        host.host_zfp_decode_i32(g.ctypes.data, f.ndim, nx, ny, nz, maxbits, o.ctypes.data)
+        assert np.array_equal(o, dec), (name, rate)
+        n += 1
+    assert n == 99

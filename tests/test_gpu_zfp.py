@@ -277,3 +277,90 @@ def test_larger_1d_2d_fields_vs_checker(torch_cuda, shape, maxbits):
     want = oracle.zfp_encode_nd(f, maxbits)
     assert np.array_equal(sb.view(np.uint64), want)
     assert np.array_equal(d.view(np.uint32), oracle.zfp_decode_nd(want, f.shape, maxbits).view(np.uint32))
+
+
+def _gpu_i32(torch, f, maxbits):
+    from cswap_amd._lib import check, lib
+
+    L = lib()
+    shp = (1,) * (3 - f.ndim) + f.shape
+    nz, ny, nx = shp
+    t = torch.from_numpy(f).cuda()
+    cap = L.cswap_zfp_stream_capacity_nd(f.ndim, nx, ny, nz, maxbits)
+    s = torch.zeros(cap + 16, dtype=torch.uint8, device="cuda")
+    check(L.cswap_zfp_compress_i32_nd(t.data_ptr(), f.ndim, nx, ny, nz, 0, 0, 0, maxbits, s.data_ptr(), None), "c")
+    o = torch.full(f.shape, -123456, dtype=torch.int32, device="cuda")
+    check(L.cswap_zfp_decompress_i32_nd(s.data_ptr(), f.ndim, nx, ny, nz, 0, 0, 0, maxbits, o.data_ptr(), None), "d")
+    torch.cuda.synchronize()
+    return s[:cap].cpu().numpy(), o.cpu().numpy()
+
+
+def test_int32_golden_vectors(torch_cuda, golden_i32):
+    """zfp_type_int32 fields of 1, 2 and 3 dimensions (cuZFP.cu:412-416,513-517)
+    against the zfp 0.5.5 vectors: stream bytes and decoded values."""
+    n = 0
+    for name, rate, maxbits, f, stream, dec in golden_cases(golden_i32):
+        s, o = _gpu_i32(torch_cuda, f, maxbits)
+        k = min(s.size, stream.size)
+        assert np.array_equal(s[:k], stream[:k]), (name, rate)
+        assert not s[k:].any() and not stream[k:].any(), (name, rate)
+        assert np.array_equal(o, dec), (name, rate)
+        n += 1
+    assert n == 99
+
+
+@pytest.mark.parametrize("shape,maxbits", [((40, 36, 132), 512), ((33, 7, 9), 288), ((300, 260), 128), ((5000,), 40),
+                                           ((64, 64, 64), 1024)])
+def test_int32_fields_vs_checker(torch_cuda, shape, maxbits):
+    import oracle
+
+    rng = np.random.default_rng(sum(shape) + maxbits)
+    f = (rng.standard_normal(shape) * 10.0 ** rng.integers(2, 8)).astype(np.int32)
+    s, o = _gpu_i32(torch_cuda, f, maxbits)
+    want = oracle.zfp_encode_i32(f, maxbits)
+    assert np.array_equal(s.view(np.uint64), want)
+    assert np.array_equal(o, oracle.zfp_decode_i32(want, f.shape, maxbits))
+
+
+def test_cuda_compress_dispatches_on_the_scalar_type(torch_cuda):
+    """cuda_compress / cuda_decompress look at field->type (cuZFP.cu:388-422): float
+    and int32 are coded, the 64-bit types report failure (size 0 / stream pointer
+    not advanced), as the reference does for a type it cannot handle."""
+    torch = torch_cuda
+    import oracle
+    from cswap_amd import api
+
+    rng = np.random.default_rng(3)
+    f = rng.integers(-2**20, 2**20, (8, 12, 16)).astype(np.int32)
+    t = torch.from_numpy(f).cuda()
+    s = api.cuda_compress(t, 512)
+    want = oracle.zfp_encode_i32(f, 512)
+    assert np.array_equal(s.cpu().numpy().view(np.uint64)[: want.size], want)
+    d = api.cuda_decompress(s, f.shape, 512, dtype=torch.int32)
+    torch.cuda.synchronize()
+    assert np.array_equal(d.cpu().numpy(), oracle.zfp_decode_i32(want, f.shape, 512))
+    with pytest.raises((RuntimeError, TypeError, ValueError)):
+        api.cuda_compress(t.to(torch.float64), 512)
+
+    # the reference-named entry points with zfp_field.type = zfp_type_int32 (1) and zfp_type_double (4)
+    import ctypes as C
+
+    from cswap_amd._lib import ZfpBitstream, ZfpField, ZfpStream, lib
+
+    L = lib()
+    cap = L.cswap_zfp_stream_capacity(16, 12, 8, 512)
+    sbuf = torch.zeros(cap, dtype=torch.uint8, device="cuda")
+    bs = ZfpBitstream(0, 0, sbuf.data_ptr(), sbuf.data_ptr(), sbuf.data_ptr() + cap)
+    zs = ZfpStream(1, 512, 64, -1074, C.pointer(bs), 0, 0, 0)
+    fld = ZfpField(1, 16, 12, 8, 0, 0, 0, 0, 0, t.data_ptr())
+    assert L.cuda_compress(C.byref(zs), C.byref(fld)) == cap
+    assert np.array_equal(sbuf.cpu().numpy().view(np.uint64), want)
+    back = torch.zeros_like(t)
+    bs.ptr = bs.begin
+    fld_out = ZfpField(1, 16, 12, 8, 0, 0, 0, 0, 0, back.data_ptr())
+    L.cuda_decompress(C.byref(zs), C.byref(fld_out))
+    assert np.array_equal(back.cpu().numpy(), oracle.zfp_decode_i32(want, f.shape, 512))
+    dbl = torch.zeros(8, 12, 16, dtype=torch.float64, device="cuda")
+    bs.ptr = bs.begin
+    fld_d = ZfpField(4, 16, 12, 8, 0, 0, 0, 0, 0, dbl.data_ptr())
+    assert L.cuda_compress(C.byref(zs), C.byref(fld_d)) == 0
