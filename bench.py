@@ -307,6 +307,8 @@ def extras(torch, api, dev):
         ex["swap_backward"] = swap.bench_backward(dev)
         from cswap_amd import planner
         ex["planner"] = planner.bench_planner(dev)
+        from cswap_amd import hooks
+        ex["train_step"] = hooks.bench_training_step(dev)
     except ImportError:
         pass
     return ex

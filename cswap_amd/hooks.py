@@ -137,3 +137,64 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
                 self.engine.release(h.ticket)
                 self._released.add(h.ticket)
         self._order.clear()
+
+
+def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int = 8 << 20) -> dict:
+    """Forward + backward of a VGG-16 (conv/BN/ReLU x13, 5 pools, linear head) on
+    random data with and without activation swapping through the saved-tensor
+    hooks: step time and peak device memory.  Stock autograd, nothing patched."""
+    import time
+
+    from .planner import _vgg_modules
+
+    torch.manual_seed(0)
+    feats = torch.nn.Sequential(*_vgg_modules(torch, dev))
+    head = torch.nn.Linear(512 * (image // 32) ** 2, 10).to(dev)
+    x = torch.randn(batch, 3, image, image, device=dev)
+    params = list(feats.parameters()) + list(head.parameters())
+
+    def step(ctx):
+        for p in params:
+            p.grad = None
+        if ctx is None:
+            loss = head(feats(x).flatten(1)).square().mean()
+        else:
+            with ctx:
+                loss = head(feats(x).flatten(1)).square().mean()
+        loss.backward()
+        if ctx is not None:
+            ctx.close()
+        return loss
+
+    def measure(make_ctx, reps=5):
+        for _ in range(2):
+            step(make_ctx())
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        best = None
+        stats = None
+        for _ in range(reps):
+            ctx = make_ctx()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            step(ctx)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+            stats = ctx.stats if ctx is not None else None
+        return best * 1e3, torch.cuda.max_memory_allocated() / 1e6, stats
+
+    res = {"model": f"VGG-16 BN, batch {batch}, 3x{image}x{image}", "min_bytes": min_bytes}
+    base_ms, base_mb, _ = measure(lambda: None)
+    res["no_swap"] = {"step_ms": round(base_ms, 2), "peak_MB": round(base_mb, 1)}
+    staging = 512 << 20
+    eng = swap.SwapEngine(pinned_bytes=4 << 30, device_bytes=staging)
+    eng.calibrate()
+    res["staging_pool_MB"] = round(staging / 1e6, 1)    # device memory the engine holds besides torch's allocator
+    for label, pol in (("raw_swap", swap.NONE), ("selector", swap.AUTO)):
+        ms, mb, st = measure(lambda: swap_saved_tensors(eng, policy=pol, min_bytes=min_bytes, prefetch=1))
+        res[label] = {"step_ms": round(ms, 2), "peak_MB": round(mb, 1),
+                      "swapped_tensors": st["swapped"], "swapped_MB": round(st["bytes_in"] / 1e6, 1),
+                      "link_MB": round(st["bytes_out"] / 1e6, 1), "prefetched": st.get("prefetched", 0)}
+    eng.close()
+    return res
