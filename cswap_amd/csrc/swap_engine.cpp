@@ -224,6 +224,14 @@ static void drop_device(cswap_engine* e, Ticket& t)
   }
 }
 
+// Error path of swap_out: kernels already queued on the compute stream may
+// still write the staging block, so it is given back only once they are done.
+static void abandon_device(cswap_engine* e, Ticket& t, hipStream_t compute)
+{
+  if (t.dev_held) (void)hipStreamSynchronize(compute);
+  drop_device(e, t);
+}
+
 extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, size_t ny, size_t nz, int policy,
                               cswap_stream_t compute_, int* ticket)
 {
@@ -243,6 +251,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     if (e->tickets[i].state == kFree) { id = (int)i; break; }
   if (id < 0) return CSWAP_E_NOMEM;
   Ticket& t = e->tickets[(size_t)id];
+  const int requested = policy;
   t.policy = policy; t.n = n; t.nnz = 0; t.nx = nx; t.ny = ny; t.nz = nz;
   t.dev_held = false;
   t.process = zvc_ok ? process_for(e, n) : 0;
@@ -271,14 +280,14 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     if (e->dpool.alloc(worst, &off)) {
       t.dev_off = off; t.dev_bytes = worst; t.dev_held = true;
       int* d_begin = (int*)(e->d_base + off);
-      if ((rc = cswap_zvc_count(d_in, (int)n, t.process, d_begin, compute))) { drop_device(e, t); return rc; }
+      if ((rc = cswap_zvc_count(d_in, (int)n, t.process, d_begin, compute))) { abandon_device(e, t, compute); return rc; }
       if ((rc = cswap_zvc_scan(d_begin, cswap_zvc_active_chunks((int)n, t.process), e->d_nnz, compute))) {
-        drop_device(e, t); return rc;
+        abandon_device(e, t, compute); return rc;
       }
       hipError_t err = hipMemcpyAsync(e->h_nnz, e->d_nnz, sizeof(int), hipMemcpyDeviceToHost, compute);
       if (err == hipSuccess) err = hipEventRecord(e->ev_probe, compute);
       if (err == hipSuccess) err = hipEventSynchronize(e->ev_probe);  // the one host round trip (Execution.h:92)
-      if (err != hipSuccess) { drop_device(e, t); return hip_fail(err); }
+      if (err != hipSuccess) { abandon_device(e, t, compute); return hip_fail(err); }
       t.nnz = (size_t)*e->h_nnz;
     } else if (policy == CSWAP_POLICY_SPARSE) {
       return CSWAP_E_NOMEM;
@@ -299,22 +308,9 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
 
   // ---- compress on the compute stream
   const void* src = nullptr;
-  if (t.policy == CSWAP_POLICY_SPARSE) {
-    const size_t hdr = zvc_header_bytes((int)n, t.process);
-    char* base = e->d_base + t.dev_off;
-    int* d_begin = (int*)base;
-    uint32_t* d_mask = (uint32_t*)(base + 4 * (size_t)t.process);
-    float* d_values = (float*)(base + hdr);
-    if ((rc = cswap_zvc_compact(d_in, (int)n, t.process, d_begin, d_values, d_mask, compute))) {
-      drop_device(e, t); return rc;
-    }
-    t.bytes_out = hdr + 4 * t.nnz;
-    e->dpool.shrink(t.dev_off, t.dev_bytes, t.bytes_out);
-    t.dev_bytes = t.bytes_out;
-    src = base;
-  } else if (t.policy == CSWAP_POLICY_ZFP) {
+  if (t.policy == CSWAP_POLICY_ZFP) {
     t.bytes_out = cswap_zfp_stream_capacity(nx, ny, nz, e->maxbits);
-    if (t.dev_held) {
+    if (t.dev_held) {  // the probe's staging block: keep its head if the stream fits
       if (t.dev_bytes >= t.bytes_out) {
         e->dpool.shrink(t.dev_off, t.dev_bytes, t.bytes_out);
         t.dev_bytes = t.bytes_out;
@@ -324,16 +320,36 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     }
     if (!t.dev_held) {
       size_t off;
-      if (!e->dpool.alloc(t.bytes_out, &off)) return CSWAP_E_NOMEM;
-      t.dev_off = off; t.dev_bytes = t.bytes_out; t.dev_held = true;
+      if (e->dpool.alloc(t.bytes_out, &off)) {
+        t.dev_off = off; t.dev_bytes = t.bytes_out; t.dev_held = true;
+      } else if (requested == CSWAP_POLICY_AUTO) {
+        t.policy = CSWAP_POLICY_NONE;  // no staging room: the selector's choice degrades to the raw swap
+      } else {
+        return CSWAP_E_NOMEM;
+      }
     }
+  }
+  if (t.policy == CSWAP_POLICY_SPARSE) {
+    const size_t hdr = zvc_header_bytes((int)n, t.process);
+    char* base = e->d_base + t.dev_off;
+    int* d_begin = (int*)base;
+    uint32_t* d_mask = (uint32_t*)(base + 4 * (size_t)t.process);
+    float* d_values = (float*)(base + hdr);
+    if ((rc = cswap_zvc_compact(d_in, (int)n, t.process, d_begin, d_values, d_mask, compute))) {
+      abandon_device(e, t, compute); return rc;
+    }
+    t.bytes_out = hdr + 4 * t.nnz;
+    e->dpool.shrink(t.dev_off, t.dev_bytes, t.bytes_out);
+    t.dev_bytes = t.bytes_out;
+    src = base;
+  } else if (t.policy == CSWAP_POLICY_ZFP) {
     uint64_t* d_stream = (uint64_t*)(e->d_base + t.dev_off);
     if ((rc = cswap_zfp_compress_f32(d_in, nx, ny, nz, 0, 0, 0, e->maxbits, d_stream, compute))) {
-      drop_device(e, t); return rc;
+      abandon_device(e, t, compute); return rc;
     }
     src = d_stream;
   } else {
-    drop_device(e, t);
+    drop_device(e, t);  // a probe's block, if any: its kernels finished before the host read nnz
     t.bytes_out = 4 * n;
     src = d_in;
   }

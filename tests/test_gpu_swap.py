@@ -225,6 +225,32 @@ def test_chunk_count_follows_size_rule_tuning_and_configuration(torch_cuda):
     eng.close()
 
 
+def test_selector_degrades_to_raw_swap_when_staging_is_full(torch_cuda):
+    """A staging pool too small for either compressed form: an explicit ZFP or
+    ZVC request is refused (no memory), the selector's request goes out raw and
+    comes back bit-exact."""
+    torch = torch_cuda
+    from cswap_amd import swap
+    from cswap_amd._lib import lib
+
+    eng = swap.SwapEngine(pinned_bytes=128 << 20, device_bytes=1 << 20)
+    x = torch.randn(64, 64, 2048, device="cuda")     # 32 MiB dense: the selector would take ZFP
+    L = lib()
+    tk = C.c_int(-1)
+    for pol in (swap.ZFP, swap.SPARSE):
+        assert L.cswap_swap_out(eng._h, x.data_ptr(), 64, 64, 2048, pol, None, C.byref(tk)) == -4
+    t = eng.pre(x, swap.AUTO)
+    eng.post(t)
+    info = eng.info(t)
+    assert info.policy == swap.NONE and info.bytes_out == x.numel() * 4
+    out = torch.empty_like(x)
+    eng.swap_in(t, out)
+    torch.cuda.synchronize()
+    eng.release(t)
+    assert torch.equal(out, x)
+    eng.close()
+
+
 def test_state_machine_errors(torch_cuda, engine):
     torch = torch_cuda
     from cswap_amd._lib import lib
