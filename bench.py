@@ -232,6 +232,26 @@ def extras(torch, api, dev):
             zfp_case(f"zfp_config3_{name}_r{rate}", t, rate)
         del t
 
+    # ---- the other scalar types cuda_compress dispatches on: same field shape (64, 64, 4096), 16 Mi values
+    g2 = torch.Generator(device=dev); g2.manual_seed(1)
+    base = torch.randn((4096, 64, 64), generator=g2, device=dev)
+    for label, t, rate in (("i32_r8", (base * 1e6).to(torch.int32), 8), ("f64_r16", base.double(), 16),
+                           ("i64_r16", (base.double() * 1e12).to(torch.int64), 16)):
+        n, esz = t.numel(), t.element_size()
+        mb = 64 * rate
+        s = torch.empty(api.zfp_stream_capacity(64, 64, 4096, mb), dtype=torch.uint8, device=dev)
+        o = torch.empty_like(t)
+        api.cuda_compress(t, mb, out=s); api.cuda_decompress(s, t.shape, mb, out=o)
+        e = ev_ms(torch, lambda: api.cuda_compress(t, mb, out=s), 20)
+        d = ev_ms(torch, lambda: api.cuda_decompress(s, t.shape, mb, out=o), 20)
+        bpv = esz + rate / 8
+        ex[f"zfp_{label}_{esz * n >> 20}MiB"] = {
+            "compress_ms": round(e, 4), "decompress_ms": round(d, 4),
+            "pair_GBs_in": round(esz * n / (e + d) / 1e6, 1),
+            "compress_hbm_frac": round(bpv * n / e / 1e6 / HBM_PEAK_GBS, 4),
+            "decompress_hbm_frac": round(bpv * n / d / 1e6 / HBM_PEAK_GBS, 4)}
+    del base
+
     # ---- ZVC compact / expand / probe
     def zvc_case(label, t):
         n = t.numel()

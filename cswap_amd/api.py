@@ -34,26 +34,39 @@ def zfp_stream_capacity(nx: int, ny: int, nz: int, maxbits: int) -> int:
     return lib().cswap_zfp_stream_capacity(nx, ny, nz, maxbits)
 
 
-def cuda_compress(t: torch.Tensor, maxbits: int, out: torch.Tensor | None = None) -> torch.Tensor:
-    """Fixed-rate ZFP of ``t`` viewed as the field (nx=last dim, ny=second to
-    last, nz=rest).  Returns the stream as a uint8 device tensor."""
-    is_int = t.dtype == torch.int32          # zfp_type_int32; every other dtype but fp32 is refused
-    if not is_int:
+# zfp_type of a field by torch dtype (zfp_type_int32 = 1, int64 = 2, float = 3, double = 4)
+_ZFP_KIND = {torch.float32: "f32", torch.int32: "i32", torch.float64: "f64", torch.int64: "i64"}
+
+
+def _need_field(t: torch.Tensor) -> str:
+    kind = _ZFP_KIND.get(t.dtype)
+    if kind is None:
+        raise TypeError(f"ZFP codes float32, float64, int32 and int64 fields, not {t.dtype}")
+    if kind == "f32":
         _need_f32_cuda(t)
     elif not (t.is_cuda and t.is_contiguous()):
-        raise TypeError("expected a contiguous int32 CUDA tensor")
+        raise TypeError(f"expected a contiguous {t.dtype} CUDA tensor")
+    return kind
+
+
+def cuda_compress(t: torch.Tensor, maxbits: int, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Fixed-rate ZFP of ``t`` viewed as the field (nx=last dim, ny=second to
+    last, nz=rest); the scalar type follows the tensor's dtype, as the reference
+    dispatches on ``field->type`` (CSWAP+/zfp/cuZFP.cu:389-423).  Returns the
+    stream as a uint8 device tensor."""
+    kind = _need_field(t)
     nx, ny, nz = field_dims(t.shape)
     cap = zfp_stream_capacity(nx, ny, nz, maxbits)
     if out is None:
         out = torch.empty(cap, dtype=torch.uint8, device=t.device)
     elif out.numel() * out.element_size() < cap:
         raise ValueError("stream buffer too small")
-    if is_int:
-        check(lib().cswap_zfp_compress_i32_nd(t.data_ptr(), 3, nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(),
-                                              _stream()), "cswap_zfp_compress_i32_nd")
-    else:
+    if kind == "f32":
         check(lib().cswap_zfp_compress_f32(t.data_ptr(), nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(), _stream()),
               "cswap_zfp_compress_f32")
+    else:
+        name = f"cswap_zfp_compress_{kind}_nd"
+        check(getattr(lib(), name)(t.data_ptr(), 3, nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(), _stream()), name)
     return out
 
 
@@ -62,19 +75,16 @@ def cuda_decompress(stream: torch.Tensor, shape, maxbits: int, out: torch.Tensor
     nx, ny, nz = field_dims(shape)
     if out is None:
         out = torch.empty(tuple(shape), dtype=dtype, device=stream.device)
-    is_int = out.dtype == torch.int32
-    if not is_int:
-        _need_f32_cuda(out)
-    elif not (out.is_cuda and out.is_contiguous()):
-        raise TypeError("expected a contiguous int32 CUDA tensor")
+    kind = _need_field(out)
     if stream.numel() * stream.element_size() < zfp_stream_capacity(nx, ny, nz, maxbits):
         raise ValueError("stream buffer too small")
-    if is_int:
-        check(lib().cswap_zfp_decompress_i32_nd(stream.data_ptr(), 3, nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(),
-                                                _stream()), "cswap_zfp_decompress_i32_nd")
-    else:
+    if kind == "f32":
         check(lib().cswap_zfp_decompress_f32(stream.data_ptr(), nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(),
                                              _stream()), "cswap_zfp_decompress_f32")
+    else:
+        name = f"cswap_zfp_decompress_{kind}_nd"
+        check(getattr(lib(), name)(stream.data_ptr(), 3, nx, ny, nz, 0, 0, 0, maxbits, out.data_ptr(), _stream()),
+              name)
     return out
 
 

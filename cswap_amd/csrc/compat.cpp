@@ -104,35 +104,39 @@ size_t cuda_compress(cswap_zfp_stream* zs, const cswap_zfp_field* f)
 {
   if (!zs || !f || !zs->stream || !f->data || !zs->stream->begin) return 0;
   const int dims = field_dims_of(f);
-  // fields of 1, 2 or 3 dimensions of float (zfp_type_float = 3) or int32 (zfp_type_int32 = 1);
-  // the 64-bit scalar types the reference also dispatches on (cuZFP.cu:400-422) are not implemented
-  if ((f->type != 3 && f->type != 1) || !dims) return 0;
-  const bool is_int = f->type == 1;
+  // fields of 1, 2 or 3 dimensions of any of the four scalar types the reference
+  // dispatches on (cuZFP.cu:389-423): zfp_type_int32 = 1, int64 = 2, float = 3, double = 4
+  if (f->type < 1 || f->type > 4 || !dims) return 0;
+  const size_t esz = (f->type == 1 || f->type == 3) ? 4 : 8;
   const unsigned maxbits = zs->maxbits;
   const size_t cap = cswap_zfp_stream_capacity_nd(dims, f->nx, f->ny, f->nz, maxbits);
   const size_t bytes = cswap_zfp_stream_bytes_nd(dims, f->nx, f->ny, f->nz, maxbits);
   const bool field_dev = is_device_ptr(f->data), stream_dev = is_device_ptr(zs->stream->begin);
-  const float* d_in = (const float*)f->data;
+  const void* d_in = f->data;
   uint64_t* d_stream = zs->stream->begin;
   void *tmp_in = nullptr, *tmp_s = nullptr;
   size_t ok = 0;
   do {
     if (!field_dev) {  // host field: contiguous only, staged like zfp/cuZFP.cu:265-312
       if (!host_field_contiguous(f)) break;
-      size_t fb = 4 * field_elems(f);
+      size_t fb = esz * field_elems(f);
       if (hipMalloc(&tmp_in, fb) != hipSuccess) break;
       if (hipMemcpy(tmp_in, f->data, fb, hipMemcpyHostToDevice) != hipSuccess) break;
-      d_in = (const float*)tmp_in;
+      d_in = tmp_in;
     }
     if (!stream_dev) {
       if (hipMalloc(&tmp_s, cap) != hipSuccess) break;
       d_stream = (uint64_t*)tmp_s;
     }
     const ptrdiff_t sx = field_dev ? f->sx : 0, sy = field_dev ? f->sy : 0, sz = field_dev ? f->sz : 0;
-    if (is_int ? cswap_zfp_compress_i32_nd((const int32_t*)d_in, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits,
-                                           d_stream, nullptr)
-               : cswap_zfp_compress_f32_nd(d_in, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits, d_stream, nullptr))
-      break;
+    int rc;
+    switch (f->type) {
+      case 1: rc = cswap_zfp_compress_i32_nd((const int32_t*)d_in, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits, d_stream, nullptr); break;
+      case 2: rc = cswap_zfp_compress_i64_nd((const int64_t*)d_in, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits, d_stream, nullptr); break;
+      case 3: rc = cswap_zfp_compress_f32_nd((const float*)d_in, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits, d_stream, nullptr); break;
+      default: rc = cswap_zfp_compress_f64_nd((const double*)d_in, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits, d_stream, nullptr); break;
+    }
+    if (rc) break;
     if (!stream_dev) {
       if (hipMemcpy(zs->stream->begin, tmp_s, cap, hipMemcpyDeviceToHost) != hipSuccess) break;
     } else if (hipStreamSynchronize(nullptr) != hipSuccess) {
@@ -153,22 +157,22 @@ void cuda_decompress(cswap_zfp_stream* zs, cswap_zfp_field* f)
 {
   if (!zs || !f || !zs->stream || !f->data || !zs->stream->begin) return;
   const int dims = field_dims_of(f);
-  if ((f->type != 3 && f->type != 1) || !dims) return;
-  const bool is_int = f->type == 1;
+  if (f->type < 1 || f->type > 4 || !dims) return;
+  const size_t esz = (f->type == 1 || f->type == 3) ? 4 : 8;
   const unsigned maxbits = zs->maxbits;
   const size_t cap = cswap_zfp_stream_capacity_nd(dims, f->nx, f->ny, f->nz, maxbits);
   const size_t bytes = cswap_zfp_stream_bytes_nd(dims, f->nx, f->ny, f->nz, maxbits);
   const bool field_dev = is_device_ptr(f->data), stream_dev = is_device_ptr(zs->stream->begin);
-  float* d_out = (float*)f->data;
+  void* d_out = f->data;
   const uint64_t* d_stream = zs->stream->begin;
   void *tmp_out = nullptr, *tmp_s = nullptr;
-  const size_t fb = 4 * field_elems(f);
+  const size_t fb = esz * field_elems(f);
   bool ok = false;
   do {
     if (!field_dev) {
       if (!host_field_contiguous(f)) break;
       if (hipMalloc(&tmp_out, fb) != hipSuccess) break;
-      d_out = (float*)tmp_out;
+      d_out = tmp_out;
     }
     if (!stream_dev) {
       if (hipMalloc(&tmp_s, cap) != hipSuccess) break;
@@ -176,10 +180,14 @@ void cuda_decompress(cswap_zfp_stream* zs, cswap_zfp_field* f)
       d_stream = (const uint64_t*)tmp_s;
     }
     const ptrdiff_t sx = field_dev ? f->sx : 0, sy = field_dev ? f->sy : 0, sz = field_dev ? f->sz : 0;
-    if (is_int ? cswap_zfp_decompress_i32_nd(d_stream, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits,
-                                             (int32_t*)d_out, nullptr)
-               : cswap_zfp_decompress_f32_nd(d_stream, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits, d_out, nullptr))
-      break;
+    int rc;
+    switch (f->type) {
+      case 1: rc = cswap_zfp_decompress_i32_nd(d_stream, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits, (int32_t*)d_out, nullptr); break;
+      case 2: rc = cswap_zfp_decompress_i64_nd(d_stream, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits, (int64_t*)d_out, nullptr); break;
+      case 3: rc = cswap_zfp_decompress_f32_nd(d_stream, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits, (float*)d_out, nullptr); break;
+      default: rc = cswap_zfp_decompress_f64_nd(d_stream, dims, f->nx, f->ny, f->nz, sx, sy, sz, maxbits, (double*)d_out, nullptr); break;
+    }
+    if (rc) break;
     if (!field_dev) {
       if (hipMemcpy(f->data, tmp_out, fb, hipMemcpyDeviceToHost) != hipSuccess) break;
     } else if (hipStreamSynchronize(nullptr) != hipSuccess) {

@@ -161,8 +161,31 @@ CSWAP_HD void inv_lift4(int32_t& x, int32_t& y, int32_t& z, int32_t& w)
   { int32_t w0 = w; w = wadd(w, x); x = wsub(x, w0); }
 }
 
+// the same two functions on int64 coefficients (zfp_type_double / zfp_type_int64)
+CSWAP_HD int64_t wadd(int64_t a, int64_t b) { return (int64_t)((uint64_t)a + (uint64_t)b); }
+CSWAP_HD int64_t wsub(int64_t a, int64_t b) { return (int64_t)((uint64_t)a - (uint64_t)b); }
+
+CSWAP_HD void fwd_lift4(int64_t& x, int64_t& y, int64_t& z, int64_t& w)
+{
+  x = wadd(x, w); x >>= 1; w = wsub(w, x);
+  z = wadd(z, y); z >>= 1; y = wsub(y, z);
+  x = wadd(x, z); x >>= 1; z = wsub(z, x);
+  w = wadd(w, y); w >>= 1; y = wsub(y, w);
+  w = wadd(w, y >> 1); y = wsub(y, w >> 1);
+}
+
+CSWAP_HD void inv_lift4(int64_t& x, int64_t& y, int64_t& z, int64_t& w)
+{
+  y = wadd(y, w >> 1); w = wsub(w, y >> 1);
+  { int64_t y0 = y; y = wadd(y, w); w = wsub(w, y0); }
+  { int64_t z0 = z; z = wadd(z, x); x = wsub(x, z0); }
+  { int64_t y0 = y; y = wadd(y, z); z = wsub(z, y0); }
+  { int64_t w0 = w; w = wadd(w, x); x = wsub(x, w0); }
+}
+
 // b[x + 4y + 16z]; forward order x, y, z; inverse z, y, x
-CSWAP_HD void fwd_xform3(int32_t (&b)[64])
+template <class I>
+CSWAP_HD void fwd_xform3(I (&b)[64])
 {
 #pragma unroll
   for (int i = 0; i < 16; i++) fwd_lift4(b[4 * i], b[4 * i + 1], b[4 * i + 2], b[4 * i + 3]);
@@ -175,7 +198,8 @@ CSWAP_HD void fwd_xform3(int32_t (&b)[64])
   for (int i = 0; i < 16; i++) fwd_lift4(b[i], b[i + 16], b[i + 32], b[i + 48]);
 }
 
-CSWAP_HD void inv_xform3_zy(int32_t (&b)[64])  // the z and y passes; the x pass is one inv_lift4 per row
+template <class I>
+CSWAP_HD void inv_xform3_zy(I (&b)[64])  // the z and y passes; the x pass is one inv_lift4 per row
 {
 #pragma unroll
   for (int i = 0; i < 16; i++) inv_lift4(b[i], b[i + 16], b[i + 32], b[i + 48]);
@@ -186,7 +210,8 @@ CSWAP_HD void inv_xform3_zy(int32_t (&b)[64])  // the z and y passes; the x pass
       inv_lift4(b[16 * z + x], b[16 * z + x + 4], b[16 * z + x + 8], b[16 * z + x + 12]);
 }
 
-CSWAP_HD void inv_xform3(int32_t (&b)[64])
+template <class I>
+CSWAP_HD void inv_xform3(I (&b)[64])
 {
   inv_xform3_zy(b);
 #pragma unroll
@@ -416,6 +441,29 @@ struct BlockEncoder {
   }
 };
 
+// 32 bit planes of 64 coefficients.  lo / hi hold the 32-bit words of the
+// coefficients 0..31 / 32..63 in coding order with the negabinary constant
+// already added (the xor happens inside the transpose); planes below kmin are
+// not coded.  Top 16 planes first; the low 16 are only transposed if some block
+// of the wavefront still has bit budget left after them.
+template <class Enc>
+CSWAP_HD void encode_planes32(uint32_t (&lo)[32], uint32_t (&hi)[32], Enc& enc, unsigned kmin = 0)
+{
+  tr_stage<16, 0, 32>(lo);
+  tr_stage<16, 0, 32>(hi);
+  tr_half<16, kNotOut>(lo);
+  tr_half<16, kNotOut>(hi);
+#pragma unroll
+  for (int k = 31; k >= 16; k--) enc.plane(((uint64_t)hi[k] << 32) | lo[k]);
+  if (CSWAP_ANY(enc.active())) {
+    tr_half<0, kNotOut>(lo);
+    tr_half<0, kNotOut>(hi);
+#pragma unroll
+    for (int k = 15; k >= 0; k--)
+      if ((unsigned)k >= kmin) enc.plane(((uint64_t)hi[k] << 32) | lo[k]);
+  }
+}
+
 // Integer back end of a 4x4x4 block: transform, reorder, bit planes, coder
 // (encode.cuh:306-345 with the callers at :347-380).  ib is overwritten.
 template <class Enc>
@@ -429,19 +477,33 @@ CSWAP_HD void encode_ints3(int32_t (&ib)[64], Enc& enc)
     lo[i] = (uint32_t)ib[kPerm3.v[i]] + kNegabinary;
     hi[i] = (uint32_t)ib[kPerm3.v[32 + i]] + kNegabinary;
   }
-  // top 16 planes first; the low 16 are only transposed if some block of the
-  // wavefront still has bit budget left after them
-  tr_stage<16, 0, 32>(lo);
-  tr_stage<16, 0, 32>(hi);
-  tr_half<16, kNotOut>(lo);
-  tr_half<16, kNotOut>(hi);
+  encode_planes32(lo, hi, enc);
+}
+
+// The same with int64 coefficients: 64 planes, coded as the 32 planes of the
+// high words followed by the 32 planes of the low words.
+constexpr uint64_t kNegabinary64 = 0xaaaaaaaaaaaaaaaaull;
+template <class Enc>
+CSWAP_HD void encode_ints3(int64_t (&ib)[64], Enc& enc, unsigned kmin)
+{
+  fwd_xform3(ib);
 #pragma unroll
-  for (int k = 31; k >= 16; k--) enc.plane(((uint64_t)hi[k] << 32) | lo[k]);
+  for (int i = 0; i < 64; i++) ib[i] = (int64_t)((uint64_t)ib[i] + kNegabinary64);
+
+  uint32_t lo[32], hi[32];
+#pragma unroll
+  for (int i = 0; i < 32; i++) {
+    lo[i] = (uint32_t)((uint64_t)ib[kPerm3.v[i]] >> 32);
+    hi[i] = (uint32_t)((uint64_t)ib[kPerm3.v[32 + i]] >> 32);
+  }
+  encode_planes32(lo, hi, enc);
   if (CSWAP_ANY(enc.active())) {
-    tr_half<0, kNotOut>(lo);
-    tr_half<0, kNotOut>(hi);
 #pragma unroll
-    for (int k = 15; k >= 0; k--) enc.plane(((uint64_t)hi[k] << 32) | lo[k]);
+    for (int i = 0; i < 32; i++) {
+      lo[i] = (uint32_t)(uint64_t)ib[kPerm3.v[i]];
+      hi[i] = (uint32_t)(uint64_t)ib[kPerm3.v[32 + i]];
+    }
+    encode_planes32(lo, hi, enc, kmin);
   }
 }
 
@@ -469,6 +531,88 @@ CSWAP_HD void encode_block_i32(int32_t (&ib)[64], unsigned pos0, unsigned maxbit
 {
   BlockEncoder<Mem, GUARD> enc(mem, pos0, maxbits);
   encode_ints3(ib, enc);
+}
+
+// ---- 64-bit element types (zfp_type_double, zfp_type_int64; cuZFP.cu:401-423)
+CSWAP_HD double f64_from_bits(uint64_t b)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __longlong_as_double((long long)b);
+#else
+  union { uint64_t u; double f; } c; c.u = b; return c.f;
+#endif
+}
+CSWAP_HD uint64_t f64_bits(double f)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  return (uint64_t)__double_as_longlong(f);
+#else
+  union { uint64_t u; double f; } c; c.f = f; return c.u;
+#endif
+}
+
+// 2^e as a double for any e: +inf above 1023, subnormal down to -1074, 0 below (ldexp(1.0, e))
+CSWAP_HD double pow2d(int e)
+{
+  if (e > 1023) return f64_from_bits(0x7ff0000000000000ull);
+  if (e >= -1022) return f64_from_bits((uint64_t)(e + 1023) << 52);
+  if (e >= -1074) return f64_from_bits((uint64_t)1 << (e + 1074));
+  return 0.0;
+}
+
+// double -> int64, truncating; saturates out of range and maps NaN to 0 (C leaves
+// both undefined; the scale 2^(62-emax) overflows for blocks below 2^-961)
+CSWAP_HD int64_t sat_i64(double v)
+{
+  if (!(v == v)) return 0;
+  if (v >= 9223372036854775808.0) return INT64_MAX;
+  if (v <= -9223372036854775808.0) return INT64_MIN;
+  return (int64_t)v;
+}
+
+// header exponent of a block of SIZE doubles given as bit patterns: E + 1 with E
+// the biased exponent field of the largest magnitude (emax = E - 1022, clamped at
+// -1022 for subnormals, encode.cuh:40-71), or 0 for an all-zero block
+template <int SIZE>
+CSWAP_HD uint32_t block_header_e64(const uint64_t (&q)[SIZE])
+{
+  uint64_t m = 0;  // magnitudes of finite doubles order like their bit patterns
+#pragma unroll
+  for (int i = 0; i < SIZE; i++) {
+    uint64_t a = q[i] & 0x7fffffffffffffffull;
+    m = a > m ? a : m;
+  }
+  return m ? (uint32_t)(m >> 52) + 1 : 0;
+}
+
+// planes below this one are not coded for a block of doubles with header
+// exponent e (encode.cuh:10-15: precision = min(64, emax + 1074 + 8), emax = e - 1023)
+CSWAP_HD unsigned kmin_f64(uint32_t e)
+{
+  int maxprec = (int)e - 1023 + 1082;
+  return maxprec >= 64 ? 0u : (unsigned)(64 - maxprec);
+}
+
+// q[x + 4y + 16z]: the (padded) block as 64-bit patterns of doubles, or of int64 when INT
+template <bool GUARD, bool INT, class Mem>
+CSWAP_HD void encode_block_w64(const uint64_t (&q)[64], unsigned pos0, unsigned maxbits, Mem& mem)
+{
+  BlockEncoder<Mem, GUARD> enc(mem, pos0, maxbits);
+  int64_t ib[64];
+  unsigned kmin = 0;
+  if (INT) {
+#pragma unroll
+    for (int i = 0; i < 64; i++) ib[i] = (int64_t)q[i];
+  } else {
+    uint32_t e = block_header_e64<64>(q);
+    if (e == 0) return;
+    enc.put(2 * (uint64_t)e + 1, 12);
+    kmin = kmin_f64(e);
+    double s = pow2d(62 - ((int)e - 1023));
+#pragma unroll
+    for (int i = 0; i < 64; i++) ib[i] = sat_i64(s * f64_from_bits(q[i]));
+  }
+  encode_ints3(ib, enc, kmin);
 }
 
 // ---------------------------------------------------------------- decoder
@@ -534,12 +678,15 @@ struct BlockDecoder {
 //                    and y; leaves ib[x + 4y + 16z] and the scale w
 //   decode_row       inverse lifting along x of one row and the cast to float
 // An empty block gives ib = 0 and w = 0, i.e. +0.0 everywhere.
-// Integer back end of a 4x4x4 block up to and including the inverse lifting
-// along z and y (decode.cuh:127-179 and the first two passes of :181-226).
+
+// 32 bit planes -> the 32-bit words of 64 coefficients (lo: 0..31, hi: 32..63 in
+// coding order).  Negabinary: the xor happens inside the transpose, the
+// subtraction of the returned constant is left to the caller.  When the low 16
+// planes are all zero they are not transposed, so their complemented odd planes
+// (0xaaaa in every value) are missing from the minuend as well.
 template <class Dec>
-CSWAP_HD void decode_ints3_zy(Dec& dec, int32_t (&ib)[64])
+CSWAP_HD uint32_t decode_planes32(Dec& dec, uint32_t (&lo)[32], uint32_t (&hi)[32])
 {
-  uint32_t lo[32], hi[32];
 #pragma unroll
   for (int k = 31; k >= 16; k--) {  // planes that no block of the wavefront can reach are zero without a read
     uint64_t x = CSWAP_ANY(dec.active()) ? dec.plane() : 0;
@@ -548,9 +695,6 @@ CSWAP_HD void decode_ints3_zy(Dec& dec, int32_t (&ib)[64])
   }
   tr_half<16, kNotIn>(lo);
   tr_half<16, kNotIn>(hi);
-  // negabinary: the xor inside the transpose, the subtraction here.  When the low
-  // 16 planes are all zero they are not transposed, so their complemented odd
-  // planes (0xaaaa in every value) are missing from the minuend as well.
   uint32_t c = kNegabinary;
   if (CSWAP_ANY(dec.active())) {
 #pragma unroll
@@ -568,13 +712,77 @@ CSWAP_HD void decode_ints3_zy(Dec& dec, int32_t (&ib)[64])
   }
   tr_stage<16, 0, 32>(lo);
   tr_stage<16, 0, 32>(hi);
+  return c;
+}
 
+// Integer back end of a 4x4x4 block up to and including the inverse lifting
+// along z and y (decode.cuh:127-179 and the first two passes of :181-226).
+template <class Dec>
+CSWAP_HD void decode_ints3_zy(Dec& dec, int32_t (&ib)[64])
+{
+  uint32_t lo[32], hi[32];
+  const uint32_t c = decode_planes32(dec, lo, hi);
 #pragma unroll
   for (int i = 0; i < 32; i++) {
     ib[kPerm3.v[i]] = (int32_t)(lo[i] - c);
     ib[kPerm3.v[32 + i]] = (int32_t)(hi[i] - c);
   }
   inv_xform3_zy(ib);
+}
+
+// int64 coefficients: the high words from the first 32 planes, the low words from
+// the next 32 (skipped, with nothing to subtract for them, when no block of the
+// wavefront has budget left); whole inverse transform
+template <class Dec>
+CSWAP_HD void decode_ints3(Dec& dec, int64_t (&ib)[64])
+{
+  uint32_t lo[32], hi[32];
+  uint64_t c = (uint64_t)decode_planes32(dec, lo, hi) << 32;
+#pragma unroll
+  for (int i = 0; i < 32; i++) {
+    ib[kPerm3.v[i]] = (int64_t)((uint64_t)lo[i] << 32);
+    ib[kPerm3.v[32 + i]] = (int64_t)((uint64_t)hi[i] << 32);
+  }
+  if (CSWAP_ANY(dec.active())) {
+    c |= decode_planes32(dec, lo, hi);
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      ib[kPerm3.v[i]] |= (int64_t)(uint64_t)lo[i];
+      ib[kPerm3.v[32 + i]] |= (int64_t)(uint64_t)hi[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 64; i++) ib[i] = (int64_t)((uint64_t)ib[i] - c);
+  inv_xform3(ib);
+}
+
+// q[x + 4y + 16z] receives the block as 64-bit patterns (doubles, or int64 when INT);
+// an empty block of doubles gives +0.0 everywhere
+template <bool INT, bool FENCED = false, class Mem>
+CSWAP_HD void decode_block_w64(Mem& mem, unsigned pos0, unsigned maxbits, uint64_t (&q)[64])
+{
+  BlockDecoder<Mem, 64, FENCED> dec(mem, pos0, maxbits);
+  int emax = 0;
+  if (!INT) {
+    uint32_t h = (uint32_t)dec.window(pos0);
+    if (!(h & 1)) {
+#pragma unroll
+      for (int i = 0; i < 64; i++) q[i] = 0;
+      return;
+    }
+    emax = (int)((h >> 1) & 0x7ff) - 1023;
+    dec.pos = pos0 + 12;
+  }
+  int64_t ib[64];
+  decode_ints3(dec, ib);
+  if (INT) {
+#pragma unroll
+    for (int i = 0; i < 64; i++) q[i] = (uint64_t)ib[i];
+  } else {
+    const double w = pow2d(emax - 62);
+#pragma unroll
+    for (int i = 0; i < 64; i++) q[i] = f64_bits(w * (double)ib[i]);
+  }
 }
 
 template <bool FENCED = false, class Mem>
@@ -735,18 +943,123 @@ CSWAP_HD void decode_block_low(Mem& mem, unsigned pos0, unsigned maxbits, float 
   for (int i = SIZE; i < 16; i++) f[i] = 0.0f;
 }
 
+// The same for 64-bit element types: q holds 64-bit patterns (doubles, or int64
+// when INT); 64 planes coded as the planes of the high words, then of the low words.
+template <int DIMS, bool GUARD, bool INT, class Mem>
+CSWAP_HD void encode_block_low_w64(const uint64_t (&q)[16], unsigned pos0, unsigned maxbits, Mem& mem)
+{
+  constexpr int SIZE = DIMS == 2 ? 16 : 4;
+  BlockEncoder<Mem, GUARD, SIZE> enc(mem, pos0, maxbits);
+  int64_t ib[16];
+  unsigned kmin = 0;
+  if (INT) {
+#pragma unroll
+    for (int i = 0; i < SIZE; i++) ib[i] = (int64_t)q[i];
+  } else {
+    uint64_t m = 0;
+#pragma unroll
+    for (int i = 0; i < SIZE; i++) {
+      uint64_t a = q[i] & 0x7fffffffffffffffull;
+      m = a > m ? a : m;
+    }
+    uint32_t e = m ? (uint32_t)(m >> 52) + 1 : 0;
+    if (e == 0) return;
+    enc.put(2 * (uint64_t)e + 1, 12);
+    kmin = kmin_f64(e);
+    double s = pow2d(62 - ((int)e - 1023));
+#pragma unroll
+    for (int i = 0; i < SIZE; i++) ib[i] = sat_i64(s * f64_from_bits(q[i]));
+  }
+  uint64_t u[16];
+  if (DIMS == 2) {
+#pragma unroll
+    for (int y = 0; y < 4; y++) fwd_lift4(ib[4 * y], ib[4 * y + 1], ib[4 * y + 2], ib[4 * y + 3]);
+#pragma unroll
+    for (int x = 0; x < 4; x++) fwd_lift4(ib[x], ib[x + 4], ib[x + 8], ib[x + 12]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) u[i] = ((uint64_t)ib[kPerm2.v[i]] + kNegabinary64) ^ kNegabinary64;
+  } else {
+    fwd_lift4(ib[0], ib[1], ib[2], ib[3]);
+#pragma unroll
+    for (int i = 0; i < 4; i++) u[i] = ((uint64_t)ib[i] + kNegabinary64) ^ kNegabinary64;
+  }
+  uint32_t a[32];
+#pragma unroll
+  for (int i = 0; i < 32; i++) a[i] = i < SIZE ? (uint32_t)(u[i < SIZE ? i : 0] >> 32) : 0u;
+  transpose32(a);
+#pragma unroll
+  for (int k = 31; k >= 0; k--) enc.plane((uint64_t)a[k]);
+#pragma unroll
+  for (int i = 0; i < 32; i++) a[i] = i < SIZE ? (uint32_t)u[i < SIZE ? i : 0] : 0u;
+  transpose32(a);
+#pragma unroll
+  for (int k = 31; k >= 0; k--)
+    if ((unsigned)k >= kmin) enc.plane((uint64_t)a[k]);
+}
+
+template <int DIMS, bool INT, class Mem>
+CSWAP_HD void decode_block_low_w64(Mem& mem, unsigned pos0, unsigned maxbits, uint64_t (&q)[16])
+{
+  constexpr int SIZE = DIMS == 2 ? 16 : 4;
+  BlockDecoder<Mem, SIZE> dec(mem, pos0, maxbits);
+  int emax = 0;
+#pragma unroll
+  for (int i = 0; i < 16; i++) q[i] = 0;
+  if (!INT) {
+    uint32_t h = (uint32_t)dec.window(pos0);
+    if (!(h & 1)) return;
+    emax = (int)((h >> 1) & 0x7ff) - 1023;
+    dec.pos = pos0 + 12;
+  }
+  uint32_t a[32];
+  uint64_t u[16];
+#pragma unroll
+  for (int k = 31; k >= 0; k--) a[k] = (uint32_t)dec.plane();
+  transpose32(a);
+#pragma unroll
+  for (int i = 0; i < SIZE; i++) u[i] = (uint64_t)a[i] << 32;
+#pragma unroll
+  for (int k = 31; k >= 0; k--) a[k] = (uint32_t)dec.plane();
+  transpose32(a);
+#pragma unroll
+  for (int i = 0; i < SIZE; i++) u[i] |= a[i];
+  int64_t ib[16];
+  if (DIMS == 2) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) ib[kPerm2.v[i]] = (int64_t)((u[i] ^ kNegabinary64) - kNegabinary64);
+#pragma unroll
+    for (int x = 0; x < 4; x++) inv_lift4(ib[x], ib[x + 4], ib[x + 8], ib[x + 12]);
+#pragma unroll
+    for (int y = 0; y < 4; y++) inv_lift4(ib[4 * y], ib[4 * y + 1], ib[4 * y + 2], ib[4 * y + 3]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; i++) ib[i] = (int64_t)((u[i] ^ kNegabinary64) - kNegabinary64);
+    inv_lift4(ib[0], ib[1], ib[2], ib[3]);
+  }
+  if (INT) {
+#pragma unroll
+    for (int i = 0; i < SIZE; i++) q[i] = (uint64_t)ib[i];
+  } else {
+    const double w = pow2d(emax - 62);
+#pragma unroll
+    for (int i = 0; i < SIZE; i++) q[i] = f64_bits(w * (double)ib[i]);
+  }
+}
+
 // ---------------------------------------------------------------- partial blocks
 // Padding rule for a 4-vector of which the first n entries are valid
 // (encode.cuh:17-38): n=1 -> (a,a,a,a), n=2 -> (a,b,b,a), n=3 -> (a,b,c,a).
-CSWAP_HD void pad4(float& a, float& b, float& c, float& d, unsigned n)
+template <class T>
+CSWAP_HD void pad4(T& a, T& b, T& c, T& d, unsigned n)
 {
-  if (n == 0) a = 0.0f;
+  if (n == 0) a = T(0);
   if (n <= 1) b = a;
   if (n <= 2) c = b;
   if (n <= 3) d = a;
 }
 
-CSWAP_HD void pad_block3(float (&f)[64], unsigned bx, unsigned by, unsigned bz)
+template <class T>
+CSWAP_HD void pad_block3(T (&f)[64], unsigned bx, unsigned by, unsigned bz)
 {
 #pragma unroll
   for (int z = 0; z < 4; z++) {

@@ -124,9 +124,6 @@ __device__ __forceinline__ void load_block(const float* __restrict__ in, const F
   }
 }
 
-// Finishes the block (inverse lifting along x, cast) and stores it.  On the
-// fast path every x-row is finished and stored on its own, so the finished
-// values never all sit in registers at once.
 // one x-row of an int32 block: last lifting pass, values handed on as bit patterns
 __device__ __forceinline__ void decode_row_i32(int32_t (&ib)[64], int row, float (&f)[4])
 {
@@ -135,6 +132,9 @@ __device__ __forceinline__ void decode_row_i32(int32_t (&ib)[64], int row, float
   for (int x = 0; x < 4; x++) f[x] = __int_as_float(ib[4 * row + x]);
 }
 
+// Finishes the block (inverse lifting along x, cast) and stores it.  Every
+// x-row is finished and stored on its own, so the finished values never all
+// sit in registers at once.
 template <bool INT>
 __device__ __forceinline__ void finish_and_store_block(float* __restrict__ out, const Field3& fd, uint32_t first,
                                                        uint32_t b, int32_t (&ib)[64], float w)
@@ -172,6 +172,66 @@ __device__ __forceinline__ void finish_and_store_block(float* __restrict__ out, 
   }
 }
 
+// ------------------------------------------------------------- LDS region <-> stream
+__device__ __forceinline__ void zero_region(uint4* lds_raw, unsigned lane, unsigned maxbits)
+{
+  const unsigned n16 = region_dwords(maxbits) / 4;
+  for (unsigned i = lane; i < n16; i += 64) lds_raw[i] = make_uint4(0, 0, 0, 0);
+}
+
+// the wave's coded blocks from LDS to the stream
+template <bool WHOLE>
+__device__ __forceinline__ void store_region(const uint32_t* lds, unsigned lane, uint32_t first, uint32_t valid,
+                                             unsigned maxbits, int stream16, uint64_t* __restrict__ stream)
+{
+  if (WHOLE) {
+    // each lane stores the words of its own block (16-byte stores where aligned)
+    if (lane < valid) {
+      const unsigned W = maxbits >> 6;
+      const uint64_t* src = reinterpret_cast<const uint64_t*>(lds + lane * (slot_bits(maxbits) / 32));
+      uint64_t* dst = stream + (size_t)(first + lane) * W;
+      if ((W & 1u) == 0 && stream16) {
+        for (unsigned j = 0; j < W; j += 2)
+          *reinterpret_cast<ulonglong2*>(dst + j) = *reinterpret_cast<const ulonglong2*>(src + j);
+      } else {
+        for (unsigned j = 0; j < W; j++) dst[j] = src[j];
+      }
+    }
+  } else {
+    const unsigned nwords = (valid * maxbits + 63u) >> 6;
+    const uint64_t* src = reinterpret_cast<const uint64_t*>(lds);
+    uint64_t* dst = stream + (size_t)(first >> 6) * maxbits;
+    for (unsigned i = lane; i < nwords; i += 64) dst[i] = src[i];
+  }
+}
+
+// the wave's coded blocks from the stream into LDS; whole-word rates get the
+// fence of ones behind every block that the fenced decoder relies on
+template <bool WHOLE>
+__device__ __forceinline__ void load_region(uint32_t* lds, unsigned lane, uint32_t first, uint32_t valid,
+                                            unsigned maxbits, int stream16, const uint64_t* __restrict__ stream)
+{
+  if (WHOLE) {
+    if (lane < valid) {
+      const unsigned W = maxbits >> 6;
+      uint64_t* dst = reinterpret_cast<uint64_t*>(lds + lane * (slot_bits(maxbits) / 32));
+      const uint64_t* src = stream + (size_t)(first + lane) * W;
+      if ((W & 1u) == 0 && stream16) {
+        for (unsigned j = 0; j < W; j += 2)
+          *reinterpret_cast<ulonglong2*>(dst + j) = *reinterpret_cast<const ulonglong2*>(src + j);
+      } else {
+        for (unsigned j = 0; j < W; j++) dst[j] = src[j];
+      }
+      dst[W] = ~0ull;
+    }
+  } else {
+    const unsigned nwords = (valid * maxbits + 63u) >> 6;
+    const uint64_t* src = stream + (size_t)(first >> 6) * maxbits;
+    uint64_t* dst = reinterpret_cast<uint64_t*>(lds);
+    for (unsigned i = lane; i < nwords + 2; i += 64) dst[i] = i < nwords ? src[i] : 0;
+  }
+}
+
 // ------------------------------------------------------------- kernels
 // grid.x = ceil(nblocks/64) workgroups of one wavefront; dynamic LDS =
 // region_dwords(maxbits) dwords.
@@ -188,11 +248,7 @@ __global__ __launch_bounds__(64) void zfp_encode3_f32_kernel(const float* __rest
   const uint32_t valid = min(64u, fd.nblocks - first);
   const unsigned slot = slot_bits(maxbits);
 
-  // zero the region: each lane clears slot bits (+ the shared padding)
-  {
-    const unsigned n16 = region_dwords(maxbits) / 4;
-    for (unsigned i = lane; i < n16; i += 64) lds_raw[i] = make_uint4(0, 0, 0, 0);
-  }
+  zero_region(lds_raw, lane, maxbits);
   __syncthreads();
 
   if (lane < valid) {
@@ -209,31 +265,13 @@ __global__ __launch_bounds__(64) void zfp_encode3_f32_kernel(const float* __rest
     }
   }
   __syncthreads();
-
-  if (WHOLE) {
-    // each lane stores the words of its own block (16-byte stores where aligned)
-    if (lane < valid) {
-      const unsigned W = maxbits >> 6;
-      const uint64_t* src = reinterpret_cast<const uint64_t*>(lds + lane * (slot / 32));
-      uint64_t* dst = stream + (size_t)(first + lane) * W;
-      if ((W & 1u) == 0 && fd.stream16) {
-        for (unsigned j = 0; j < W; j += 2)
-          *reinterpret_cast<ulonglong2*>(dst + j) = *reinterpret_cast<const ulonglong2*>(src + j);
-      } else {
-        for (unsigned j = 0; j < W; j++) dst[j] = src[j];
-      }
-    }
-  } else {
-    const unsigned nwords = (valid * maxbits + 63u) >> 6;
-    const uint64_t* src = reinterpret_cast<const uint64_t*>(lds);
-    uint64_t* dst = stream + (size_t)blockIdx.x * maxbits;
-    for (unsigned i = lane; i < nwords; i += 64) dst[i] = src[i];
-  }
+  store_region<WHOLE>(lds, lane, first, valid, maxbits, fd.stream16, stream);
 }
 
-// Five wavefronts per SIMD (96 registers, five of them spilled around the
-// store phase): measured 2.5 % faster than the four that 105 registers allow;
-// six (80 registers, 20 spills) is slower again.
+// Five wavefronts per SIMD (at most 96 registers, which the row-wise finish
+// and the late block coordinates below reach without spilling): measured
+// 2.5 % faster than the four that the unconstrained 105 registers allow; six
+// (80 registers) spills and is slower again.
 template <bool WHOLE, bool INT = false>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void zfp_decode3_f32_kernel(const uint64_t* __restrict__ stream, Field3 fd,
                                                              unsigned maxbits, float* __restrict__ out)
@@ -245,25 +283,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void
   const uint32_t valid = min(64u, fd.nblocks - first);
   const unsigned slot = slot_bits(maxbits);
 
-  if (WHOLE) {
-    if (lane < valid) {
-      const unsigned W = maxbits >> 6;
-      uint64_t* dst = reinterpret_cast<uint64_t*>(lds + lane * (slot / 32));
-      const uint64_t* src = stream + (size_t)(first + lane) * W;
-      if ((W & 1u) == 0 && fd.stream16) {
-        for (unsigned j = 0; j < W; j += 2)
-          *reinterpret_cast<ulonglong2*>(dst + j) = *reinterpret_cast<const ulonglong2*>(src + j);
-      } else {
-        for (unsigned j = 0; j < W; j++) dst[j] = src[j];
-      }
-      dst[W] = ~0ull;  // the fence the decoder relies on: ones right after the block
-    }
-  } else {
-    const unsigned nwords = (valid * maxbits + 63u) >> 6;
-    const uint64_t* src = stream + (size_t)blockIdx.x * maxbits;
-    uint64_t* dst = reinterpret_cast<uint64_t*>(lds);
-    for (unsigned i = lane; i < nwords + 2; i += 64) dst[i] = i < nwords ? src[i] : 0;
-  }
+  load_region<WHOLE>(lds, lane, first, valid, maxbits, fd.stream16, stream);
   __syncthreads();
 
   if (lane < valid) {
@@ -284,6 +304,111 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void
     asm volatile("" : "+v"(zero) : "v"(ib[0]));
     const uint32_t b = first + __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));  // lane id again
     finish_and_store_block<INT>(out, fd, first, b, ib, w);
+  }
+}
+
+// ------------------------------------------------------------- 64-bit elements
+// Fields of doubles or int64 (zfp_type_double, zfp_type_int64): the same
+// decomposition, values moved as 64-bit patterns.  Fast path: full block whose
+// x-rows are contiguous and 16-byte aligned (two 16-byte accesses per row).
+__device__ __forceinline__ void load_block_w64(const uint64_t* __restrict__ in, const Field3& fd, uint32_t b,
+                                               uint64_t (&q)[64])
+{
+  uint32_t x0, y0, z0;
+  block_origin(fd, b, x0, y0, z0);
+  const uint32_t bx = min(4u, fd.nx - x0), by = min(4u, fd.ny - y0), bz = min(4u, fd.nz - z0);
+  const uint64_t* p = in + (long long)x0 * fd.sx + (long long)y0 * fd.sy + (long long)z0 * fd.sz;
+  if (fd.rows16 && bx == 4 && by == 4 && bz == 4) {
+#pragma unroll
+    for (int z = 0; z < 4; z++)
+#pragma unroll
+      for (int y = 0; y < 4; y++) {
+        const ulonglong2* r = reinterpret_cast<const ulonglong2*>(p + y * fd.sy + z * fd.sz);
+        const ulonglong2 a = r[0], c = r[1];
+        q[16 * z + 4 * y + 0] = a.x;
+        q[16 * z + 4 * y + 1] = a.y;
+        q[16 * z + 4 * y + 2] = c.x;
+        q[16 * z + 4 * y + 3] = c.y;
+      }
+  } else {
+#pragma unroll
+    for (int z = 0; z < 4; z++)
+#pragma unroll
+      for (int y = 0; y < 4; y++)
+#pragma unroll
+        for (int x = 0; x < 4; x++) {
+          bool ok = (uint32_t)x < bx && (uint32_t)y < by && (uint32_t)z < bz;
+          q[16 * z + 4 * y + x] = ok ? p[x * fd.sx + y * fd.sy + z * fd.sz] : 0ull;
+        }
+    if (bx < 4 || by < 4 || bz < 4) pad_block3(q, bx, by, bz);
+  }
+}
+
+__device__ __forceinline__ void store_block_w64(uint64_t* __restrict__ out, const Field3& fd, uint32_t b,
+                                                const uint64_t (&q)[64])
+{
+  uint32_t x0, y0, z0;
+  block_origin(fd, b, x0, y0, z0);
+  const uint32_t bx = min(4u, fd.nx - x0), by = min(4u, fd.ny - y0), bz = min(4u, fd.nz - z0);
+  uint64_t* p = out + (long long)x0 * fd.sx + (long long)y0 * fd.sy + (long long)z0 * fd.sz;
+  if (fd.rows16 && bx == 4 && by == 4 && bz == 4) {
+#pragma unroll
+    for (int z = 0; z < 4; z++)
+#pragma unroll
+      for (int y = 0; y < 4; y++) {
+        ulonglong2* r = reinterpret_cast<ulonglong2*>(p + y * fd.sy + z * fd.sz);
+        r[0] = make_ulonglong2(q[16 * z + 4 * y + 0], q[16 * z + 4 * y + 1]);
+        r[1] = make_ulonglong2(q[16 * z + 4 * y + 2], q[16 * z + 4 * y + 3]);
+      }
+  } else {
+#pragma unroll
+    for (int z = 0; z < 4; z++)
+#pragma unroll
+      for (int y = 0; y < 4; y++)
+#pragma unroll
+        for (int x = 0; x < 4; x++)
+          if ((uint32_t)x < bx && (uint32_t)y < by && (uint32_t)z < bz)
+            p[x * fd.sx + y * fd.sy + z * fd.sz] = q[16 * z + 4 * y + x];
+  }
+}
+
+template <bool WHOLE, bool INT>
+__global__ __launch_bounds__(64) void zfp_encode3_w64_kernel(const uint64_t* __restrict__ in, Field3 fd,
+                                                             unsigned maxbits, uint64_t* __restrict__ stream)
+{
+  extern __shared__ uint4 lds_raw[];
+  uint32_t* lds = reinterpret_cast<uint32_t*>(lds_raw);
+  const unsigned lane = threadIdx.x;
+  const uint32_t first = blockIdx.x * 64u;
+  const uint32_t valid = min(64u, fd.nblocks - first);
+  zero_region(lds_raw, lane, maxbits);
+  __syncthreads();
+  if (lane < valid) {
+    uint64_t q[64];
+    load_block_w64(in, fd, first + lane, q);
+    LdsBits mem{lds};
+    encode_block_w64<!WHOLE, INT>(q, lane * slot_bits(maxbits), maxbits, mem);
+  }
+  __syncthreads();
+  store_region<WHOLE>(lds, lane, first, valid, maxbits, fd.stream16, stream);
+}
+
+template <bool WHOLE, bool INT>
+__global__ __launch_bounds__(64) void zfp_decode3_w64_kernel(const uint64_t* __restrict__ stream, Field3 fd,
+                                                             unsigned maxbits, uint64_t* __restrict__ out)
+{
+  extern __shared__ uint4 lds_raw[];
+  uint32_t* lds = reinterpret_cast<uint32_t*>(lds_raw);
+  const unsigned lane = threadIdx.x;
+  const uint32_t first = blockIdx.x * 64u;
+  const uint32_t valid = min(64u, fd.nblocks - first);
+  load_region<WHOLE>(lds, lane, first, valid, maxbits, fd.stream16, stream);
+  __syncthreads();
+  if (lane < valid) {
+    uint64_t q[64];
+    LdsBits mem{lds};
+    decode_block_w64<INT, WHOLE>(mem, lane * slot_bits(maxbits), maxbits, q);
+    store_block_w64(out, fd, first + lane, q);
   }
 }
 
@@ -384,13 +509,87 @@ __global__ __launch_bounds__(64) void zfp_decode_low_f32_kernel(const uint64_t* 
   }
 }
 
+// 64-bit elements, 2-D / 1-D
+template <int DIMS, bool INT>
+__global__ __launch_bounds__(64) void zfp_encode_low_w64_kernel(const uint64_t* __restrict__ in, FieldLow fd,
+                                                                unsigned maxbits, uint64_t* __restrict__ stream)
+{
+  extern __shared__ uint4 lds_raw[];
+  uint32_t* lds = reinterpret_cast<uint32_t*>(lds_raw);
+  const unsigned lane = threadIdx.x;
+  const uint32_t first = blockIdx.x * 64u;
+  const uint32_t valid = min(64u, fd.nblocks - first);
+  const unsigned n16 = (2u * maxbits + 4u + 3u) / 4u;
+  for (unsigned i = lane; i < n16; i += 64) lds_raw[i] = make_uint4(0, 0, 0, 0);
+  __syncthreads();
+  if (lane < valid) {
+    const uint32_t b = first + lane;
+    const uint32_t r = b / fd.mx;
+    const uint32_t x0 = (b - r * fd.mx) * 4, y0 = DIMS == 2 ? r * 4 : 0;
+    const uint64_t* p = in + (long long)x0 * fd.sx + (long long)y0 * fd.sy;
+    const uint32_t bx = min(4u, fd.nx - x0), by = DIMS == 2 ? min(4u, fd.ny - y0) : 1u;
+    uint64_t q[16];
+#pragma unroll
+    for (int y = 0; y < 4; y++)
+#pragma unroll
+      for (int x = 0; x < 4; x++) {
+        bool ok = (uint32_t)x < bx && (uint32_t)y < by;
+        q[4 * y + x] = ok ? p[x * fd.sx + y * fd.sy] : 0ull;
+      }
+#pragma unroll
+    for (int y = 0; y < (DIMS == 2 ? 4 : 1); y++) pad4(q[4 * y], q[4 * y + 1], q[4 * y + 2], q[4 * y + 3], bx);
+    if (DIMS == 2) {
+#pragma unroll
+      for (int x = 0; x < 4; x++) pad4(q[x], q[x + 4], q[x + 8], q[x + 12], by);
+    }
+    LdsBits mem{lds};
+    encode_block_low_w64<DIMS, true, INT>(q, lane * maxbits, maxbits, mem);
+  }
+  __syncthreads();
+  const unsigned nwords = (valid * maxbits + 63u) >> 6;
+  const uint64_t* src = reinterpret_cast<const uint64_t*>(lds);
+  uint64_t* dst = stream + (size_t)blockIdx.x * maxbits;
+  for (unsigned i = lane; i < nwords; i += 64) dst[i] = src[i];
+}
+
+template <int DIMS, bool INT>
+__global__ __launch_bounds__(64) void zfp_decode_low_w64_kernel(const uint64_t* __restrict__ stream, FieldLow fd,
+                                                                unsigned maxbits, uint64_t* __restrict__ out)
+{
+  extern __shared__ uint4 lds_raw[];
+  uint32_t* lds = reinterpret_cast<uint32_t*>(lds_raw);
+  const unsigned lane = threadIdx.x;
+  const uint32_t first = blockIdx.x * 64u;
+  const uint32_t valid = min(64u, fd.nblocks - first);
+  const unsigned nwords = (valid * maxbits + 63u) >> 6;
+  const uint64_t* src = stream + (size_t)blockIdx.x * maxbits;
+  uint64_t* dst = reinterpret_cast<uint64_t*>(lds);
+  for (unsigned i = lane; i < nwords + 2; i += 64) dst[i] = i < nwords ? src[i] : 0;
+  __syncthreads();
+  if (lane < valid) {
+    uint64_t q[16];
+    LdsBits mem{lds};
+    decode_block_low_w64<DIMS, INT>(mem, lane * maxbits, maxbits, q);
+    const uint32_t b = first + lane;
+    const uint32_t r = b / fd.mx;
+    const uint32_t x0 = (b - r * fd.mx) * 4, y0 = DIMS == 2 ? r * 4 : 0;
+    uint64_t* p = out + (long long)x0 * fd.sx + (long long)y0 * fd.sy;
+    const uint32_t bx = min(4u, fd.nx - x0), by = DIMS == 2 ? min(4u, fd.ny - y0) : 1u;
+#pragma unroll
+    for (int y = 0; y < 4; y++)
+#pragma unroll
+      for (int x = 0; x < 4; x++)
+        if ((uint32_t)x < bx && (uint32_t)y < by) p[x * fd.sx + y * fd.sy] = q[4 * y + x];
+  }
+}
+
 static int make_field_low(FieldLow& fd, int dims, const void* base, const void* stream, size_t nx, size_t ny,
-                          ptrdiff_t sx, ptrdiff_t sy, unsigned maxbits)
+                          ptrdiff_t sx, ptrdiff_t sy, unsigned maxbits, unsigned elem)
 {
   if (dims == 1) ny = 1;
   if (!nx || !ny || maxbits < 16 || maxbits > 4096) return CSWAP_E_ARG;
   if (nx > 0x7fffffffu || ny > 0x7fffffffu) return CSWAP_E_ARG;
-  if (((uintptr_t)stream % 8) != 0 || ((uintptr_t)base % 4) != 0) return CSWAP_E_ARG;
+  if (((uintptr_t)stream % 8) != 0 || ((uintptr_t)base % elem) != 0) return CSWAP_E_ARG;
   size_t mx = (nx + 3) / 4, my = dims == 2 ? (ny + 3) / 4 : 1;
   size_t nb = mx * my;
   if (nb > 0xfffffff0ull) return CSWAP_E_ARG;
@@ -402,9 +601,9 @@ static int make_field_low(FieldLow& fd, int dims, const void* base, const void* 
 
 // ------------------------------------------------------------- host side
 static int make_field(Field3& fd, const void* base, const void* stream, size_t nx, size_t ny, size_t nz,
-                      ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits)
+                      ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, unsigned elem)
 {
-  if (((uintptr_t)stream % 8) != 0 || ((uintptr_t)base % 4) != 0) return CSWAP_E_ARG;
+  if (((uintptr_t)stream % 8) != 0 || ((uintptr_t)base % elem) != 0) return CSWAP_E_ARG;
   if (!nx || !ny || !nz) return CSWAP_E_ARG;
   if (maxbits < 16 || maxbits > 4096) return CSWAP_E_ARG;
   if (nx > 0x7fffffffu || ny > 0x7fffffffu || nz > 0x7fffffffu) return CSWAP_E_ARG;
@@ -424,9 +623,10 @@ static int make_field(Field3& fd, const void* base, const void* stream, size_t n
   // 64 consecutive blocks can touch (one more than they fill) stay below 4 GiB, so
   // every block of a wavefront is within a 32-bit byte offset of its first block
   const size_t slabs = (64 + mx * my - 1) / (mx * my) + 1;
-  fd.rows16 = fd.sx == 1 && (fd.sy % 4) == 0 && (fd.sz % 4) == 0 && ((uintptr_t)base % 16) == 0 &&
+  const ptrdiff_t per16 = (ptrdiff_t)(16 / elem);  // elements in 16 bytes
+  fd.rows16 = fd.sx == 1 && (fd.sy % per16) == 0 && (fd.sz % per16) == 0 && ((uintptr_t)base % 16) == 0 &&
               fd.sy >= (ptrdiff_t)nx && fd.sz >= fd.sy * (ptrdiff_t)ny &&
-              (unsigned long long)fd.sz * 16ull * slabs < 0xfff00000ull;
+              (unsigned long long)fd.sz * 4ull * elem * slabs < 0xfff00000ull;
   fd.stream16 = ((uintptr_t)stream % 16) == 0;
   return CSWAP_OK;
 }
@@ -447,65 +647,79 @@ extern "C" size_t cswap_zfp_stream_capacity(size_t nx, size_t ny, size_t nz, uns
   return ((nb * maxbits + 63) / 64) * 8;
 }
 
-// d_in / d_out are fields of 32-bit elements: fp32, or int32 when is_int
-static int compress3(const void* d_in, bool is_int, size_t nx, size_t ny, size_t nz, ptrdiff_t sx, ptrdiff_t sy,
+// element kinds of a field
+enum Elem { kF32 = 0, kI32 = 1, kF64 = 2, kI64 = 3 };
+static unsigned elem_bytes(Elem e) { return e == kF32 || e == kI32 ? 4u : 8u; }
+
+#define CSWAP_LAUNCH3(KERNEL_, T_, ARG0_, ARG3_)                                                                   \
+  do {                                                                                                              \
+    if (whole && !is_int)                                                                                           \
+      hipLaunchKernelGGL((KERNEL_<true, false>), dim3(grid), dim3(64), lds_bytes, st, ARG0_, fd, maxbits, ARG3_);   \
+    else if (!whole && !is_int)                                                                                     \
+      hipLaunchKernelGGL((KERNEL_<false, false>), dim3(grid), dim3(64), lds_bytes, st, ARG0_, fd, maxbits, ARG3_);  \
+    else if (whole)                                                                                                 \
+      hipLaunchKernelGGL((KERNEL_<true, true>), dim3(grid), dim3(64), lds_bytes, st, ARG0_, fd, maxbits, ARG3_);    \
+    else                                                                                                            \
+      hipLaunchKernelGGL((KERNEL_<false, true>), dim3(grid), dim3(64), lds_bytes, st, ARG0_, fd, maxbits, ARG3_);   \
+  } while (0)
+
+static int compress3(const void* d_in, Elem elem, size_t nx, size_t ny, size_t nz, ptrdiff_t sx, ptrdiff_t sy,
                      ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream, cswap_stream_t stream)
 {
   if (!d_in || !d_stream) return CSWAP_E_ARG;
   Field3 fd;
-  int rc = make_field(fd, d_in, d_stream, nx, ny, nz, sx, sy, sz, maxbits);
+  int rc = make_field(fd, d_in, d_stream, nx, ny, nz, sx, sy, sz, maxbits, elem_bytes(elem));
   if (rc) return rc;
-  const float* in = static_cast<const float*>(d_in);
   unsigned grid = (fd.nblocks + 63) / 64;
   size_t lds_bytes = (size_t)region_dwords(maxbits) * 4;
   hipStream_t st = (hipStream_t)stream;
   const bool whole = (maxbits & 63u) == 0;
-  if (whole && !is_int)
-    hipLaunchKernelGGL((zfp_encode3_f32_kernel<true, false>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
-  else if (!whole && !is_int)
-    hipLaunchKernelGGL((zfp_encode3_f32_kernel<false, false>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
-  else if (whole)
-    hipLaunchKernelGGL((zfp_encode3_f32_kernel<true, true>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
-  else
-    hipLaunchKernelGGL((zfp_encode3_f32_kernel<false, true>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
+  const bool is_int = elem == kI32 || elem == kI64;
+  if (elem_bytes(elem) == 4) {
+    const float* in = static_cast<const float*>(d_in);
+    CSWAP_LAUNCH3(zfp_encode3_f32_kernel, float, in, d_stream);
+  } else {
+    const uint64_t* in = static_cast<const uint64_t*>(d_in);
+    CSWAP_LAUNCH3(zfp_encode3_w64_kernel, uint64_t, in, d_stream);
+  }
   return check_launch();
 }
 
-static int decompress3(const uint64_t* d_stream, bool is_int, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
+static int decompress3(const uint64_t* d_stream, Elem elem, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
                        ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, void* d_out, cswap_stream_t stream)
 {
   if (!d_out || !d_stream) return CSWAP_E_ARG;
   Field3 fd;
-  int rc = make_field(fd, d_out, d_stream, nx, ny, nz, sx, sy, sz, maxbits);
+  int rc = make_field(fd, d_out, d_stream, nx, ny, nz, sx, sy, sz, maxbits, elem_bytes(elem));
   if (rc) return rc;
-  float* out = static_cast<float*>(d_out);
   unsigned grid = (fd.nblocks + 63) / 64;
   size_t lds_bytes = (size_t)region_dwords(maxbits) * 4;
   hipStream_t st = (hipStream_t)stream;
   const bool whole = (maxbits & 63u) == 0;
-  if (whole && !is_int)
-    hipLaunchKernelGGL((zfp_decode3_f32_kernel<true, false>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
-  else if (!whole && !is_int)
-    hipLaunchKernelGGL((zfp_decode3_f32_kernel<false, false>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
-  else if (whole)
-    hipLaunchKernelGGL((zfp_decode3_f32_kernel<true, true>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
-  else
-    hipLaunchKernelGGL((zfp_decode3_f32_kernel<false, true>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
+  const bool is_int = elem == kI32 || elem == kI64;
+  if (elem_bytes(elem) == 4) {
+    float* out = static_cast<float*>(d_out);
+    CSWAP_LAUNCH3(zfp_decode3_f32_kernel, float, d_stream, out);
+  } else {
+    uint64_t* out = static_cast<uint64_t*>(d_out);
+    CSWAP_LAUNCH3(zfp_decode3_w64_kernel, uint64_t, d_stream, out);
+  }
   return check_launch();
 }
+#undef CSWAP_LAUNCH3
 
 extern "C" int cswap_zfp_compress_f32(const float* d_in, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
                                       ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream,
                                       cswap_stream_t stream)
 {
-  return compress3(d_in, false, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
+  return compress3(d_in, kF32, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
 }
 
 extern "C" int cswap_zfp_decompress_f32(const uint64_t* d_stream, size_t nx, size_t ny, size_t nz,
                                         ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
                                         float* d_out, cswap_stream_t stream)
 {
-  return decompress3(d_stream, false, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
+  return decompress3(d_stream, kF32, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
 }
 
 // ------------------------------------------------------------- any dimensionality
@@ -530,77 +744,116 @@ extern "C" size_t cswap_zfp_stream_bytes_nd(int dims, size_t nx, size_t ny, size
   return cswap_zfp_stream_capacity_nd(dims, nx, ny, nz, maxbits);  // 1-D and 2-D round up (zfp/shared.h:42-71)
 }
 
-static int compress_nd(const void* d_in, bool is_int, int dims, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
+#define CSWAP_LAUNCH_LOW(KERNEL_, ARG0_, ARG3_)                                                                  \
+  do {                                                                                                             \
+    if (dims == 2 && !is_int)                                                                                      \
+      hipLaunchKernelGGL((KERNEL_<2, false>), dim3(grid), dim3(64), lds_bytes, st, ARG0_, fd, maxbits, ARG3_);     \
+    else if (dims == 2)                                                                                            \
+      hipLaunchKernelGGL((KERNEL_<2, true>), dim3(grid), dim3(64), lds_bytes, st, ARG0_, fd, maxbits, ARG3_);      \
+    else if (!is_int)                                                                                              \
+      hipLaunchKernelGGL((KERNEL_<1, false>), dim3(grid), dim3(64), lds_bytes, st, ARG0_, fd, maxbits, ARG3_);     \
+    else                                                                                                           \
+      hipLaunchKernelGGL((KERNEL_<1, true>), dim3(grid), dim3(64), lds_bytes, st, ARG0_, fd, maxbits, ARG3_);      \
+  } while (0)
+
+static int compress_nd(const void* d_in, Elem elem, int dims, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
                        ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream, cswap_stream_t stream)
 {
-  if (dims == 3) return compress3(d_in, is_int, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
+  if (dims == 3) return compress3(d_in, elem, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
   if (!d_in || !d_stream || (dims != 1 && dims != 2)) return CSWAP_E_ARG;
   FieldLow fd;
-  int rc = make_field_low(fd, dims, d_in, d_stream, nx, ny, sx, sy, maxbits);
+  int rc = make_field_low(fd, dims, d_in, d_stream, nx, ny, sx, sy, maxbits, elem_bytes(elem));
   if (rc) return rc;
-  const float* in = static_cast<const float*>(d_in);
   unsigned grid = (fd.nblocks + 63) / 64;
   size_t lds_bytes = (size_t)((2u * maxbits + 4u + 3u) / 4u) * 16;
   hipStream_t st = (hipStream_t)stream;
-  if (dims == 2 && !is_int)
-    hipLaunchKernelGGL((zfp_encode_low_f32_kernel<2, false>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
-  else if (dims == 2)
-    hipLaunchKernelGGL((zfp_encode_low_f32_kernel<2, true>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
-  else if (!is_int)
-    hipLaunchKernelGGL((zfp_encode_low_f32_kernel<1, false>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
-  else
-    hipLaunchKernelGGL((zfp_encode_low_f32_kernel<1, true>), dim3(grid), dim3(64), lds_bytes, st, in, fd, maxbits, d_stream);
+  const bool is_int = elem == kI32 || elem == kI64;
+  if (elem_bytes(elem) == 4) {
+    const float* in = static_cast<const float*>(d_in);
+    CSWAP_LAUNCH_LOW(zfp_encode_low_f32_kernel, in, d_stream);
+  } else {
+    const uint64_t* in = static_cast<const uint64_t*>(d_in);
+    CSWAP_LAUNCH_LOW(zfp_encode_low_w64_kernel, in, d_stream);
+  }
   return check_launch();
 }
 
-static int decompress_nd(const uint64_t* d_stream, bool is_int, int dims, size_t nx, size_t ny, size_t nz,
+static int decompress_nd(const uint64_t* d_stream, Elem elem, int dims, size_t nx, size_t ny, size_t nz,
                          ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, void* d_out,
                          cswap_stream_t stream)
 {
-  if (dims == 3) return decompress3(d_stream, is_int, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
+  if (dims == 3) return decompress3(d_stream, elem, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
   if (!d_out || !d_stream || (dims != 1 && dims != 2)) return CSWAP_E_ARG;
   FieldLow fd;
-  int rc = make_field_low(fd, dims, d_out, d_stream, nx, ny, sx, sy, maxbits);
+  int rc = make_field_low(fd, dims, d_out, d_stream, nx, ny, sx, sy, maxbits, elem_bytes(elem));
   if (rc) return rc;
-  float* out = static_cast<float*>(d_out);
   unsigned grid = (fd.nblocks + 63) / 64;
   size_t lds_bytes = (size_t)((2u * maxbits + 4u + 3u) / 4u) * 16;
   hipStream_t st = (hipStream_t)stream;
-  if (dims == 2 && !is_int)
-    hipLaunchKernelGGL((zfp_decode_low_f32_kernel<2, false>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
-  else if (dims == 2)
-    hipLaunchKernelGGL((zfp_decode_low_f32_kernel<2, true>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
-  else if (!is_int)
-    hipLaunchKernelGGL((zfp_decode_low_f32_kernel<1, false>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
-  else
-    hipLaunchKernelGGL((zfp_decode_low_f32_kernel<1, true>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd, maxbits, out);
+  const bool is_int = elem == kI32 || elem == kI64;
+  if (elem_bytes(elem) == 4) {
+    float* out = static_cast<float*>(d_out);
+    CSWAP_LAUNCH_LOW(zfp_decode_low_f32_kernel, d_stream, out);
+  } else {
+    uint64_t* out = static_cast<uint64_t*>(d_out);
+    CSWAP_LAUNCH_LOW(zfp_decode_low_w64_kernel, d_stream, out);
+  }
   return check_launch();
 }
+#undef CSWAP_LAUNCH_LOW
 
 extern "C" int cswap_zfp_compress_f32_nd(const float* d_in, int dims, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
                                          ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream,
                                          cswap_stream_t stream)
 {
-  return compress_nd(d_in, false, dims, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
+  return compress_nd(d_in, kF32, dims, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
 }
 
 extern "C" int cswap_zfp_decompress_f32_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
                                            ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, float* d_out,
                                            cswap_stream_t stream)
 {
-  return decompress_nd(d_stream, false, dims, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
+  return decompress_nd(d_stream, kF32, dims, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
 }
 
 extern "C" int cswap_zfp_compress_i32_nd(const int32_t* d_in, int dims, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
                                          ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream,
                                          cswap_stream_t stream)
 {
-  return compress_nd(d_in, true, dims, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
+  return compress_nd(d_in, kI32, dims, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
 }
 
 extern "C" int cswap_zfp_decompress_i32_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
                                            ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
                                            int32_t* d_out, cswap_stream_t stream)
 {
-  return decompress_nd(d_stream, true, dims, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
+  return decompress_nd(d_stream, kI32, dims, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
+}
+
+extern "C" int cswap_zfp_compress_f64_nd(const double* d_in, int dims, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
+                                         ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream,
+                                         cswap_stream_t stream)
+{
+  return compress_nd(d_in, kF64, dims, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
+}
+
+extern "C" int cswap_zfp_decompress_f64_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
+                                           ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, double* d_out,
+                                           cswap_stream_t stream)
+{
+  return decompress_nd(d_stream, kF64, dims, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
+}
+
+extern "C" int cswap_zfp_compress_i64_nd(const int64_t* d_in, int dims, size_t nx, size_t ny, size_t nz, ptrdiff_t sx,
+                                         ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, uint64_t* d_stream,
+                                         cswap_stream_t stream)
+{
+  return compress_nd(d_in, kI64, dims, nx, ny, nz, sx, sy, sz, maxbits, d_stream, stream);
+}
+
+extern "C" int cswap_zfp_decompress_i64_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
+                                           ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
+                                           int64_t* d_out, cswap_stream_t stream)
+{
+  return decompress_nd(d_stream, kI64, dims, nx, ny, nz, sx, sy, sz, maxbits, d_out, stream);
 }

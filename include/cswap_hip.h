@@ -81,13 +81,32 @@ int cswap_zfp_decompress_f32_nd(const uint64_t* d_stream, int dims, size_t nx, s
  * zfp/cuZFP.cu:412-416,513-517): the same transform and coder applied to the
  * values themselves -- no exponent header, no cast, the whole maxbits is the
  * coder's budget (zfp/encode.cuh:371-380,393-402,415-424).  Same stream sizes as
- * above.  64-bit scalar types (double, int64) are not implemented. */
+ * above. */
 int cswap_zfp_compress_i32_nd(const int32_t* d_in, int dims, size_t nx, size_t ny, size_t nz,
                               ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
                               uint64_t* d_stream, cswap_stream_t stream);
 int cswap_zfp_decompress_i32_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
                                 ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
                                 int32_t* d_out, cswap_stream_t stream);
+/* double and int64 fields (zfp_type_double, zfp_type_int64 in cuda_compress /
+ * cuda_decompress, zfp/cuZFP.cu:401-411,418-423,479-504): 64 bit planes over
+ * int64 coefficients; doubles carry a 12-bit block header (flag + 11-bit
+ * exponent, zfp/type_info.cuh:8-17) and are scaled by 2^(62-emax)
+ * (zfp/encode.cuh:136-149); int64 has no header.  Strides are in elements;
+ * d_in / d_out must be 8-byte aligned.  maxbits counts bits per block of 4^dims
+ * values as above (so a rate of r bits per value is maxbits = r * 4^dims). */
+int cswap_zfp_compress_f64_nd(const double* d_in, int dims, size_t nx, size_t ny, size_t nz,
+                              ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
+                              uint64_t* d_stream, cswap_stream_t stream);
+int cswap_zfp_decompress_f64_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
+                                ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
+                                double* d_out, cswap_stream_t stream);
+int cswap_zfp_compress_i64_nd(const int64_t* d_in, int dims, size_t nx, size_t ny, size_t nz,
+                              ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
+                              uint64_t* d_stream, cswap_stream_t stream);
+int cswap_zfp_decompress_i64_nd(const uint64_t* d_stream, int dims, size_t nx, size_t ny, size_t nz,
+                                ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
+                                int64_t* d_out, cswap_stream_t stream);
 
 /* ------------------------------------------------------------------ ZVC -----
  * Zero-value compaction in the reference's format (zfp/compression.cu).  The

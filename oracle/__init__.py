@@ -58,6 +58,10 @@ def _sig(lib: C.CDLL) -> C.CDLL:
     lib.orc_zfp_encode_i32.argtypes = [vp, i, sz, sz, sz, pd, pd, pd, u, vp]
     lib.orc_zfp_decode_i32.restype = None
     lib.orc_zfp_decode_i32.argtypes = [vp, i, sz, sz, sz, pd, pd, pd, u, vp]
+    lib.orc_zfp_encode_64.restype = sz
+    lib.orc_zfp_encode_64.argtypes = [vp, i, i, sz, sz, sz, pd, pd, pd, u, vp]
+    lib.orc_zfp_decode_64.restype = None
+    lib.orc_zfp_decode_64.argtypes = [vp, i, i, sz, sz, sz, pd, pd, pd, u, vp]
     lib.orc_zfp_encode_block_f32.restype = None
     lib.orc_zfp_encode_block_f32.argtypes = [vp, u, sz, vp]
     lib.orc_zfp_decode_block_f32.restype = None
@@ -189,6 +193,29 @@ def zfp_decode_i32(stream: np.ndarray, shape, maxbits: int) -> np.ndarray:
     s[: w.size] = w
     out = np.zeros(tuple(shape), dtype=np.int32)
     lib().orc_zfp_decode_i32(_p(s), dims, nx, ny, nz, 0, 0, 0, maxbits, _p(out))
+    return out
+
+
+def zfp_encode_64(field: np.ndarray, maxbits: int) -> np.ndarray:
+    """1-D, 2-D or 3-D C-contiguous float64 or int64 field (x fastest) -> stream words."""
+    assert field.dtype in (np.float64, np.int64) and field.flags.c_contiguous and 1 <= field.ndim <= 3
+    dims, nx, ny, nz = _dims3(field.shape)
+    blocks = int(np.prod([(n + 3) // 4 for n in field.shape]))
+    out = np.zeros((blocks * maxbits + 63) // 64 + 1, dtype=np.uint64)
+    lib().orc_zfp_encode_64(_p(field), int(field.dtype == np.int64), dims, nx, ny, nz, 0, 0, 0, maxbits, _p(out))
+    return out[:-1]
+
+
+def zfp_decode_64(stream: np.ndarray, shape, maxbits: int, dtype) -> np.ndarray:
+    dtype = np.dtype(dtype)
+    assert dtype in (np.float64, np.int64)
+    dims, nx, ny, nz = _dims3(shape)
+    blocks = int(np.prod([(n + 3) // 4 for n in shape]))
+    s = np.zeros((blocks * maxbits + 63) // 64 + 1, dtype=np.uint64)
+    w = np.ascontiguousarray(stream).view(np.uint64)
+    s[: w.size] = w
+    out = np.zeros(tuple(shape), dtype=dtype)
+    lib().orc_zfp_decode_64(_p(s), int(dtype == np.int64), dims, nx, ny, nz, 0, 0, 0, maxbits, _p(out))
     return out
 
 

@@ -27,11 +27,16 @@
  *   orc_perm3 : permutation sorted by (i+j+k, i^2+j^2+k^2).
  *   orc_zfp_encode2/decode2/encode1/decode1 : byte-exact against zfp 0.5.5 2-D and
  *       1-D golden vectors (tests/golden/zfp_golden_12d.npz).
+ *   orc_zfp_encode_i32 / orc_zfp_decode_i32 : byte-exact against zfp 0.5.5 -t i32
+ *       vectors of 1, 2 and 3 dimensions (tests/golden/zfp_golden_i32.npz).
+ *   orc_zfp_encode_64 / orc_zfp_decode_64 : byte-exact against zfp 0.5.5 -d and
+ *       -t i64 vectors of 1, 2 and 3 dimensions (tests/golden/zfp_golden_64.npz).
  *   orc_zvc_* : numpy boolean indexing / packbits / cumsum.
  *
  * Undefined in the reference and therefore unpinned here: blocks whose largest
  * magnitude is non-zero but below 2^-97 (the float scale factor 2^(30-emax)
- * overflows, CSWAP+/zfp/encode.cuh:127-132), NaN/Inf inputs to the ZFP path,
+ * overflows, CSWAP+/zfp/encode.cuh:127-132; for doubles below 2^-961, where in
+ * addition the cast to int64 is made saturating here), NaN/Inf inputs to the ZFP path,
  * and ZVC mask words past the end of a partially filled last chunk.
  */
 #include <math.h>
@@ -669,6 +674,285 @@ void orc_zfp_decode_i32(const word_t *stream, int dims, size_t nx, size_t ny, si
         memset(q, 0, sizeof q);
         decode_block_i32(stream, dims, maxbits, b, q);
         int32_t *p = out + (ptrdiff_t)x0 * sx + (ptrdiff_t)y0 * sy + (ptrdiff_t)z0 * sz;
+        for (unsigned z = 0; z < bz; z++)
+            for (unsigned y = 0; y < by; y++)
+                for (unsigned x = 0; x < bx; x++) p[x * sx + y * sy + z * sz] = q[16 * z + 4 * y + x];
+    }
+}
+
+/* ------------------------------------------------------------------------ */
+/* 64-bit element types (zfp_type_double, zfp_type_int64; cuZFP.cu:401-423,   */
+/* 479-504).  Same structure with 64-bit integers and 64 bit planes:          */
+/*   double: 12 header bits (flag + 11-bit biased exponent, type_info.cuh:8-17),*/
+/*           scale 2^(62-emax) (encode.cuh:136-149), block precision           */
+/*           min(64, emax + 1074 + 8) (encode.cuh:10-15 -- the "+ 8" is used   */
+/*           for every dimensionality), so blocks whose largest magnitude is   */
+/*           below 2^-1018 code fewer than 64 planes; the decoder always reads */
+/*           down to plane 0 (decode.cuh:131-133), which finds zero bits there.*/
+/*   int64 : no header, no cast (encode.cuh:382-391 and the 1-D/2-D twins).    */
+/* Conversions double -> int64 saturate (what the reference's GPU does for the */
+/* overflowing scale of near-subnormal blocks; C leaves them undefined).      */
+/* Values travel as 64-bit patterns.                                          */
+/* ------------------------------------------------------------------------ */
+
+#define NB64 0xaaaaaaaaaaaaaaaaull
+
+static inline int64_t wadd64(int64_t a, int64_t b) { return (int64_t)((uint64_t)a + (uint64_t)b); }
+static inline int64_t wsub64(int64_t a, int64_t b) { return (int64_t)((uint64_t)a - (uint64_t)b); }
+static inline int64_t wshl64(int64_t a) { return (int64_t)((uint64_t)a << 1); }
+static inline int64_t asr64(int64_t a) { return a >> 1; }
+
+static void fwd_lift64(int64_t *p, ptrdiff_t s)
+{
+    int64_t x = p[0], y = p[s], z = p[2 * s], w = p[3 * s];
+    x = wadd64(x, w); x = asr64(x); w = wsub64(w, x);
+    z = wadd64(z, y); z = asr64(z); y = wsub64(y, z);
+    x = wadd64(x, z); x = asr64(x); z = wsub64(z, x);
+    w = wadd64(w, y); w = asr64(w); y = wsub64(y, w);
+    w = wadd64(w, asr64(y)); y = wsub64(y, asr64(w));
+    p[0] = x; p[s] = y; p[2 * s] = z; p[3 * s] = w;
+}
+
+static void inv_lift64(int64_t *p, ptrdiff_t s)
+{
+    int64_t x = p[0], y = p[s], z = p[2 * s], w = p[3 * s];
+    y = wadd64(y, asr64(w)); w = wsub64(w, asr64(y));
+    y = wadd64(y, w); w = wshl64(w); w = wsub64(w, y);
+    z = wadd64(z, x); x = wshl64(x); x = wsub64(x, z);
+    y = wadd64(y, z); z = wshl64(z); z = wsub64(z, y);
+    w = wadd64(w, x); x = wshl64(x); x = wsub64(x, w);
+    p[0] = x; p[s] = y; p[2 * s] = z; p[3 * s] = w;
+}
+
+static void fwd_xform64(int64_t *b, int dims)
+{
+    int x, y, z;
+    if (dims == 3) {
+        for (z = 0; z < 4; z++) for (y = 0; y < 4; y++) fwd_lift64(b + 4 * y + 16 * z, 1);
+        for (x = 0; x < 4; x++) for (z = 0; z < 4; z++) fwd_lift64(b + 16 * z + x, 4);
+        for (y = 0; y < 4; y++) for (x = 0; x < 4; x++) fwd_lift64(b + x + 4 * y, 16);
+    } else if (dims == 2) {
+        for (y = 0; y < 4; y++) fwd_lift64(b + 4 * y, 1);
+        for (x = 0; x < 4; x++) fwd_lift64(b + x, 4);
+    } else {
+        fwd_lift64(b, 1);
+    }
+}
+
+static void inv_xform64(int64_t *b, int dims)
+{
+    int x, y, z;
+    if (dims == 3) {
+        for (y = 0; y < 4; y++) for (x = 0; x < 4; x++) inv_lift64(b + x + 4 * y, 16);
+        for (x = 0; x < 4; x++) for (z = 0; z < 4; z++) inv_lift64(b + 16 * z + x, 4);
+        for (z = 0; z < 4; z++) for (y = 0; y < 4; y++) inv_lift64(b + 4 * y + 16 * z, 1);
+    } else if (dims == 2) {
+        for (x = 0; x < 4; x++) inv_lift64(b + x, 4);
+        for (y = 0; y < 4; y++) inv_lift64(b + 4 * y, 1);
+    } else {
+        inv_lift64(b, 1);
+    }
+}
+
+/* the coder of encode.cuh:306-345 on 64-bit coefficients; planes below kmin are not coded */
+static void encode_ints64(bitcur *c, unsigned budget, const uint64_t *u, unsigned size, unsigned kmin)
+{
+    unsigned bits = budget;
+    unsigned n = 0;
+    for (int k = 63; k >= (int)kmin && bits; k--) {
+        word_t x = 0;
+        for (unsigned i = 0; i < size; i++) x |= (word_t)((u[i] >> k) & 1u) << i;
+        unsigned m = n < bits ? n : bits;
+        bits -= m;
+        put_bits(c, x, m);
+        x = (m < 64) ? (x >> m) : 0;
+        while (n < size && bits) {
+            bits--;
+            unsigned any = (x != 0);
+            put_bits(c, any, 1);
+            if (!any) break;
+            while (n < size - 1 && bits) {
+                bits--;
+                unsigned b = (unsigned)(x & 1u);
+                put_bits(c, b, 1);
+                if (b) break;
+                x >>= 1; n++;
+            }
+            x >>= 1; n++;
+        }
+    }
+}
+
+static void decode_ints64(bitcur *c, unsigned budget, uint64_t *u, unsigned size)
+{
+    unsigned bits = budget;
+    unsigned n = 0;
+    memset(u, 0, size * sizeof(uint64_t));
+    for (int k = 63; k >= 0 && bits; k--) {
+        unsigned m = n < bits ? n : bits;
+        bits -= m;
+        word_t x = get_bits(c, m);
+        while (bits && n < size) {
+            bits--;
+            if (!get_bit(c)) break;
+            while (bits && n < size - 1) {
+                bits--;
+                if (get_bit(c)) break;
+                n++;
+            }
+            x += (word_t)1 << n;
+            n++;
+        }
+        for (unsigned i = 0; i < size; i++, x >>= 1) u[i] += (uint64_t)(x & 1u) << k;
+    }
+}
+
+static int64_t sat_i64(double v)
+{
+    if (v != v) return 0;
+    if (v >= 9223372036854775808.0) return INT64_MAX;
+    if (v <= -9223372036854775808.0) return INT64_MIN;
+    return (int64_t)v;
+}
+
+static const unsigned char *perm_for(int dims)
+{
+    static const unsigned char ident[4] = { 0, 1, 2, 3 };
+    return dims == 3 ? PERM3 : dims == 2 ? PERM2 : ident;
+}
+
+/* q: the gathered and padded block as 64-bit patterns (overwritten) */
+static void encode_block_64(uint64_t *q, int is_int, int dims, unsigned maxbits, size_t block_idx, word_t *stream)
+{
+    const unsigned size = dims == 3 ? 64 : dims == 2 ? 16 : 4;
+    bitcur c = { stream, block_idx * (size_t)maxbits };
+    int64_t ib[64];
+    unsigned budget = maxbits, kmin = 0;
+    if (is_int) {
+        memcpy(ib, q, size * sizeof(int64_t));
+    } else {
+        double fb[64], m = 0.0;
+        memcpy(fb, q, size * sizeof(double));
+        for (unsigned i = 0; i < size; i++) m = fmax(m, fabs(fb[i]));
+        int emax = -1023;
+        if (m > 0.0) {
+            frexp(m, &emax);
+            if (emax < -1022) emax = -1022;
+        }
+        int maxprec = emax + 1074 + 8;
+        if (maxprec > 64) maxprec = 64;
+        if (maxprec < 0) maxprec = 0;
+        unsigned e = maxprec ? (unsigned)(emax + 1023) : 0;
+        if (!e) return;
+        put_bits(&c, 2 * (word_t)e + 1, 12);
+        budget = maxbits - 12;
+        kmin = 64 - (unsigned)maxprec;
+        double s = ldexp(1.0, 62 - emax);
+        for (unsigned i = 0; i < size; i++) ib[i] = sat_i64(s * fb[i]);
+    }
+    fwd_xform64(ib, dims);
+    const unsigned char *perm = perm_for(dims);
+    uint64_t ub[64];
+    for (unsigned i = 0; i < size; i++) ub[i] = ((uint64_t)ib[perm[i]] + NB64) ^ NB64;
+    encode_ints64(&c, budget, ub, size, kmin);
+}
+
+/* q receives the block as 64-bit patterns; an empty double block leaves it untouched */
+static void decode_block_64(const word_t *stream, int is_int, int dims, unsigned maxbits, size_t block_idx, uint64_t *q)
+{
+    const unsigned size = dims == 3 ? 64 : dims == 2 ? 16 : 4;
+    bitcur c = { (word_t *)stream, block_idx * (size_t)maxbits };
+    unsigned budget = maxbits;
+    int emax = 0;
+    if (!is_int) {
+        if (!get_bit(&c)) return;
+        emax = (int)get_bits(&c, 11) - 1023;
+        budget = maxbits - 12;
+    }
+    uint64_t ub[64];
+    int64_t ib[64];
+    decode_ints64(&c, budget, ub, size);
+    const unsigned char *perm = perm_for(dims);
+    for (unsigned i = 0; i < size; i++) ib[perm[i]] = (int64_t)((ub[i] ^ NB64) - NB64);
+    inv_xform64(ib, dims);
+    if (is_int) {
+        memcpy(q, ib, size * sizeof(int64_t));
+    } else {
+        double w = ldexp(1.0, emax - 62), fb[64];
+        for (unsigned i = 0; i < size; i++) fb[i] = w * (double)ib[i];
+        memcpy(q, fb, size * sizeof(double));
+    }
+}
+
+static void pad_vec_64(uint64_t *p, unsigned n, ptrdiff_t s)
+{
+    switch (n) {
+    case 0: p[0] = 0; /* fall through */
+    case 1: p[s] = p[0]; /* fall through */
+    case 2: p[2 * s] = p[s]; /* fall through */
+    case 3: p[3 * s] = p[0]; /* fall through */
+    default: break;
+    }
+}
+
+/* in: a[nz][ny][nx] of doubles (is_int 0) or int64 (is_int 1); strides in elements, 0 = contiguous */
+size_t orc_zfp_encode_64(const void *in_, int is_int, int dims, size_t nx, size_t ny, size_t nz,
+                         ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, word_t *stream)
+{
+    const uint64_t *in = (const uint64_t *)in_;
+    if (dims < 2) ny = 1;
+    if (dims < 3) nz = 1;
+    if (!sx) sx = 1;
+    if (!sy) sy = (ptrdiff_t)nx;
+    if (!sz) sz = (ptrdiff_t)(nx * ny);
+    size_t mx = pad4(nx) / 4, my = dims >= 2 ? pad4(ny) / 4 : 1, mz = dims >= 3 ? pad4(nz) / 4 : 1;
+    size_t blocks = mx * my * mz;
+    memset(stream, 0, ((blocks * (size_t)maxbits + 63) / 64) * sizeof(word_t));
+    for (size_t b = 0; b < blocks; b++) {
+        uint64_t q[64];
+        size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
+        unsigned bx = (unsigned)(nx - x0 < 4 ? nx - x0 : 4);
+        unsigned by = dims >= 2 ? (unsigned)(ny - y0 < 4 ? ny - y0 : 4) : 1;
+        unsigned bz = dims >= 3 ? (unsigned)(nz - z0 < 4 ? nz - z0 : 4) : 1;
+        const uint64_t *p = in + (ptrdiff_t)x0 * sx + (ptrdiff_t)y0 * sy + (ptrdiff_t)z0 * sz;
+        memset(q, 0, sizeof q);
+        for (unsigned z = 0; z < bz; z++) {
+            for (unsigned y = 0; y < by; y++) {
+                for (unsigned x = 0; x < bx; x++) q[16 * z + 4 * y + x] = p[x * sx + y * sy + z * sz];
+                pad_vec_64(q + 16 * z + 4 * y, bx, 1);
+            }
+            if (dims >= 2)
+                for (unsigned x = 0; x < 4; x++) pad_vec_64(q + 16 * z + x, by, 4);
+        }
+        if (dims >= 3)
+            for (unsigned y = 0; y < 4; y++)
+                for (unsigned x = 0; x < 4; x++) pad_vec_64(q + 4 * y + x, bz, 16);
+        encode_block_64(q, is_int, dims, maxbits, b, stream);
+    }
+    if (dims == 3) return orc_zfp_stream_bytes3(nx, ny, nz, maxbits);
+    return ((blocks * (size_t)maxbits + 63) / 64) * sizeof(word_t);
+}
+
+void orc_zfp_decode_64(const word_t *stream, int is_int, int dims, size_t nx, size_t ny, size_t nz,
+                       ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits, void *out_)
+{
+    uint64_t *out = (uint64_t *)out_;
+    if (dims < 2) ny = 1;
+    if (dims < 3) nz = 1;
+    if (!sx) sx = 1;
+    if (!sy) sy = (ptrdiff_t)nx;
+    if (!sz) sz = (ptrdiff_t)(nx * ny);
+    size_t mx = pad4(nx) / 4, my = dims >= 2 ? pad4(ny) / 4 : 1, mz = dims >= 3 ? pad4(nz) / 4 : 1;
+    size_t blocks = mx * my * mz;
+    for (size_t b = 0; b < blocks; b++) {
+        uint64_t q[64];
+        size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
+        unsigned bx = (unsigned)(nx - x0 < 4 ? nx - x0 : 4);
+        unsigned by = dims >= 2 ? (unsigned)(ny - y0 < 4 ? ny - y0 : 4) : 1;
+        unsigned bz = dims >= 3 ? (unsigned)(nz - z0 < 4 ? nz - z0 : 4) : 1;
+        memset(q, 0, sizeof q);
+        decode_block_64(stream, is_int, dims, maxbits, b, q);
+        uint64_t *p = out + (ptrdiff_t)x0 * sx + (ptrdiff_t)y0 * sy + (ptrdiff_t)z0 * sz;
         for (unsigned z = 0; z < bz; z++)
             for (unsigned y = 0; y < by; y++)
                 for (unsigned x = 0; x < bx; x++) p[x * sx + y * sy + z * sz] = q[16 * z + 4 * y + x];

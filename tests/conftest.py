@@ -34,6 +34,13 @@ def golden_i32():
 
 
 @pytest.fixture(scope="session")
+def golden_64():
+    import numpy as np
+
+    return np.load(os.path.join(ROOT, "tests", "golden", "zfp_golden_64.npz"))
+
+
+@pytest.fixture(scope="session")
 def digests():
     import json
 

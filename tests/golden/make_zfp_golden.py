@@ -15,6 +15,8 @@ Fixture contents
   zfp_golden_12d.npz  the same for 2-D (ny,nx) and 1-D (nx,) fields.
   zfp_golden_i32.npz  int32 fields of 1, 2 and 3 dimensions (``-t i32``); written
                    alone by ``make_zfp_golden.py --i32``.
+  zfp_golden_64.npz   float64 (``-d``) and int64 (``-t i64``) fields of 1, 2 and 3
+                   dimensions; written alone by ``make_zfp_golden.py --w64``.
   zfp_digests.json SHA-256 of input, stream and decoded output for the large
                    seeded configurations (inputs are re-created from the seed).
 """
@@ -37,8 +39,8 @@ from cswap_amd.workloads import config1_field, config3_fields  # noqa: E402
 def run_zfp(field: np.ndarray, rate: float):
     """field: (nz, ny, nx), (ny, nx) or (nx,) -- x is always the fastest axis."""
     dims = [str(n) for n in reversed(field.shape)]
-    is_int = field.dtype == np.int32
-    dt, flag = ("<i4", ["-t", "i32"]) if is_int else ("<f4", ["-f"])
+    dt, flag = {"int32": ("<i4", ["-t", "i32"]), "float32": ("<f4", ["-f"]),
+                "int64": ("<i8", ["-t", "i64"]), "float64": ("<f8", ["-d"])}[field.dtype.name]
     with tempfile.TemporaryDirectory() as d:
         fi, fz, fo = (os.path.join(d, n) for n in ("in.raw", "out.zfp", "out.raw"))
         field.astype(dt).tofile(fi)
@@ -84,6 +86,63 @@ def main_i32():
             out[f"{name}/r{r}/dec"] = dec
     np.savez_compressed(os.path.join(HERE, "zfp_golden_i32.npz"), **out)
     print("wrote", len(out), "int32 arrays")
+
+
+def wide_fields():
+    """float64 and int64 fields of 1, 2 and 3 dimensions."""
+    rng = np.random.default_rng(4242)
+    f = {}
+    f["d3_rand_8x8x8"] = rng.standard_normal((8, 8, 8))
+    f["d3_partial_7x5x6"] = rng.standard_normal((7, 5, 6)) * 1e3
+    z = rng.standard_normal((8, 8, 8))
+    z[0:4, 0:4, 0:4] = 0.0
+    z[4:8, 4:8, 4:8] = -7.5
+    z[0:4, 4:8, 0:4] = -0.0
+    f["d3_zero_const_blocks"] = z
+    g = np.arange(12, dtype=np.float64)
+    zz, yy, xx = np.meshgrid(g, g, g, indexing="ij")
+    f["d3_smooth_12"] = np.exp(-((xx - 5) ** 2 + (yy - 6) ** 2 + (zz - 4) ** 2) / 30)
+    w = rng.standard_normal((4, 8, 8)) * 2.0 ** rng.integers(-300, 300, size=(4, 8, 8))
+    f["d3_wide_range"] = w
+    f["d3_big_small"] = rng.standard_normal((4, 4, 8)) * np.array([1e250, 1e-250] * 4)
+    f["d3_nx2_ny2_8x2x2"] = rng.standard_normal((8, 2, 2))
+    f["d3_single"] = np.array([[[3.25]]])
+    f["d2_rand_8x12"] = rng.standard_normal((8, 12))
+    f["d2_partial_7x9"] = rng.standard_normal((7, 9)) * 1e-5
+    f["d2_smooth_20x20"] = np.exp(-((g[None, :] - 5) ** 2 + (g[:, None] - 6) ** 2) / 40)
+    f["d1_rand_64"] = rng.standard_normal(64)
+    o = rng.standard_normal(41)
+    o[8:16] = 0.0
+    f["d1_partial_zero_41"] = o
+    f["d1_smooth_100"] = np.sin(np.arange(100) / 9.0)
+    f["l3_rand_8x8x8"] = rng.integers(-2**40, 2**40, (8, 8, 8))
+    f["l3_partial_7x5x6"] = rng.integers(-1000, 1000, (7, 5, 6))
+    f["l3_wide_4x4x8"] = rng.integers(-2**61, 2**61, (4, 4, 8))
+    zi = rng.integers(-500, 500, (8, 8, 8))
+    zi[0:4, 0:4, 0:4] = 0
+    zi[4:8, 4:8, 4:8] = 123456789012
+    f["l3_zero_const_blocks"] = zi
+    f["l3_smooth_12"] = (1e15 * np.exp(-((xx - 5) ** 2 + (yy - 6) ** 2 + (zz - 4) ** 2) / 30)).astype(np.int64)
+    f["l2_rand_8x12"] = rng.integers(-2**50, 2**50, (8, 12))
+    f["l2_partial_7x9"] = rng.integers(-99, 99, (7, 9))
+    f["l1_rand_64"] = rng.integers(-2**60, 2**60, 64)
+    f["l1_partial_13"] = rng.integers(-5, 5, 13)
+    return {k: np.ascontiguousarray(v.astype(np.int64 if k[0] == "l" else np.float64)) for k, v in f.items()}
+
+
+RATES_64 = {3: [1, 2.5, 4, 8, 9.75, 16, 32, 48, 64], 2: [2, 4, 8, 12.5, 16, 32, 64], 1: [4, 8, 12, 16, 24, 32, 64]}
+
+
+def main_w64():
+    out = {}
+    for name, fld in wide_fields().items():
+        out[f"{name}/in"] = fld
+        for r in RATES_64[fld.ndim]:
+            stream, dec = run_zfp(fld, r)
+            out[f"{name}/r{r}/stream"] = stream
+            out[f"{name}/r{r}/dec"] = dec
+    np.savez_compressed(os.path.join(HERE, "zfp_golden_64.npz"), **out)
+    print("wrote", len(out), "64-bit arrays")
 
 
 def small_fields():
@@ -194,6 +253,9 @@ def main():
 if __name__ == "__main__":
     if "--i32" in sys.argv:
         main_i32()
+    elif "--w64" in sys.argv:
+        main_w64()
     else:
         main()
         main_i32()
+        main_w64()

@@ -175,4 +175,71 @@ void host_zfp_decode_i32(const uint64_t* stream, int dims, size_t nx, size_t ny,
 uint32_t host_div31(uint32_t b, uint32_t d) { return cswap::div31(b, cswap::make_div31(d)); }
 void host_transpose32(uint32_t* a) { uint32_t t[32]; memcpy(t, a, sizeof t); cswap::transpose32(t); memcpy(a, t, sizeof t); }
 
+
+// 64-bit element types: in / out are 64-bit patterns of doubles (is_int 0) or int64 (is_int 1);
+// dims 1..3, a[nz][ny][nx] contiguous
+void host_zfp_encode_w64(const uint64_t* in, int is_int, int dims, size_t nx, size_t ny, size_t nz, unsigned maxbits,
+                         uint64_t* stream)
+{
+  if (dims < 2) ny = 1;
+  if (dims < 3) nz = 1;
+  size_t mx = (nx + 3) / 4, my = dims >= 2 ? (ny + 3) / 4 : 1, mz = dims >= 3 ? (nz + 3) / 4 : 1;
+  for (size_t b = 0; b < mx * my * mz; b++) {
+    size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
+    unsigned bx = nx - x0 < 4 ? nx - x0 : 4, by = dims >= 2 ? (ny - y0 < 4 ? ny - y0 : 4) : 1,
+             bz = dims >= 3 ? (nz - z0 < 4 ? nz - z0 : 4) : 1;
+    uint64_t q[64];
+    for (int i = 0; i < 64; i++) q[i] = 0;
+    for (unsigned z = 0; z < bz; z++) for (unsigned y = 0; y < by; y++) for (unsigned x = 0; x < bx; x++)
+      q[x + 4 * y + 16 * z] = in[(x0 + x) + nx * ((y0 + y) + ny * (z0 + z))];
+    ArrayBits mem{reinterpret_cast<uint32_t*>(stream)};
+    const unsigned pos = (unsigned)(b * (size_t)maxbits);
+    if (dims == 3) {
+      if (bx < 4 || by < 4 || bz < 4) cswap::pad_block3(q, bx, by, bz);
+      if (is_int) cswap::encode_block_w64<true, true>(q, pos, maxbits, mem);
+      else cswap::encode_block_w64<true, false>(q, pos, maxbits, mem);
+    } else {
+      uint64_t r[16];
+      for (int i = 0; i < 16; i++) r[i] = q[i];
+      for (int y = 0; y < (dims == 2 ? 4 : 1); y++) cswap::pad4(r[4 * y], r[4 * y + 1], r[4 * y + 2], r[4 * y + 3], bx);
+      if (dims == 2)
+        for (int x = 0; x < 4; x++) cswap::pad4(r[x], r[x + 4], r[x + 8], r[x + 12], by);
+      if (dims == 2 && is_int) cswap::encode_block_low_w64<2, true, true>(r, pos, maxbits, mem);
+      else if (dims == 2) cswap::encode_block_low_w64<2, true, false>(r, pos, maxbits, mem);
+      else if (is_int) cswap::encode_block_low_w64<1, true, true>(r, pos, maxbits, mem);
+      else cswap::encode_block_low_w64<1, true, false>(r, pos, maxbits, mem);
+    }
+  }
+}
+
+void host_zfp_decode_w64(const uint64_t* stream, int is_int, int dims, size_t nx, size_t ny, size_t nz,
+                         unsigned maxbits, uint64_t* out)
+{
+  if (dims < 2) ny = 1;
+  if (dims < 3) nz = 1;
+  size_t mx = (nx + 3) / 4, my = dims >= 2 ? (ny + 3) / 4 : 1, mz = dims >= 3 ? (nz + 3) / 4 : 1;
+  for (size_t b = 0; b < mx * my * mz; b++) {
+    size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
+    unsigned bx = nx - x0 < 4 ? nx - x0 : 4, by = dims >= 2 ? (ny - y0 < 4 ? ny - y0 : 4) : 1,
+             bz = dims >= 3 ? (nz - z0 < 4 ? nz - z0 : 4) : 1;
+    uint64_t q[64];
+    for (int i = 0; i < 64; i++) q[i] = 0;
+    ArrayBits mem{reinterpret_cast<uint32_t*>(const_cast<uint64_t*>(stream))};
+    const unsigned pos = (unsigned)(b * (size_t)maxbits);
+    if (dims == 3) {
+      if (is_int) cswap::decode_block_w64<true>(mem, pos, maxbits, q);
+      else cswap::decode_block_w64<false>(mem, pos, maxbits, q);
+    } else {
+      uint64_t r[16];
+      if (dims == 2 && is_int) cswap::decode_block_low_w64<2, true>(mem, pos, maxbits, r);
+      else if (dims == 2) cswap::decode_block_low_w64<2, false>(mem, pos, maxbits, r);
+      else if (is_int) cswap::decode_block_low_w64<1, true>(mem, pos, maxbits, r);
+      else cswap::decode_block_low_w64<1, false>(mem, pos, maxbits, r);
+      for (int i = 0; i < 16; i++) q[i] = r[i];
+    }
+    for (unsigned z = 0; z < bz; z++) for (unsigned y = 0; y < by; y++) for (unsigned x = 0; x < bx; x++)
+      out[(x0 + x) + nx * ((y0 + y) + ny * (z0 + z))] = q[x + 4 * y + 16 * z];
+  }
+}
+
 }

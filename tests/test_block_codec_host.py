@@ -129,3 +129,60 @@ def test_int32_block_codec_matches_golden_vectors(host, golden_i32):
         assert np.array_equal(o, dec), (name, rate)
         n += 1
     assert n == 99
+
+
+def test_64_bit_block_codec_matches_golden_vectors(host, golden_64):
+    """The float64 / int64 front ends of the header the GPU lanes run (64 planes as
+    two passes over 32-bit words, 12-bit header for doubles) against the zfp 0.5.5
+    vectors for 1-D, 2-D and 3-D fields."""
+    A = [C.c_void_p, C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
+    host.host_zfp_encode_w64.argtypes = A
+    host.host_zfp_decode_w64.argtypes = A
+    n = 0
+    for name, rate, maxbits, f, stream, dec in golden_cases(golden_64):
+        is_int = int(f.dtype == np.int64)
+        shp = (1,) * (3 - f.ndim) + f.shape
+        nz, ny, nx = shp
+        blocks = int(np.prod([-(-d // 4) for d in f.shape]))
+        words = (blocks * maxbits + 63) // 64
+        s = np.zeros(words + 2, dtype=np.uint64)
+        host.host_zfp_encode_w64(f.ctypes.data, is_int, f.ndim, nx, ny, nz, maxbits, s.ctypes.data)
+        sb = s[:words].view(np.uint8)
+        k = min(sb.size, stream.size)
+        assert np.array_equal(sb[:k], stream[:k]), (name, rate)
+        assert not sb[k:].any() and not stream[k:].any()
+        g = np.zeros((words + 2) * 8, dtype=np.uint8)
+        g[:k] = stream[:k]
+        o = np.zeros_like(f)
+        host.host_zfp_decode_w64(g.ctypes.data, is_int, f.ndim, nx, ny, nz, maxbits, o.ctypes.data)
+        assert np.array_equal(o.view(np.uint64), dec.view(np.uint64)), (name, rate)
+        n += 1
+    assert n == 187
+
+
+def test_64_bit_block_codec_agrees_with_checker_on_tiny_and_huge_doubles(host):
+    """Blocks near the bottom of the double range: the scale 2^(62-emax) overflows
+    below 2^-961 (the cast saturates) and fewer than 64 planes are coded below
+    2^-1018; the reference leaves these undefined, the two implementations here
+    agree on them.  Also infinities of the scale's other end (values near 1e308)."""
+    import oracle
+
+    A = [C.c_void_p, C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
+    host.host_zfp_encode_w64.argtypes = A
+    host.host_zfp_decode_w64.argtypes = A
+    rng = np.random.default_rng(9)
+    for scale in (1e-300, 1e-306, 3e-308, 5e-320, 1e300, 1.5e308):
+        with np.errstate(over="ignore"):
+            f = np.ascontiguousarray(rng.standard_normal((4, 8, 4)) * scale)
+        if scale > 1e307:
+            f = np.clip(f, -1.7e308, 1.7e308)
+        for maxbits in (512, 1030, 4096):
+            words = 2 * maxbits // 64 + 1
+            s = np.zeros(words + 2, dtype=np.uint64)
+            host.host_zfp_encode_w64(f.ctypes.data, 0, 3, 4, 8, 4, maxbits, s.ctypes.data)
+            want = oracle.zfp_encode_64(f, maxbits)
+            assert np.array_equal(s[: want.size], want), (scale, maxbits)
+            o = np.zeros_like(f)
+            host.host_zfp_decode_w64(s.ctypes.data, 0, 3, 4, 8, 4, maxbits, o.ctypes.data)
+            d = oracle.zfp_decode_64(want, f.shape, maxbits, np.float64)
+            assert np.array_equal(o.view(np.uint64), d.view(np.uint64)), (scale, maxbits)

@@ -323,44 +323,155 @@ def test_int32_fields_vs_checker(torch_cuda, shape, maxbits):
 
 
 def test_cuda_compress_dispatches_on_the_scalar_type(torch_cuda):
-    """cuda_compress / cuda_decompress look at field->type (cuZFP.cu:388-422): float
-    and int32 are coded, the 64-bit types report failure (size 0 / stream pointer
-    not advanced), as the reference does for a type it cannot handle."""
+    """cuda_compress / cuda_decompress look at field->type (cuZFP.cu:388-423): all
+    four scalar types are coded; an unknown type reports failure (size 0 / stream
+    pointer not advanced)."""
     torch = torch_cuda
-    import oracle
-    from cswap_amd import api
-
-    rng = np.random.default_rng(3)
-    f = rng.integers(-2**20, 2**20, (8, 12, 16)).astype(np.int32)
-    t = torch.from_numpy(f).cuda()
-    s = api.cuda_compress(t, 512)
-    want = oracle.zfp_encode_i32(f, 512)
-    assert np.array_equal(s.cpu().numpy().view(np.uint64)[: want.size], want)
-    d = api.cuda_decompress(s, f.shape, 512, dtype=torch.int32)
-    torch.cuda.synchronize()
-    assert np.array_equal(d.cpu().numpy(), oracle.zfp_decode_i32(want, f.shape, 512))
-    with pytest.raises((RuntimeError, TypeError, ValueError)):
-        api.cuda_compress(t.to(torch.float64), 512)
-
-    # the reference-named entry points with zfp_field.type = zfp_type_int32 (1) and zfp_type_double (4)
     import ctypes as C
 
+    import oracle
+    from cswap_amd import api
     from cswap_amd._lib import ZfpBitstream, ZfpField, ZfpStream, lib
 
     L = lib()
-    cap = L.cswap_zfp_stream_capacity(16, 12, 8, 512)
-    sbuf = torch.zeros(cap, dtype=torch.uint8, device="cuda")
-    bs = ZfpBitstream(0, 0, sbuf.data_ptr(), sbuf.data_ptr(), sbuf.data_ptr() + cap)
-    zs = ZfpStream(1, 512, 64, -1074, C.pointer(bs), 0, 0, 0)
-    fld = ZfpField(1, 16, 12, 8, 0, 0, 0, 0, 0, t.data_ptr())
-    assert L.cuda_compress(C.byref(zs), C.byref(fld)) == cap
-    assert np.array_equal(sbuf.cpu().numpy().view(np.uint64), want)
-    back = torch.zeros_like(t)
+    rng = np.random.default_rng(3)
+    fields = {1: rng.integers(-2**20, 2**20, (8, 12, 16)).astype(np.int32),
+              2: rng.integers(-2**50, 2**50, (8, 12, 16)),
+              3: rng.standard_normal((8, 12, 16)).astype(np.float32),
+              4: rng.standard_normal((8, 12, 16)) * 1e10}
+    for ztype, f in fields.items():
+        t = torch.from_numpy(f).cuda()
+        if ztype == 1:
+            want = oracle.zfp_encode_i32(f, 512)
+            dec = oracle.zfp_decode_i32(want, f.shape, 512)
+        elif ztype == 3:
+            want = oracle.zfp_encode3(f, 512)
+            dec = oracle.zfp_decode3(want, f.shape, 512)
+        else:
+            want = oracle.zfp_encode_64(f, 512)
+            dec = oracle.zfp_decode_64(want, f.shape, 512, f.dtype)
+        # torch-facing wrapper
+        s = api.cuda_compress(t, 512)
+        assert np.array_equal(s.cpu().numpy().view(np.uint64)[: want.size], want), ztype
+        d = api.cuda_decompress(s, f.shape, 512, dtype=t.dtype)
+        torch.cuda.synchronize()
+        assert np.array_equal(d.cpu().numpy().view(np.uint8), dec.view(np.uint8)), ztype
+        # the reference-named entry points with zfp_field.type = ztype
+        cap = L.cswap_zfp_stream_capacity(16, 12, 8, 512)
+        sbuf = torch.zeros(cap, dtype=torch.uint8, device="cuda")
+        bs = ZfpBitstream(0, 0, sbuf.data_ptr(), sbuf.data_ptr(), sbuf.data_ptr() + cap)
+        zs = ZfpStream(1, 512, 64, -1074, C.pointer(bs), 0, 0, 0)
+        fld = ZfpField(ztype, 16, 12, 8, 0, 0, 0, 0, 0, t.data_ptr())
+        assert L.cuda_compress(C.byref(zs), C.byref(fld)) == cap
+        assert np.array_equal(sbuf.cpu().numpy().view(np.uint64), want), ztype
+        back = torch.zeros_like(t)
+        bs.ptr = bs.begin
+        fld_out = ZfpField(ztype, 16, 12, 8, 0, 0, 0, 0, 0, back.data_ptr())
+        L.cuda_decompress(C.byref(zs), C.byref(fld_out))
+        assert bs.ptr == bs.begin + cap
+        assert np.array_equal(back.cpu().numpy().view(np.uint8), dec.view(np.uint8)), ztype
+        # a host-resident field of the same type goes through the staged path
+        hs = np.zeros(cap // 8, dtype=np.uint64)
+        hb = ZfpBitstream(0, 0, hs.ctypes.data, hs.ctypes.data, hs.ctypes.data + cap)
+        hz = ZfpStream(1, 512, 64, -1074, C.pointer(hb), 0, 0, 0)
+        hf = ZfpField(ztype, 16, 12, 8, 0, 0, 0, 0, 0, f.ctypes.data)
+        assert L.cuda_compress(C.byref(hz), C.byref(hf)) == cap
+        assert np.array_equal(hs, want), ztype
+    with pytest.raises((RuntimeError, TypeError, ValueError)):
+        api.cuda_compress(torch.zeros(4, 4, 4, dtype=torch.float16, device="cuda"), 512)
     bs.ptr = bs.begin
-    fld_out = ZfpField(1, 16, 12, 8, 0, 0, 0, 0, 0, back.data_ptr())
-    L.cuda_decompress(C.byref(zs), C.byref(fld_out))
-    assert np.array_equal(back.cpu().numpy(), oracle.zfp_decode_i32(want, f.shape, 512))
-    dbl = torch.zeros(8, 12, 16, dtype=torch.float64, device="cuda")
-    bs.ptr = bs.begin
-    fld_d = ZfpField(4, 16, 12, 8, 0, 0, 0, 0, 0, dbl.data_ptr())
-    assert L.cuda_compress(C.byref(zs), C.byref(fld_d)) == 0
+    bad = ZfpField(0, 16, 12, 8, 0, 0, 0, 0, 0, t.data_ptr())
+    assert L.cuda_compress(C.byref(zs), C.byref(bad)) == 0
+
+
+def _gpu_w64(torch, f, maxbits, strides=None):
+    from cswap_amd._lib import check, lib
+
+    L = lib()
+    kind = "i64" if f.dtype == np.int64 else "f64"
+    shp = (1,) * (3 - f.ndim) + f.shape
+    nz, ny, nx = shp
+    t = torch.from_numpy(f).cuda()
+    cap = L.cswap_zfp_stream_capacity_nd(f.ndim, nx, ny, nz, maxbits)
+    s = torch.zeros(cap + 16, dtype=torch.uint8, device="cuda")
+    check(getattr(L, f"cswap_zfp_compress_{kind}_nd")(t.data_ptr(), f.ndim, nx, ny, nz, 0, 0, 0, maxbits,
+                                                        s.data_ptr(), None), "c")
+    o = torch.full(f.shape, -123456, dtype=t.dtype, device="cuda")
+    check(getattr(L, f"cswap_zfp_decompress_{kind}_nd")(s.data_ptr(), f.ndim, nx, ny, nz, 0, 0, 0, maxbits,
+                                                          o.data_ptr(), None), "d")
+    torch.cuda.synchronize()
+    return s[:cap].cpu().numpy(), o.cpu().numpy()
+
+
+def test_64_bit_golden_vectors(torch_cuda, golden_64):
+    """zfp_type_double and zfp_type_int64 fields of 1, 2 and 3 dimensions
+    (cuZFP.cu:401-423,479-504) against the zfp 0.5.5 vectors: stream bytes and
+    decoded values, rates 1 to 64 bits per value."""
+    n = 0
+    for name, rate, maxbits, f, stream, dec in golden_cases(golden_64):
+        s, o = _gpu_w64(torch_cuda, f, maxbits)
+        k = min(s.size, stream.size)
+        assert np.array_equal(s[:k], stream[:k]), (name, rate)
+        assert not s[k:].any() and not stream[k:].any(), (name, rate)
+        assert np.array_equal(o.view(np.uint64), dec.view(np.uint64)), (name, rate)
+        n += 1
+    assert n == 187
+
+
+@pytest.mark.parametrize("dtype", ["f64", "i64"])
+@pytest.mark.parametrize("shape,maxbits", [((40, 36, 132), 512), ((33, 7, 9), 1030), ((300, 260), 256), ((5000,), 72),
+                                           ((64, 64, 64), 2048), ((16, 64, 64), 4096)])
+def test_64_bit_fields_vs_checker(torch_cuda, dtype, shape, maxbits):
+    import oracle
+
+    rng = np.random.default_rng(sum(shape) + maxbits)
+    if dtype == "f64":
+        f = rng.standard_normal(shape) * 10.0 ** rng.integers(-30, 30, size=shape[:1] + (1,) * (len(shape) - 1))
+    else:
+        f = (rng.standard_normal(shape) * 10.0 ** rng.integers(2, 17)).astype(np.int64)
+    f = np.ascontiguousarray(f)
+    s, o = _gpu_w64(torch_cuda, f, maxbits)
+    want = oracle.zfp_encode_64(f, maxbits)
+    assert np.array_equal(s.view(np.uint64), want)
+    assert np.array_equal(o.view(np.uint64), oracle.zfp_decode_64(want, f.shape, maxbits, f.dtype).view(np.uint64))
+
+
+def test_64_bit_strided_and_edge_doubles(torch_cuda):
+    """A sub-volume of a larger double tensor through element strides (general
+    path), and blocks at the bottom of the double range where the scale overflows
+    and fewer than 64 planes are coded: same bits as the checker."""
+    torch = torch_cuda
+    import oracle
+    from cswap_amd._lib import check, lib
+
+    L = lib()
+    rng = np.random.default_rng(77)
+    big = rng.standard_normal((12, 20, 30))
+    sub = np.ascontiguousarray(big[1:9, 2:13, 3:22])          # 8 x 11 x 19, partial blocks, odd offsets
+    t = torch.from_numpy(big).cuda()
+    nz, ny, nx = sub.shape
+    cap = L.cswap_zfp_stream_capacity(nx, ny, nz, 1024)
+    s = torch.zeros(cap, dtype=torch.uint8, device="cuda")
+    base = t.data_ptr() + 8 * (1 * 600 + 2 * 30 + 3)
+    check(L.cswap_zfp_compress_f64_nd(base, 3, nx, ny, nz, 1, 30, 600, 1024, s.data_ptr(), None), "c")
+    want = oracle.zfp_encode_64(sub, 1024)
+    assert np.array_equal(s.cpu().numpy().view(np.uint64), want)
+    o = torch.zeros_like(t)
+    check(L.cswap_zfp_decompress_f64_nd(s.data_ptr(), 3, nx, ny, nz, 1, 30, 600, 1024,
+                                        o.data_ptr() + 8 * (1 * 600 + 2 * 30 + 3), None), "d")
+    torch.cuda.synchronize()
+    got = o.cpu().numpy()
+    assert np.array_equal(got[1:9, 2:13, 3:22].view(np.uint64),
+                          oracle.zfp_decode_64(want, sub.shape, 1024, np.float64).view(np.uint64))
+    mask = np.ones_like(got, dtype=bool)
+    mask[1:9, 2:13, 3:22] = False
+    assert not got[mask].any()                                # nothing outside the sub-volume was written
+
+    for scale in (1e-300, 1e-306, 3e-308, 5e-320, 1e300):
+        f = np.ascontiguousarray(rng.standard_normal((4, 8, 8)) * scale)
+        for maxbits in (512, 4096):
+            sb, ob = _gpu_w64(torch, f, maxbits)
+            w = oracle.zfp_encode_64(f, maxbits)
+            assert np.array_equal(sb.view(np.uint64), w), (scale, maxbits)
+            assert np.array_equal(ob.view(np.uint64),
+                                  oracle.zfp_decode_64(w, f.shape, maxbits, np.float64).view(np.uint64)), (scale, maxbits)

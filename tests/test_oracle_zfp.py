@@ -293,6 +293,49 @@ def test_int32_fields_match_golden_vectors(golden_i32):
     assert n == 99
 
 
+def _words(stream):
+    if stream.size % 8 == 0:
+        return stream.view(np.uint64)
+    return np.frombuffer(stream.tobytes() + bytes(8 - stream.size % 8), dtype=np.uint64)
+
+
+def test_64_bit_fields_match_golden_vectors(golden_64):
+    """zfp_type_double and zfp_type_int64 (cuZFP.cu:401-423,479-504): 64 bit planes,
+    for doubles a 12-bit header and the scale 2^(62-emax).  Streams and decoded
+    values of the zfp 0.5.5 command-line codec (-d, -t i64) for 1-D, 2-D and 3-D
+    fields: partial, all-zero, negative-zero and constant blocks, magnitudes from
+    1e-250 to 1e250 inside one field, integers up to 2^61, rates 1 to 64."""
+    import oracle
+
+    n = 0
+    for name, rate, maxbits, f, stream, dec in golden_cases(golden_64):
+        assert f.dtype == (np.int64 if name[0] == "l" else np.float64)
+        sb = oracle.zfp_encode_64(f, maxbits).view(np.uint8)
+        k = min(sb.size, stream.size)
+        assert np.array_equal(sb[:k], stream[:k]), (name, rate)
+        assert not sb[k:].any() and not stream[k:].any(), (name, rate)
+        d = oracle.zfp_decode_64(_words(stream), f.shape, maxbits, f.dtype)
+        assert np.array_equal(d.view(np.uint64), dec.view(np.uint64)), (name, rate)
+        n += 1
+    assert n == 187
+
+
+def test_64_bit_high_rate_is_nearly_lossless():
+    import oracle
+
+    rng = np.random.default_rng(6)
+    f = rng.integers(-2**58, 2**58, (8, 8, 8))
+    d = oracle.zfp_decode_64(oracle.zfp_encode_64(f, 64 * 72), f.shape, 64 * 72, np.int64)
+    assert np.abs(d - f).max() <= 32
+    x = rng.standard_normal((4, 8, 12))
+    y = oracle.zfp_decode_64(oracle.zfp_encode_64(x, 64 * 64), x.shape, 64 * 64, np.float64)
+    assert np.abs(y - x).max() < 1e-15 * 64
+    z = np.zeros((4, 4, 4))
+    assert not oracle.zfp_encode_64(z, 512).any()
+    # the reference's decoder leaves an empty block untouched; the field level pre-zeroes it
+    assert not oracle.zfp_decode_64(np.zeros(8, dtype=np.uint64), z.shape, 512, np.float64).any()
+
+
 def test_int32_high_rate_is_nearly_lossless():
     """With 32 bits per value the coder runs through every plane; what is left is
     the rounding of the lifting transform: at most a few units per component."""
