@@ -23,47 +23,62 @@ E_NOMEM = -4   # CSWAP_E_NOMEM
 
 
 class _Handle:
-    __slots__ = ("ticket", "shape", "keep")
+    __slots__ = ("ticket", "shape", "keep", "key", "refs", "out")
 
-    def __init__(self, ticket, shape, keep):
-        self.ticket, self.shape, self.keep = ticket, shape, keep
+    def __init__(self, ticket, shape, keep, key):
+        self.ticket, self.shape, self.keep, self.key = ticket, shape, keep, key
+        self.refs = 1        # how many autograd nodes saved this tensor
+        self.out = None      # the swapped-in tensor while further nodes still have to ask for it
 
 
 class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
     """Swap eligible saved activations (contiguous fp32 device tensors of at
     least ``min_bytes``) through ``engine``; everything else is saved as usual.
 
-    The outbound copy of tensor i overlaps with whatever the compute stream does
-    until tensor i+1 is packed, at which point its completion is awaited and the
-    device copy is let go (the reference does the same one layer later,
-    CSWAP+/vgg16-cifar10.cpp:221-228).
+    The outbound copy of a tensor overlaps with whatever the compute stream does
+    next.  Up to ``depth`` copies are left in flight: packing one more first waits
+    for the oldest and lets its device copy go (the reference waits one layer
+    later, CSWAP+/vgg16-cifar10.cpp:221-228, i.e. depth 1).  With depth 2 the
+    probe and the compression of tensor i run while tensor i-1 is still on the
+    link, so the link does not idle between tensors.
+
+    A tensor that several nodes save (the output of a ReLU is saved by the ReLU
+    and by the convolution or pooling that consumes it) is swapped once: while its
+    device copy is still held, packing the same storage, shape and version again
+    returns the same handle, and backward hands the one swapped-in tensor to
+    every node that asks for it.
 
     Backward asks for the tensors in roughly the reverse of the order they were
     packed in, so each unpack also starts the inbound copy of the ``prefetch``
     tensors packed just before the one it returns: their transfer then runs on
-    the copy stream under the backward kernels of the current layer."""
+    the copy stream under the backward kernels of the current layer.  (VGG-16 at
+    batch 128 on one MI355X: looking two tensors ahead keeps the link busy through
+    layers whose backward is short; deeper look-ahead gains nothing more.)"""
 
     def __init__(self, engine: "swap.SwapEngine", policy: int = swap.AUTO, min_bytes: int = 1 << 20,
-                 prefetch: int = 1):
+                 prefetch: int = 2, depth: int = 2):
         self.engine = engine
         self.policy = policy
         self.min_bytes = min_bytes
         self.prefetch = prefetch
+        self.depth = max(1, depth)
         self._order = []           # handles in pack order
         self._fetched = set()      # tickets already swapped in or being prefetched
         self._released = set()
-        self._pending = None       # handle whose outbound copy may still be in flight
-        self._to_release = []      # tickets whose swap-in has been launched
-        self.stats = {"swapped": 0, "bytes_in": 0, "bytes_out": 0, "kept": 0}
+        self._pending = []         # handles whose outbound copy may still be in flight, oldest first
+        self._live = {}            # key -> handle, only while the handle holds its device tensor
+        self._to_release = []      # handles whose swap-in has been launched
+        self.stats = {"swapped": 0, "bytes_in": 0, "bytes_out": 0, "kept": 0, "shared": 0}
         super().__init__(self._pack, self._unpack)
 
     # -- forward side
-    def _settle(self):
-        h = self._pending
-        if h is not None:
+    def _settle(self, keep_in_flight: int = 0):
+        """Wait for the oldest outbound copies until at most ``keep_in_flight`` are left."""
+        while len(self._pending) > keep_in_flight:
+            h = self._pending.pop(0)
             self.engine.post(h.ticket)   # Execution::post: copy done, device memory may go
             h.keep = None
-            self._pending = None
+            self._live.pop(h.key, None)
 
     def _pack(self, t: torch.Tensor):
         eligible = (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.dim() >= 1
@@ -72,35 +87,50 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         if not eligible:
             self.stats["kept"] += 1
             return t
-        self._settle()
+        key = (t.data_ptr(), tuple(t.shape), t._version)
+        h = self._live.get(key)
+        if h is not None:                # same tensor saved by another node: one swap serves both
+            h.refs += 1
+            self.stats["shared"] += 1
+            return h
+        self._settle(self.depth - 1)
         self._drain()
         ticket = self.engine.pre(t.detach(), self.policy)
         info = self.engine.info(ticket)
         self.stats["swapped"] += 1
         self.stats["bytes_in"] += info.bytes_in
         self.stats["bytes_out"] += info.bytes_out
-        h = _Handle(ticket, tuple(t.shape), t)   # keep the device copy alive until the copy finished
-        self._pending = h
+        h = _Handle(ticket, tuple(t.shape), t, key)   # keeps the device copy alive until the copy finished
+        self._pending.append(h)
+        self._live[key] = h
         self._order.append(h)
         return h
 
     # -- backward side
     def _drain(self):
-        for tk in self._to_release:
-            self.engine.release(tk)
-            self._released.add(tk)
+        for h in self._to_release:
+            self.engine.release(h.ticket)
+            self._released.add(h.ticket)
         self._to_release.clear()
 
     def _unpack(self, h):
         if not isinstance(h, _Handle):
             return h
-        if self._pending is h:
-            self._settle()
+        if h.out is not None:            # another node already had it swapped in
+            out = h.out
+            h.refs -= 1
+            if h.refs <= 0:
+                h.out = None
+            return out
+        self._settle()
         self._drain()
         out = torch.empty(h.shape, dtype=torch.float32, device="cuda")
         self.engine.swap_in(h.ticket, out)
         self._fetched.add(h.ticket)
-        self._to_release.append(h.ticket)   # released once the next swap-in is issued (or at close)
+        self._to_release.append(h)       # released once the next swap-in is issued (or at close)
+        h.refs -= 1
+        if h.refs > 0:
+            h.out = out
         self._prefetch_before(h)
         return out
 
@@ -115,8 +145,6 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
                 break
             if g.ticket in self._fetched:
                 continue
-            if self._pending is g:
-                self._settle()
             try:
                 self.engine.prefetch(g.ticket)
             except CswapError as err:
@@ -133,6 +161,7 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         torch.cuda.synchronize()
         self._drain()
         for h in self._order:              # saved but never asked for by backward
+            h.out = None
             if h.ticket not in self._released:
                 self.engine.release(h.ticket)
                 self._released.add(h.ticket)
@@ -192,9 +221,10 @@ def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int =
     eng.calibrate()
     res["staging_pool_MB"] = round(staging / 1e6, 1)    # device memory the engine holds besides torch's allocator
     for label, pol in (("raw_swap", swap.NONE), ("selector", swap.AUTO)):
-        ms, mb, st = measure(lambda: swap_saved_tensors(eng, policy=pol, min_bytes=min_bytes, prefetch=1))
+        ms, mb, st = measure(lambda: swap_saved_tensors(eng, policy=pol, min_bytes=min_bytes, prefetch=2, depth=2))
         res[label] = {"step_ms": round(ms, 2), "peak_MB": round(mb, 1),
                       "swapped_tensors": st["swapped"], "swapped_MB": round(st["bytes_in"] / 1e6, 1),
-                      "link_MB": round(st["bytes_out"] / 1e6, 1), "prefetched": st.get("prefetched", 0)}
+                      "link_MB": round(st["bytes_out"] / 1e6, 1), "shared": st["shared"],
+                      "prefetched": st.get("prefetched", 0)}
     eng.close()
     return res

@@ -77,6 +77,32 @@ def test_lossless_policies_keep_gradients_bit_identical(torch_cuda, policy_name)
     eng.close()
 
 
+def test_tensor_saved_by_two_nodes_is_swapped_once(torch_cuda):
+    """The output of a ReLU is saved by the ReLU and by the layer that consumes
+    it: one swap serves both (the reference swaps by tensor id, once).  Gradients
+    stay bit-identical for every depth of the outbound pipeline."""
+    torch = torch_cuda
+    from cswap_amd import swap
+    from cswap_amd.hooks import swap_saved_tensors
+
+    net = make_mlp(torch)
+    x = torch.randn(2048, 512, device="cuda")
+    loss0, g0 = grads(torch, net, x)
+    eng = swap.SwapEngine(pinned_bytes=256 << 20, device_bytes=256 << 20)
+    seen = {}
+    for depth in (1, 2, 4):
+        ctx = swap_saved_tensors(eng, policy=swap.SPARSE, min_bytes=1 << 16, depth=depth)
+        loss1, g1 = grads(torch, net, x, ctx)
+        assert loss1 == loss0 and all(torch.equal(a, b) for a, b in zip(g0, g1)), depth
+        assert ctx.stats["shared"] >= 2, ctx.stats        # both ReLU outputs were packed twice
+        seen[depth] = (ctx.stats["swapped"], ctx.stats["shared"], ctx.stats["bytes_in"])
+    assert seen[1] == seen[2] == seen[4]
+    # every ticket went back to the engine
+    from cswap_amd._lib import lib
+    assert all(lib().cswap_swap_release(eng._h, i) == -5 for i in range(8))
+    eng.close()
+
+
 def test_conv_net_round_trip_close(torch_cuda):
     """Convolution backward is not bit-reproducible run to run, so compare with a
     tolerance; the swapped activations themselves are restored exactly."""
