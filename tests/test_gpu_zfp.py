@@ -475,3 +475,72 @@ def test_64_bit_strided_and_edge_doubles(torch_cuda):
             assert np.array_equal(sb.view(np.uint64), w), (scale, maxbits)
             assert np.array_equal(ob.view(np.uint64),
                                   oracle.zfp_decode_64(w, f.shape, maxbits, np.float64).view(np.uint64)), (scale, maxbits)
+
+
+def test_random_shapes_rates_types_and_strides_vs_checker(torch_cuda):
+    """240 seeded cases: dimensionality 1-3, extents 1-37 (partial blocks on any
+    axis), block budgets from 16 to 4096 bits that are and are not whole words, all
+    four scalar types, and the field embedded with element strides in a larger
+    array.  Stream words and decoded values equal the checker's; nothing outside
+    the field is written."""
+    torch = torch_cuda
+    import oracle
+    from cswap_amd._lib import check, lib
+
+    L = lib()
+    rng = np.random.default_rng(20240)
+    kinds = {"f32": (np.float32, torch.float32), "i32": (np.int32, torch.int32),
+             "f64": (np.float64, torch.float64), "i64": (np.int64, torch.int64)}
+    for case in range(240):
+        kind = ("f32", "i32", "f64", "i64")[case % 4]
+        npdt, tdt = kinds[kind]
+        dims = int(rng.integers(1, 4))
+        shape = tuple(int(v) for v in rng.integers(1, 38, size=dims))            # (nz, ny, nx)[-dims:]
+        pad = tuple(int(v) for v in rng.integers(0, 4, size=dims))               # extra elements per axis
+        off = tuple(int(rng.integers(0, p + 1)) for p in pad)
+        big_shape = tuple(s + p for s, p in zip(shape, pad))
+        if kind[0] == "f":
+            big = rng.standard_normal(big_shape) * 10.0 ** int(rng.integers(-6, 7))
+            if rng.random() < 0.3:
+                big[rng.random(big_shape) < 0.5] = 0.0
+        else:
+            big = rng.integers(-2 ** int(rng.integers(4, 30 if kind == "i32" else 61)),
+                               2 ** int(rng.integers(4, 30 if kind == "i32" else 61)) + 1, size=big_shape)
+        big = np.ascontiguousarray(big.astype(npdt))
+        sl = tuple(slice(o, o + s) for o, s in zip(off, shape))
+        sub = np.ascontiguousarray(big[sl])
+        maxbits = int(rng.choice([16, 40, 64, 100, 128, 200, 256, 500, 512, 1000, 1024, 2048, 4000, 4096]))
+        if kind == "f64":
+            maxbits = max(maxbits, 24)                                               # room for the 12-bit header
+        st = [int(v) for v in np.array(big.strides) // big.itemsize]              # element strides, slowest first
+        nzyx = (1,) * (3 - dims) + shape
+        sz, sy, sx = ([0] * (3 - dims) + st)
+        nz, ny, nx = nzyx
+        t = torch.from_numpy(big).cuda()
+        base = t.data_ptr() + big.itemsize * sum(o * s for o, s in zip(off, st))
+        cap = L.cswap_zfp_stream_capacity_nd(dims, nx, ny, nz, maxbits)
+        s = torch.zeros(cap, dtype=torch.uint8, device="cuda")
+        tag = (case, kind, shape, pad, off, maxbits)
+        check(getattr(L, f"cswap_zfp_compress_{kind}_nd")(base, dims, nx, ny, nz, sx, sy, sz, maxbits,
+                                                            s.data_ptr(), None), "compress")
+        if kind == "f32":
+            want = oracle.zfp_encode_nd(sub, maxbits)
+            dec = oracle.zfp_decode_nd(want, sub.shape, maxbits)
+        elif kind == "i32":
+            want = oracle.zfp_encode_i32(sub, maxbits)
+            dec = oracle.zfp_decode_i32(want, sub.shape, maxbits)
+        else:
+            want = oracle.zfp_encode_64(sub, maxbits)
+            dec = oracle.zfp_decode_64(want, sub.shape, maxbits, npdt)
+        got = s.cpu().numpy().view(np.uint64)
+        assert np.array_equal(got, want[: got.size]), tag
+        o = torch.zeros(big_shape, dtype=tdt, device="cuda")
+        obase = o.data_ptr() + big.itemsize * sum(oo * ss for oo, ss in zip(off, st))
+        check(getattr(L, f"cswap_zfp_decompress_{kind}_nd")(s.data_ptr(), dims, nx, ny, nz, sx, sy, sz, maxbits,
+                                                              obase, None), "decompress")
+        torch.cuda.synchronize()
+        back = o.cpu().numpy()
+        assert np.array_equal(back[sl].view(np.uint8), dec.view(np.uint8)), tag
+        outside = np.ones(big_shape, dtype=bool)
+        outside[sl] = False
+        assert not back[outside].any(), tag

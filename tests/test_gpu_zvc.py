@@ -204,3 +204,40 @@ def test_full_size_round_trip(torch_cuda):
     m = mask.cpu().numpy().view(np.uint8)
     assert int(np.unpackbits(m).sum()) == k
     assert torch.equal(values[:k], t[t != 0])
+
+
+def test_random_sizes_chunk_counts_and_sparsities(torch_cuda):
+    """120 seeded cases: n from 1 to 400 000, chunk counts from 1 to 65 536 (more
+    chunks than elements included), zero fractions from 0 to 1 with special values
+    mixed in, plain and single-pass compaction, and a destination that is not
+    16-byte aligned (the one-element-per-lane expansion)."""
+    torch = torch_cuda
+    from cswap_amd import api
+
+    rng = np.random.default_rng(99)
+    specials = np.array([-0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3.4e38], dtype=np.float32)
+    for case in range(120):
+        n = int(rng.choice([rng.integers(1, 100), rng.integers(100, 5000), rng.integers(5000, 400_000)]))
+        process = int(rng.choice([1, 3, 7, 64, 1000, 1024, 4096, 16384, 65536]))
+        zeros = float(rng.choice([0.0, 0.05, 0.5, 0.9, 0.999, 1.0]))
+        x = rng.standard_normal(n).astype(np.float32)
+        x[rng.random(n) < zeros] = 0.0
+        k = rng.integers(0, 8)
+        if k and n > 8:
+            x[rng.integers(0, n, size=k)] = rng.choice(specials, size=k)
+        fused = bool(case % 2)
+        tag = (case, n, process, zeros, fused)
+        print(tag, flush=True)
+        got = run_gpu(torch, x, process, fused=fused)
+        check_against_oracle(x, got, process)
+        # unaligned destination
+        t = torch.from_numpy(x).cuda()
+        values, mask, begin, nnz = api.zvc_compress(t, process)
+        buf = torch.full((n + 8,), -1.0, device="cuda")
+        shift = 1 + case % 3
+        api.GPUdecompression(values, buf[shift:shift + n], mask, begin, process)
+        torch.cuda.synchronize()
+        b = buf.cpu().numpy()
+        want = np.where(x != 0, x, np.float32(0))
+        assert np.array_equal(b[shift:shift + n].view(np.uint32), want.view(np.uint32)), tag
+        assert (b[:shift] == -1).all() and (b[shift + n:] == -1).all(), tag
