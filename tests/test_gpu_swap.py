@@ -451,3 +451,88 @@ def test_reference_harness_binary_runs_against_this_library(torch_cuda):
     assert 0 <= cnt <= n
     loss = float(re.search(r"Final accuray loss is -> ([0-9.eE+-]+)", out.stdout).group(1))
     assert loss < 0.05
+
+
+def test_random_ticket_traffic_with_small_pools(torch_cuda):
+    """600 random engine operations (swap-out under every policy, wait, prefetch,
+    swap-in, release, in any legal order) on pools small enough to fill up and
+    fragment: a refused request (no memory) leaves the engine usable, every tensor
+    that comes back is bit-identical to what its policy promises, and in the end
+    both pools are whole again."""
+    torch = torch_cuda
+    from cswap_amd import api, swap
+    from cswap_amd._lib import CswapError
+
+    eng = swap.SwapEngine(pinned_bytes=6 << 20, device_bytes=3 << 20, max_tickets=24)
+    rng = np.random.default_rng(4711)
+    shapes = [(64, 64, 16), (32, 32, 64), (8, 8, 2048), (4, 4, 1000), (128, 64, 32), (2, 2, 4096), (64, 64, 128)]
+    pool = []
+    for i, shp in enumerate(shapes):
+        x = relu_tensor(torch, shp, [0.3, 0.6, 0.9][i % 3], 100 + i)
+        if i % 2:
+            x = x + 0.25 * torch.randn_like(x) * (x != 0)
+        s = api.cuda_compress(x, 512)
+        zfp = api.cuda_decompress(s, x.shape, 512)
+        pool.append((x, zfp))
+    torch.cuda.synchronize()
+    live = {}          # ticket -> (tensor index, state)
+    refused = done = 0
+    for step in range(600):
+        op = rng.choice(["out", "out", "wait", "prefetch", "in", "release"])
+        if op == "out" or not live:
+            i = int(rng.integers(len(pool)))
+            pol = int(rng.choice([swap.NONE, swap.SPARSE, swap.ZFP, swap.AUTO]))
+            try:
+                tk = eng.pre(pool[i][0], pol)
+            except CswapError as err:
+                assert err.code == -4, (step, err)
+                refused += 1
+                if live:                                   # make room: retire the oldest ticket
+                    old = next(iter(live))
+                    eng.release(old)
+                    del live[old]
+                continue
+            assert tk not in live
+            live[tk] = i
+            continue
+        tk = int(rng.choice(list(live)))
+        i = live[tk]
+        if op == "wait":
+            st = eng.info(tk).state
+            if st in (1, 2):
+                eng.post(tk)
+        elif op == "prefetch":
+            if eng.info(tk).state in (1, 2, 4):
+                try:
+                    eng.prefetch(tk)
+                except CswapError as err:
+                    assert err.code == -4, (step, err)
+                    refused += 1
+        elif op == "in":
+            if eng.info(tk).state in (1, 2, 4):
+                out = torch.full_like(pool[i][0], -7.0)
+                try:
+                    eng.swap_in(tk, out)
+                except CswapError as err:
+                    assert err.code == -4, (step, err)
+                    refused += 1
+                    continue
+                torch.cuda.synchronize()
+                pol = eng.info(tk).policy
+                want = pool[i][1] if pol == swap.ZFP else pool[i][0]
+                assert torch.equal(out.view(torch.int32), want.view(torch.int32)), (step, tk, i, pol)
+                eng.release(tk)
+                del live[tk]
+                done += 1
+        else:
+            eng.release(tk)
+            del live[tk]
+    for tk in list(live):
+        eng.release(tk)
+    assert done > 50 and refused > 0, (done, refused)
+    # both pools are whole again: one allocation of (almost) the full size fits
+    big = torch.zeros(64, 64, (6 << 20) // 4 // 4096 - 1, device="cuda")       # 6 MiB less 16 KiB
+    tk = eng.pre(big, swap.NONE)
+    eng.post(tk)
+    eng.release(tk)
+    eng.close()
