@@ -642,31 +642,40 @@ struct BlockDecoder {
   // mirror of BlockEncoder::plane (decode.cuh:141-173).  Written without early
   // exits: a block that is out of budget reads zero verbatim bits and never
   // enters the step loop, and when every coefficient is already significant the
-  // plane is one 64-bit read.
+  // plane is one 64-bit read.  Every group test is read from a window that is
+  // already in registers: the first one sits right behind the verbatim bits, the
+  // one after a run right behind the run's terminating one-bit, so the step loop
+  // turns once per positive test and not at all for a plane that adds nothing.
   CSWAP_HD uint64_t plane()
   {
     unsigned left = sub_sat(limit, pos);
     unsigned m = n < left ? n : left;
-    uint64_t x = window(pos) & low_mask(m);
+    uint64_t w = window(pos);
+    uint64_t x = w & low_mask(m);
     pos += m;
-    while (n < SIZE && pos < limit) {
-      uint64_t w = window(pos);
+    bool go = n < SIZE && pos < limit;            // a group test follows (then m = n < 64)
+    bool test = go && ((w >> (m & 63)) & 1);
+    pos += go ? 1u : 0u;
+    while (test) {                                // positive group test: a run of zeros, then a one
+      w = window(pos);
       settle(w);
-      pos++;
-      if (!(w & 1)) break;  // negative group test: plane done
-      w >>= 1;              // 63 valid bits
       unsigned maxrun = SIZE - 1 - n;
       if (!FENCED) {
         unsigned avail = limit - pos;
         maxrun = maxrun < avail ? maxrun : avail;
       }
       unsigned t = (unsigned)ctz64(w);
-      bool found = t < maxrun;  // t zeros then a one; else ran into position 63 or the budget
+      bool found = t < maxrun;  // t zeros then a one; else ran into the last position or the budget
       unsigned r = found ? t : maxrun;
       pos += r + (found ? 1u : 0u);  // FENCED and out of budget: "finds" the fence, pos = limit + 1
       n += r;
       x |= (uint64_t)1 << n;
       n++;
+      // not found: n == SIZE or the budget is spent, either way the plane is over;
+      // found: t <= 62, so the next group test (bit t + 1) is still inside this window
+      go = found && n < SIZE && pos < limit;
+      test = go && ((w >> ((t + 1) & 63)) & 1);
+      pos += go ? 1u : 0u;
     }
     return x;
   }

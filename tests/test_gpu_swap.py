@@ -336,8 +336,8 @@ def test_reference_named_entry_points(torch_cuda):
     t2.zero_()
     L.cuda_decompress(C.byref(zs3), C.byref(fld4))
     assert np.array_equal(t2.cpu().numpy().view(np.uint32), oracle.zfp_decode_nd(want2, f2.shape, 128).view(np.uint32))
-    # unsupported: double fields -> failure value 0
-    fld3 = ZfpField(4, 16, 8, 12, 0, 0, 0, 0, 0, t.data_ptr())
+    # a type value outside zfp_type -> failure value 0, nothing launched
+    fld3 = ZfpField(7, 16, 8, 12, 0, 0, 0, 0, 0, t.data_ptr())
     assert L.cuda_compress(C.byref(zs), C.byref(fld3)) == 0
 
     # compress / decompress / setRatio on a flat activation (viewed as 32x32 rows)
