@@ -368,6 +368,15 @@ CSWAP_HD void settle(uint64_t& v)
 #endif
 }
 
+CSWAP_HD void settle32(uint32_t& v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" : "+v"(v));
+#else
+  (void)v;
+#endif
+}
+
 CSWAP_HD uint32_t funnel_shr(uint32_t hi, uint32_t lo, unsigned s)  // ({hi,lo} >> (s & 31)) low word
 {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -451,6 +460,15 @@ CSWAP_HD void encode_planes32(uint32_t (&lo)[32], uint32_t (&hi)[32], Enc& enc, 
 {
   tr_stage<16, 0, 32>(lo);
   tr_stage<16, 0, 32>(hi);
+  // The low 16 rows are only used if the low planes get coded.  Left alone, the
+  // compiler postpones computing them until then and keeps all 64 inputs of this
+  // stage in registers through the coding of the top planes; pinning the 32
+  // results here lets the inputs go (32 registers less, one more wavefront per SIMD).
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    settle32(lo[r]);
+    settle32(hi[r]);
+  }
   tr_half<16, kNotOut>(lo);
   tr_half<16, kNotOut>(hi);
 #pragma unroll
