@@ -377,6 +377,23 @@ CSWAP_HD void settle32(uint32_t& v)
 #endif
 }
 
+// Makes the compiler finish computing rows R0 .. R0+15 at this point of the
+// instruction stream.  Left alone it postpones whichever half of a butterfly
+// stage's results is needed later and keeps the stage's inputs in registers
+// until then, next to the results already made.
+template <int R0>
+CSWAP_HD void settle16(uint32_t (&a)[32])
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" : "+v"(a[R0 + 0]), "+v"(a[R0 + 1]), "+v"(a[R0 + 2]), "+v"(a[R0 + 3]), "+v"(a[R0 + 4]),
+                    "+v"(a[R0 + 5]), "+v"(a[R0 + 6]), "+v"(a[R0 + 7]), "+v"(a[R0 + 8]), "+v"(a[R0 + 9]),
+                    "+v"(a[R0 + 10]), "+v"(a[R0 + 11]), "+v"(a[R0 + 12]), "+v"(a[R0 + 13]), "+v"(a[R0 + 14]),
+                    "+v"(a[R0 + 15]));
+#else
+  (void)a;
+#endif
+}
+
 CSWAP_HD uint32_t funnel_shr(uint32_t hi, uint32_t lo, unsigned s)  // ({hi,lo} >> (s & 31)) low word
 {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -464,13 +481,22 @@ CSWAP_HD void encode_planes32(uint32_t (&lo)[32], uint32_t (&hi)[32], Enc& enc, 
   // compiler postpones computing them until then and keeps all 64 inputs of this
   // stage in registers through the coding of the top planes; pinning the 32
   // results here lets the inputs go (32 registers less, one more wavefront per SIMD).
-#pragma unroll
-  for (int r = 0; r < 16; r++) {
-    settle32(lo[r]);
-    settle32(hi[r]);
-  }
-  tr_half<16, kNotOut>(lo);
-  tr_half<16, kNotOut>(hi);
+  settle16<0>(lo);
+  settle16<0>(hi);
+  tr_stage<8, 16, 32>(lo);
+  tr_stage<8, 16, 32>(hi);
+  settle16<16>(lo);
+  settle16<16>(hi);
+  tr_stage<4, 16, 32>(lo);
+  tr_stage<4, 16, 32>(hi);
+  settle16<16>(lo);
+  settle16<16>(hi);
+  tr_stage<2, 16, 32>(lo);
+  tr_stage<2, 16, 32>(hi);
+  settle16<16>(lo);
+  settle16<16>(hi);
+  tr_stage<1, 16, 32, kNotOut>(lo);
+  tr_stage<1, 16, 32, kNotOut>(hi);
 #pragma unroll
   for (int k = 31; k >= 16; k--) enc.plane(((uint64_t)hi[k] << 32) | lo[k]);
   if (CSWAP_ANY(enc.active())) {

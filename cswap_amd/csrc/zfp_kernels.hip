@@ -237,7 +237,7 @@ __device__ __forceinline__ void load_region(uint32_t* lds, unsigned lane, uint32
 // region_dwords(maxbits) dwords.
 // INT: the field holds int32 values (moved as 32-bit patterns through the same loads and stores)
 template <bool WHOLE, bool INT = false>
-__global__ __launch_bounds__(64) void zfp_encode3_f32_kernel(const float* __restrict__ in, Field3 fd,
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void zfp_encode3_f32_kernel(const float* __restrict__ in, Field3 fd,
                                                              unsigned maxbits,
                                                              uint64_t* __restrict__ stream)
 {
