@@ -100,6 +100,9 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         self.stats["swapped"] += 1
         self.stats["bytes_in"] += info.bytes_in
         self.stats["bytes_out"] += info.bytes_out
+        by = self.stats.setdefault("by_policy", {})
+        name = {swap.NONE: "raw", swap.SPARSE: "zvc", swap.ZFP: "zfp"}.get(info.policy, str(info.policy))
+        by[name] = by.get(name, 0) + 1
         h = _Handle(ticket, tuple(t.shape), t, key)   # keeps the device copy alive until the copy finished
         self._pending.append(h)
         self._live[key] = h
@@ -225,6 +228,7 @@ def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int =
         res[label] = {"step_ms": round(ms, 2), "peak_MB": round(mb, 1),
                       "swapped_tensors": st["swapped"], "swapped_MB": round(st["bytes_in"] / 1e6, 1),
                       "link_MB": round(st["bytes_out"] / 1e6, 1), "shared": st["shared"],
+                      "by_policy": dict(st.get("by_policy", {})),
                       "prefetched": st.get("prefetched", 0)}
     eng.close()
     return res
