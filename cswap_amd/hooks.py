@@ -50,7 +50,9 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
 
     Backward asks for the tensors in roughly the reverse of the order they were
     packed in, so each unpack also starts the inbound copy of the ``prefetch``
-    tensors packed just before the one it returns: their transfer then runs on
+    tensors packed just before the one it returns (one context serves one forward
+    and one backward pass: a swapped tensor is handed back once per node that saved
+    it and its host copy is released right after): their transfer then runs on
     the copy stream under the backward kernels of the current layer.  (VGG-16 at
     batch 128 on one MI355X: looking two tensors ahead keeps the link busy through
     layers whose backward is short; deeper look-ahead gains nothing more.)"""
