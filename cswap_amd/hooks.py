@@ -176,7 +176,8 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
 def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int = 8 << 20) -> dict:
     """Forward + backward of a VGG-16 (conv/BN/ReLU x13, 5 pools, linear head) on
     random data with and without activation swapping through the saved-tensor
-    hooks: step time and peak device memory.  Stock autograd, nothing patched."""
+    hooks: step time and peak device memory of the step (torch's allocator, above
+    what is allocated before the step).  Stock autograd, nothing patched."""
     import time
 
     from .planner import _vgg_modules
@@ -203,7 +204,10 @@ def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int =
     def measure(make_ctx, reps=5):
         for _ in range(2):
             step(make_ctx())
+        for p in params:
+            p.grad = None
         torch.cuda.synchronize()
+        base = torch.cuda.memory_allocated()     # weights, input and whatever else the process holds
         torch.cuda.reset_peak_memory_stats()
         best = None
         stats = None
@@ -216,18 +220,18 @@ def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int =
             dt = time.perf_counter() - t0
             best = dt if best is None else min(best, dt)
             stats = ctx.stats if ctx is not None else None
-        return best * 1e3, torch.cuda.max_memory_allocated() / 1e6, stats
+        return best * 1e3, (torch.cuda.max_memory_allocated() - base) / 1e6, stats
 
     res = {"model": f"VGG-16 BN, batch {batch}, 3x{image}x{image}", "min_bytes": min_bytes}
     base_ms, base_mb, _ = measure(lambda: None)
-    res["no_swap"] = {"step_ms": round(base_ms, 2), "peak_MB": round(base_mb, 1)}
+    res["no_swap"] = {"step_ms": round(base_ms, 2), "step_peak_MB": round(base_mb, 1)}
     staging = 512 << 20
     eng = swap.SwapEngine(pinned_bytes=4 << 30, device_bytes=staging)
     eng.calibrate()
     res["staging_pool_MB"] = round(staging / 1e6, 1)    # device memory the engine holds besides torch's allocator
     for label, pol in (("raw_swap", swap.NONE), ("selector", swap.AUTO)):
         ms, mb, st = measure(lambda: swap_saved_tensors(eng, policy=pol, min_bytes=min_bytes, prefetch=2, depth=2))
-        res[label] = {"step_ms": round(ms, 2), "peak_MB": round(mb, 1),
+        res[label] = {"step_ms": round(ms, 2), "step_peak_MB": round(mb, 1),
                       "swapped_tensors": st["swapped"], "swapped_MB": round(st["bytes_in"] / 1e6, 1),
                       "link_MB": round(st["bytes_out"] / 1e6, 1), "shared": st["shared"],
                       "by_policy": dict(st.get("by_policy", {})),
