@@ -97,6 +97,8 @@ struct Ticket {
   size_t host_off = 0, host_bytes = 0;
   size_t dev_off = 0, dev_bytes = 0;
   bool dev_held = false;
+  size_t probe_off = 0, probe_bytes = 0;  // the probe's chunk counts (ZVC offsets), kept until the payload has them
+  bool probe_held = false;
   hipEvent_t ev_ready = nullptr;  // compute stream: compressed data / destination ready
   hipEvent_t ev_copy = nullptr;   // copy stream: transfer finished
   hipEvent_t ev_done = nullptr;   // compute stream: decompression finished
@@ -222,13 +224,17 @@ static void drop_device(cswap_engine* e, Ticket& t)
     e->dpool.free(t.dev_off, t.dev_bytes);
     t.dev_held = false;
   }
+  if (t.probe_held) {
+    e->dpool.free(t.probe_off, t.probe_bytes);
+    t.probe_held = false;
+  }
 }
 
 // Error path of swap_out: kernels already queued on the compute stream may
 // still write the staging block, so it is given back only once they are done.
 static void abandon_device(cswap_engine* e, Ticket& t, hipStream_t compute)
 {
-  if (t.dev_held) (void)hipStreamSynchronize(compute);
+  if (t.dev_held || t.probe_held) (void)hipStreamSynchronize(compute);
   drop_device(e, t);
 }
 
@@ -254,6 +260,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   const int requested = policy;
   t.policy = policy; t.n = n; t.nnz = 0; t.nx = nx; t.ny = ny; t.nz = nz;
   t.dev_held = false;
+  t.probe_held = false;
   t.process = zvc_ok ? process_for(e, n) : 0;
   cswap_costs costs = e->costs;  // the selector prices the ZVC header with this tensor's chunk count
   if (t.process) costs.process = t.process;
@@ -272,16 +279,15 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     }
   }
   if (want_probe) {
-    // Worst-case ZVC staging; the chunk counts go straight into its header so
-    // that a later compaction needs no second counting pass.
-    const size_t hdr = zvc_header_bytes((int)n, t.process);
-    const size_t worst = hdr + 4 * n;
+    // The probe needs room for the chunk counts only; the payload is allocated
+    // once nnz is known, at its exact size.
+    const size_t cnt_bytes = 4 * (size_t)t.process;
     size_t off;
-    if (e->dpool.alloc(worst, &off)) {
-      t.dev_off = off; t.dev_bytes = worst; t.dev_held = true;
-      int* d_begin = (int*)(e->d_base + off);
-      if ((rc = cswap_zvc_count(d_in, (int)n, t.process, d_begin, compute))) { abandon_device(e, t, compute); return rc; }
-      if ((rc = cswap_zvc_scan(d_begin, cswap_zvc_active_chunks((int)n, t.process), e->d_nnz, compute))) {
+    if (e->dpool.alloc(cnt_bytes, &off)) {
+      t.probe_off = off; t.probe_bytes = cnt_bytes; t.probe_held = true;
+      int* d_counts = (int*)(e->d_base + off);
+      if ((rc = cswap_zvc_count(d_in, (int)n, t.process, d_counts, compute))) { abandon_device(e, t, compute); return rc; }
+      if ((rc = cswap_zvc_scan(d_counts, cswap_zvc_active_chunks((int)n, t.process), e->d_nnz, compute))) {
         abandon_device(e, t, compute); return rc;
       }
       hipError_t err = hipMemcpyAsync(e->h_nnz, e->d_nnz, sizeof(int), hipMemcpyDeviceToHost, compute);
@@ -301,32 +307,31 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   if (policy == CSWAP_POLICY_AUTO) {
     cswap_choice ch;
     cswap_costs c = costs;
-    if (!t.dev_held) c.sparse_max_ratio = 0.0;  // not probed: ZVC is not an option
+    if (!t.probe_held) c.sparse_max_ratio = 0.0;  // not probed: ZVC is not an option
     if ((rc = cswap_select_field(nx, ny, nz, t.nnz, e->maxbits, &c, &ch))) { drop_device(e, t); return rc; }
     t.policy = ch.policy;
   }
 
-  // ---- compress on the compute stream
+  // ---- compress on the compute stream into a staging block of the exact size
   const void* src = nullptr;
-  if (t.policy == CSWAP_POLICY_ZFP) {
+  if (t.policy == CSWAP_POLICY_SPARSE) {
+    t.bytes_out = zvc_header_bytes((int)n, t.process) + 4 * t.nnz;
+  } else if (t.policy == CSWAP_POLICY_ZFP) {
     t.bytes_out = cswap_zfp_stream_capacity(nx, ny, nz, e->maxbits);
-    if (t.dev_held) {  // the probe's staging block: keep its head if the stream fits
-      if (t.dev_bytes >= t.bytes_out) {
-        e->dpool.shrink(t.dev_off, t.dev_bytes, t.bytes_out);
-        t.dev_bytes = t.bytes_out;
-      } else {
-        drop_device(e, t);
-      }
+    if (t.probe_held) {  // the counts are of no further use (their kernels finished before the host read nnz)
+      e->dpool.free(t.probe_off, t.probe_bytes);
+      t.probe_held = false;
     }
-    if (!t.dev_held) {
-      size_t off;
-      if (e->dpool.alloc(t.bytes_out, &off)) {
-        t.dev_off = off; t.dev_bytes = t.bytes_out; t.dev_held = true;
-      } else if (requested == CSWAP_POLICY_AUTO) {
-        t.policy = CSWAP_POLICY_NONE;  // no staging room: the selector's choice degrades to the raw swap
-      } else {
-        return CSWAP_E_NOMEM;
-      }
+  }
+  if (t.policy == CSWAP_POLICY_SPARSE || t.policy == CSWAP_POLICY_ZFP) {
+    size_t off;
+    if (e->dpool.alloc(t.bytes_out, &off)) {
+      t.dev_off = off; t.dev_bytes = t.bytes_out; t.dev_held = true;
+    } else if (requested == CSWAP_POLICY_AUTO) {
+      t.policy = CSWAP_POLICY_NONE;  // no staging room: the selector's choice degrades to the raw swap
+    } else {
+      abandon_device(e, t, compute);
+      return CSWAP_E_NOMEM;
     }
   }
   if (t.policy == CSWAP_POLICY_SPARSE) {
@@ -335,12 +340,14 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     int* d_begin = (int*)base;
     uint32_t* d_mask = (uint32_t*)(base + 4 * (size_t)t.process);
     float* d_values = (float*)(base + hdr);
+    // the scanned counts become the payload's offset table; the probe's block stays
+    // allocated until the ticket lets go of its staging, so nothing can reuse it under this copy
+    hipError_t err = hipMemcpyAsync(d_begin, e->d_base + t.probe_off, 4 * (size_t)t.process,
+                                    hipMemcpyDeviceToDevice, compute);
+    if (err != hipSuccess) { abandon_device(e, t, compute); return hip_fail(err); }
     if ((rc = cswap_zvc_compact(d_in, (int)n, t.process, d_begin, d_values, d_mask, compute))) {
       abandon_device(e, t, compute); return rc;
     }
-    t.bytes_out = hdr + 4 * t.nnz;
-    e->dpool.shrink(t.dev_off, t.dev_bytes, t.bytes_out);
-    t.dev_bytes = t.bytes_out;
     src = base;
   } else if (t.policy == CSWAP_POLICY_ZFP) {
     uint64_t* d_stream = (uint64_t*)(e->d_base + t.dev_off);

@@ -225,7 +225,7 @@ def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int =
     res = {"model": f"VGG-16 BN, batch {batch}, 3x{image}x{image}", "min_bytes": min_bytes}
     base_ms, base_mb, _ = measure(lambda: None)
     res["no_swap"] = {"step_ms": round(base_ms, 2), "step_peak_MB": round(base_mb, 1)}
-    staging = 512 << 20
+    staging = 192 << 20
     eng = swap.SwapEngine(pinned_bytes=4 << 30, device_bytes=staging)
     eng.calibrate()
     res["staging_pool_MB"] = round(staging / 1e6, 1)    # device memory the engine holds besides torch's allocator
