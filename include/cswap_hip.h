@@ -239,7 +239,10 @@ typedef struct cswap_engine cswap_engine;
 
 typedef struct {
   size_t pinned_pool_bytes;   /* host side: compressed tensors live here while swapped out */
-  size_t device_pool_bytes;   /* device staging for compressed data in flight */
+  size_t device_pool_bytes;   /* device staging for compressed data in flight: every tensor between swap_out and
+                                 swap_wait, and between prefetch / swap_in and release, holds a block of its
+                                 compressed size (raw swaps hold none going out).  When the pool is full an
+                                 AUTO request goes out raw, an explicit one and a prefetch return CSWAP_E_NOMEM. */
   int    process;             /* ZVC chunk count; 0 = per tensor size (cswap_engine_tune result, else cswap_zvc_pick_process) */
   unsigned zfp_maxbits;       /* bits per 4x4x4 block for policy ZFP; 0 = 512 (8 bits/value) */
   int    max_tickets;         /* tensors that may be swapped out at once; 0 = 256 */
