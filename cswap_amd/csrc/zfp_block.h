@@ -695,10 +695,12 @@ struct BlockDecoder {
     unsigned left = sub_sat(limit, pos);
     unsigned m = n < left ? n : left;
     uint64_t w = window(pos);
-    uint64_t x = w & low_mask(m);
+    uint64_t above = w >> (m & 63);               // what follows the m verbatim bits (m = 64: not used)
+    settle(above);                                // one shift serves the verbatim mask and the group test
+    uint64_t x = w ^ (m < 64 ? above << m : 0);   // the low m bits of w
     pos += m;
     bool go = n < SIZE && pos < limit;            // a group test follows (then m = n < 64)
-    bool test = go && ((w >> (m & 63)) & 1);
+    bool test = go && ((uint32_t)above & 1u);
     pos += go ? 1u : 0u;
     while (test) {                                // positive group test: a run of zeros, then a one
       w = window(pos);
@@ -718,7 +720,7 @@ struct BlockDecoder {
       // not found: n == SIZE or the budget is spent, either way the plane is over;
       // found: t <= 62, so the next group test (bit t + 1) is still inside this window
       go = found && n < SIZE && pos < limit;
-      test = go && ((w >> ((t + 1) & 63)) & 1);
+      test = go && ((uint32_t)(w >> ((t + 1) & 63)) & 1u);
       pos += go ? 1u : 0u;
     }
     return x;
