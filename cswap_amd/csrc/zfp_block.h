@@ -845,16 +845,14 @@ CSWAP_HD void decode_block_zy(Mem& mem, unsigned pos0, unsigned maxbits, int32_t
 {
   BlockDecoder<Mem, 64, FENCED> dec(mem, pos0, maxbits);
   uint32_t h = (uint32_t)dec.window(pos0);
-  if (!(h & 1)) {
-#pragma unroll
-    for (int i = 0; i < 64; i++) ib[i] = 0;
-    w = 0.0f;
-    return;
-  }
+  // An empty block (flag bit 0) takes the same path with its bit budget already
+  // spent: every plane then reads as zero, the coefficients come out as zero and
+  // the scale is zero, i.e. +0.0 everywhere, without a separate zero-fill of ib.
+  const bool coded = (h & 1) != 0;
   int emax = (int)((h >> 1) & 0xff) - 127;
-  dec.pos = pos0 + 9;
+  dec.pos = coded ? pos0 + 9 : dec.limit;
   decode_ints3_zy(dec, ib);
-  w = pow2f(emax - 30);
+  w = coded ? pow2f(emax - 30) : 0.0f;
 }
 
 // int32 block (zfp_type_int32): no header; finish each x-row with inv_lift4
