@@ -134,6 +134,21 @@ CSWAP_HD float pow2f(int e)
   return 0.0f;
 }
 
+// 2^(e8 - 157) for the 8-bit exponent field e8 of a block header (0..255): the
+// decoder's scale 2^(emax - 30) with emax = e8 - 127, as ldexpf(1, emax - 30)
+// gives it: normal from e8 = 31, subnormal down to e8 = 8, zero below.
+CSWAP_HD float decode_scale(uint32_t e8)
+{
+  uint32_t normal = (e8 - 30u) << 23;
+  uint32_t sub = e8 >= 8u ? 1u << ((e8 - 8u) & 31u) : 0u;
+  return f32_from_bits(e8 >= 31u ? normal : sub);
+}
+
+// The encoder's scale 2^(30 - emax) = 2^(157 - e) for the header exponent
+// e = emax + 127 of a non-empty block (1..256): the exponent is -99..156, i.e. a
+// normal float, or +inf above 127, as (float)ldexp(1.0, 30 - emax) gives it.
+CSWAP_HD float encode_scale(uint32_t e) { return f32_from_bits(e < 30u ? 0x7f800000u : (284u - e) << 23); }
+
 // ---------------------------------------------------------------- lifting
 // wrap-around int32 arithmetic (as on the GPU the reference runs on)
 CSWAP_HD int32_t wadd(int32_t a, int32_t b) { return (int32_t)((uint32_t)a + (uint32_t)b); }
@@ -561,7 +576,7 @@ CSWAP_HD void encode_block(const float (&f)[64], unsigned pos0, unsigned maxbits
   enc.put(2 * e + 1, 9);
 
   // block-floating-point cast: scale 2^(30-emax) as a float, truncate
-  float s = pow2f(30 - ((int)e - 127));
+  float s = encode_scale(e);
   int32_t ib[64];
 #pragma unroll
   for (int i = 0; i < 64; i++) ib[i] = (int32_t)(s * f[i]);
@@ -849,10 +864,9 @@ CSWAP_HD void decode_block_zy(Mem& mem, unsigned pos0, unsigned maxbits, int32_t
   // spent: every plane then reads as zero, the coefficients come out as zero and
   // the scale is zero, i.e. +0.0 everywhere, without a separate zero-fill of ib.
   const bool coded = (h & 1) != 0;
-  int emax = (int)((h >> 1) & 0xff) - 127;
   dec.pos = coded ? pos0 + 9 : dec.limit;
   decode_ints3_zy(dec, ib);
-  w = coded ? pow2f(emax - 30) : 0.0f;
+  w = coded ? decode_scale((h >> 1) & 0xffu) : 0.0f;
 }
 
 // int32 block (zfp_type_int32): no header; finish each x-row with inv_lift4
