@@ -144,11 +144,6 @@ CSWAP_HD float decode_scale(uint32_t e8)
   return f32_from_bits(e8 >= 31u ? normal : sub);
 }
 
-// The encoder's scale 2^(30 - emax) = 2^(157 - e) for the header exponent
-// e = emax + 127 of a non-empty block (1..256): the exponent is -99..156, i.e. a
-// normal float, or +inf above 127, as (float)ldexp(1.0, 30 - emax) gives it.
-CSWAP_HD float encode_scale(uint32_t e) { return f32_from_bits(e < 30u ? 0x7f800000u : (284u - e) << 23); }
-
 // ---------------------------------------------------------------- lifting
 // wrap-around int32 arithmetic (as on the GPU the reference runs on)
 CSWAP_HD int32_t wadd(int32_t a, int32_t b) { return (int32_t)((uint32_t)a + (uint32_t)b); }
@@ -575,8 +570,9 @@ CSWAP_HD void encode_block(const float (&f)[64], unsigned pos0, unsigned maxbits
   BlockEncoder<Mem, GUARD> enc(mem, pos0, maxbits);
   enc.put(2 * e + 1, 9);
 
-  // block-floating-point cast: scale 2^(30-emax) as a float, truncate
-  float s = encode_scale(e);
+  // block-floating-point cast: scale 2^(30-emax) as a float, truncate.  (A branch-free
+  // form of this power of two costs the register allocator three spills at 96 registers.)
+  float s = pow2f(30 - ((int)e - 127));
   int32_t ib[64];
 #pragma unroll
   for (int i = 0; i < 64; i++) ib[i] = (int32_t)(s * f[i]);

@@ -176,16 +176,6 @@ uint32_t host_div31(uint32_t b, uint32_t d) { return cswap::div31(b, cswap::make
 
 float host_decode_scale(uint32_t e8) { return cswap::decode_scale(e8); }
 
-// the encoder's scale for header exponent e, through a one-value block: returns (int32)(s * v)
-int32_t host_encode_cast(float v)
-{
-  float f[64];
-  for (int i = 0; i < 64; i++) f[i] = 0.0f;
-  f[0] = v;
-  uint32_t e = cswap::block_header_e(f);
-  float s = cswap::encode_scale(e);
-  return (int32_t)(s * v);
-}
 void host_transpose32(uint32_t* a) { uint32_t t[32]; memcpy(t, a, sizeof t); cswap::transpose32(t); memcpy(a, t, sizeof t); }
 
 

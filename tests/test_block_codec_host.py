@@ -49,9 +49,8 @@ def test_multiply_shift_division_matches_integer_division(host):
 
 
 def test_scale_factors_equal_ldexp(host):
-    """The decoder's 2^(emax-30) for every 8-bit header exponent and the encoder's
-    cast of a block's largest value, against ldexp (the reference's LDEXP,
-    encode.cuh:120-149, shared.h:184-205)."""
+    """The decoder's 2^(emax-30) for every 8-bit header exponent against ldexp
+    (the reference's LDEXP, shared.h:184-205)."""
     import math
 
     host.host_decode_scale.restype = C.c_float
@@ -59,15 +58,6 @@ def test_scale_factors_equal_ldexp(host):
     for e8 in range(256):
         want = np.float32(math.ldexp(1.0, e8 - 127 - 30))
         assert np.float32(host.host_decode_scale(e8)).view(np.uint32) == want.view(np.uint32), e8
-    host.host_encode_cast.restype = C.c_int32
-    host.host_encode_cast.argtypes = [C.c_float]
-    rng = np.random.default_rng(1)
-    for ex in range(-96, 128):                       # below 2^-97 the reference's scale overflows
-        v = np.float32(math.ldexp(float(rng.uniform(0.5, 1.0)), ex)) * np.float32(rng.choice([-1, 1]))
-        emax = math.frexp(abs(float(v)))[1]
-        want = int(np.float32(np.float32(math.ldexp(1.0, 30 - emax)) * v))
-        assert host.host_encode_cast(float(v)) == want, (ex, v)
-        assert 2**29 <= abs(want) < 2**30
 
 
 def test_transpose32_is_a_bit_matrix_transpose(host):
