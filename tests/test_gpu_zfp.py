@@ -2,6 +2,7 @@
 be bit-exact against the committed zfp 0.5.5 golden vectors and against the CPU
 checker on the same seeded inputs."""
 import hashlib
+import os
 
 import numpy as np
 import pytest
@@ -544,3 +545,77 @@ def test_random_shapes_rates_types_and_strides_vs_checker(torch_cuda):
         outside = np.ones(big_shape, dtype=bool)
         outside[sl] = False
         assert not back[outside].any(), tag
+
+
+def _libzfp():
+    """The stock zfp 0.5.5 library of the build image (the codec version the
+    reference snapshots, CSWAP+/zfp/version.h:9-15; not part of the reference tree),
+    if this machine has it."""
+    import ctypes as C
+    import ctypes.util
+
+    for cand in ("/opt/conda/lib/libzfp.so.0.5.5", ctypes.util.find_library("zfp")):
+        if cand and (os.path.exists(cand) or "/" not in cand):
+            try:
+                L = C.CDLL(cand)
+            except OSError:
+                continue
+            L.stream_open.restype = C.c_void_p
+            L.stream_open.argtypes = [C.c_void_p, C.c_size_t]
+            L.stream_close.argtypes = [C.c_void_p]
+            L.zfp_stream_open.restype = C.c_void_p
+            L.zfp_stream_open.argtypes = [C.c_void_p]
+            L.zfp_stream_close.argtypes = [C.c_void_p]
+            L.zfp_stream_set_rate.restype = C.c_double
+            L.zfp_stream_set_rate.argtypes = [C.c_void_p, C.c_double, C.c_int, C.c_uint, C.c_int]
+            L.zfp_stream_rewind.argtypes = [C.c_void_p]
+            L.zfp_field_3d.restype = C.c_void_p
+            L.zfp_field_3d.argtypes = [C.c_void_p, C.c_int, C.c_uint, C.c_uint, C.c_uint]
+            L.zfp_field_free.argtypes = [C.c_void_p]
+            L.zfp_compress.restype = C.c_size_t
+            L.zfp_compress.argtypes = [C.c_void_p, C.c_void_p]
+            L.zfp_decompress.restype = C.c_size_t
+            L.zfp_decompress.argtypes = [C.c_void_p, C.c_void_p]
+            return L
+    return None
+
+
+def test_full_size_tensor_equals_the_zfp_library(torch_cuda):
+    """The benchmark's own 402 MB tensor (softmax(N(0,1)) [32,12,512,512], field
+    512 x 512 x 384, rate 8) against the stock zfp 0.5.5 serial codec running on
+    this machine's CPU: all 100,663,296 stream bytes and all decoded values."""
+    torch = torch_cuda
+    from cswap_amd import api
+
+    L = _libzfp()
+    if L is None:
+        pytest.skip("no zfp 0.5.5 library on this machine")
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    x = torch.softmax(torch.randn((32, 12, 512, 512), generator=g, device="cuda"), dim=-1).contiguous()
+    s = api.cuda_compress(x, 512)
+    d = api.cuda_decompress(s, x.shape, 512)
+    torch.cuda.synchronize()
+    xs = x.cpu().numpy().reshape(384, 512, 512)
+    nbytes = s.numel()
+    assert nbytes == xs.size                                   # 8 bits per value
+    buf = np.zeros(nbytes + 64, dtype=np.uint8)
+    bs = L.stream_open(buf.ctypes.data, buf.size)
+    zs = L.zfp_stream_open(bs)
+    assert L.zfp_stream_set_rate(zs, 8.0, 3, 3, 0) == 8.0       # zfp_type_float = 3
+    fld = L.zfp_field_3d(xs.ctypes.data, 3, 512, 512, 384)
+    L.zfp_stream_rewind(zs)
+    print("zfp library: compressing 402 MB on one core", flush=True)
+    assert L.zfp_compress(zs, fld) == nbytes
+    got = s.cpu().numpy()
+    assert np.array_equal(got, buf[:nbytes])
+    out = np.empty_like(xs)
+    fo = L.zfp_field_3d(out.ctypes.data, 3, 512, 512, 384)
+    L.zfp_stream_rewind(zs)
+    print("zfp library: decompressing", flush=True)
+    assert L.zfp_decompress(zs, fo) == nbytes
+    assert np.array_equal(d.cpu().numpy().reshape(out.shape).view(np.uint32), out.view(np.uint32))
+    for f in (fld, fo):
+        L.zfp_field_free(f)
+    L.zfp_stream_close(zs)
+    L.stream_close(bs)
