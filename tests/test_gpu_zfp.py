@@ -619,3 +619,73 @@ def test_full_size_tensor_equals_the_zfp_library(torch_cuda):
         L.zfp_field_free(f)
     L.zfp_stream_close(zs)
     L.stream_close(bs)
+
+
+@pytest.mark.parametrize("kind", ["f32", "i32", "f64", "i64"])
+@pytest.mark.parametrize("shape,rate", [((33, 47, 65), 8.0), ((64, 64, 64), 16.0), ((300, 257), 12.0), ((70001,), 10.0),
+                                        ((9, 130, 130), 3.0)])
+def test_mid_size_fields_equal_the_zfp_library(torch_cuda, kind, shape, rate):
+    """Fields of a few hundred thousand values of every scalar type and
+    dimensionality against the stock zfp 0.5.5 library on this machine's CPU."""
+    torch = torch_cuda
+    import ctypes as C
+
+    from cswap_amd._lib import check, lib
+
+    Z = _libzfp()
+    if Z is None:
+        pytest.skip("no zfp 0.5.5 library on this machine")
+    for fn in ("zfp_field_1d", "zfp_field_2d"):
+        getattr(Z, fn).restype = C.c_void_p
+    Z.zfp_field_1d.argtypes = [C.c_void_p, C.c_int, C.c_uint]
+    Z.zfp_field_2d.argtypes = [C.c_void_p, C.c_int, C.c_uint, C.c_uint]
+    npdt, ztype = {"f32": (np.float32, 3), "i32": (np.int32, 1), "f64": (np.float64, 4), "i64": (np.int64, 2)}[kind]
+    rng = np.random.default_rng(len(shape) * 1000 + int(rate))
+    smooth = np.cumsum(rng.standard_normal(shape), axis=-1)
+    if kind[0] == "i":
+        f = np.ascontiguousarray((smooth * (1 << (20 if kind == "i32" else 40))).astype(npdt))
+    else:
+        f = np.ascontiguousarray(smooth.astype(npdt))
+    dims = f.ndim
+    nz, ny, nx = (1,) * (3 - dims) + f.shape
+
+    def field(arr):
+        if dims == 3:
+            return Z.zfp_field_3d(arr.ctypes.data, ztype, nx, ny, nz)
+        if dims == 2:
+            return Z.zfp_field_2d(arr.ctypes.data, ztype, nx, ny)
+        return Z.zfp_field_1d(arr.ctypes.data, ztype, nx)
+
+    buf = np.zeros(f.nbytes + 4096, dtype=np.uint8)
+    bs = Z.stream_open(buf.ctypes.data, buf.size)
+    zs = Z.zfp_stream_open(bs)
+    Z.zfp_stream_set_rate(zs, rate, ztype, dims, 0)
+    maxbits = int((C.c_uint * 4).from_address(zs)[1])           # zfp_stream: minbits, maxbits, maxprec, minexp
+    fi = field(f)
+    Z.zfp_stream_rewind(zs)
+    n = Z.zfp_compress(zs, fi)
+    assert n > 0
+
+    L = lib()
+    t = torch.from_numpy(f).cuda()
+    cap = L.cswap_zfp_stream_capacity_nd(dims, nx, ny, nz, maxbits)
+    s = torch.zeros(cap, dtype=torch.uint8, device="cuda")
+    check(getattr(L, f"cswap_zfp_compress_{kind}_nd")(t.data_ptr(), dims, nx, ny, nz, 0, 0, 0, maxbits,
+                                                        s.data_ptr(), None), "compress")
+    got = s.cpu().numpy()
+    k = min(n, cap)
+    assert np.array_equal(got[:k], buf[:k]), (kind, shape, maxbits)
+    assert not got[k:].any() and not buf[k:n].any()
+    o = torch.zeros_like(t)
+    check(getattr(L, f"cswap_zfp_decompress_{kind}_nd")(s.data_ptr(), dims, nx, ny, nz, 0, 0, 0, maxbits,
+                                                          o.data_ptr(), None), "decompress")
+    torch.cuda.synchronize()
+    out = np.empty_like(f)
+    fo = field(out)
+    Z.zfp_stream_rewind(zs)
+    Z.zfp_decompress(zs, fo)
+    assert np.array_equal(o.cpu().numpy().view(np.uint8), out.view(np.uint8)), (kind, shape, maxbits)
+    Z.zfp_field_free(fi)
+    Z.zfp_field_free(fo)
+    Z.zfp_stream_close(zs)
+    Z.stream_close(bs)
