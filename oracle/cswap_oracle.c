@@ -31,6 +31,9 @@
  *       vectors of 1, 2 and 3 dimensions (tests/golden/zfp_golden_i32.npz).
  *   orc_zfp_encode_64 / orc_zfp_decode_64 : byte-exact against zfp 0.5.5 -d and
  *       -t i64 vectors of 1, 2 and 3 dimensions (tests/golden/zfp_golden_64.npz).
+ *   all of the ZFP entry points above, additionally: byte-exact against the stock
+ *       zfp 0.5.5 library itself (where the machine has it) on fields of a few
+ *       hundred thousand values of every scalar type and dimensionality.
  *   orc_zvc_* : numpy boolean indexing / packbits / cumsum.
  *
  * Undefined in the reference and therefore unpinned here: blocks whose largest

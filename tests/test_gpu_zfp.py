@@ -7,7 +7,7 @@ import os
 import numpy as np
 import pytest
 
-from conftest import golden_cases
+from conftest import MID_SIZE_CASES, golden_cases, libzfp as _libzfp, libzfp_round_trip, mid_size_field
 
 pytestmark = pytest.mark.gpu
 
@@ -547,39 +547,6 @@ def test_random_shapes_rates_types_and_strides_vs_checker(torch_cuda):
         assert not back[outside].any(), tag
 
 
-def _libzfp():
-    """The stock zfp 0.5.5 library of the build image (the codec version the
-    reference snapshots, CSWAP+/zfp/version.h:9-15; not part of the reference tree),
-    if this machine has it."""
-    import ctypes as C
-    import ctypes.util
-
-    for cand in ("/opt/conda/lib/libzfp.so.0.5.5", ctypes.util.find_library("zfp")):
-        if cand and (os.path.exists(cand) or "/" not in cand):
-            try:
-                L = C.CDLL(cand)
-            except OSError:
-                continue
-            L.stream_open.restype = C.c_void_p
-            L.stream_open.argtypes = [C.c_void_p, C.c_size_t]
-            L.stream_close.argtypes = [C.c_void_p]
-            L.zfp_stream_open.restype = C.c_void_p
-            L.zfp_stream_open.argtypes = [C.c_void_p]
-            L.zfp_stream_close.argtypes = [C.c_void_p]
-            L.zfp_stream_set_rate.restype = C.c_double
-            L.zfp_stream_set_rate.argtypes = [C.c_void_p, C.c_double, C.c_int, C.c_uint, C.c_int]
-            L.zfp_stream_rewind.argtypes = [C.c_void_p]
-            L.zfp_field_3d.restype = C.c_void_p
-            L.zfp_field_3d.argtypes = [C.c_void_p, C.c_int, C.c_uint, C.c_uint, C.c_uint]
-            L.zfp_field_free.argtypes = [C.c_void_p]
-            L.zfp_compress.restype = C.c_size_t
-            L.zfp_compress.argtypes = [C.c_void_p, C.c_void_p]
-            L.zfp_decompress.restype = C.c_size_t
-            L.zfp_decompress.argtypes = [C.c_void_p, C.c_void_p]
-            return L
-    return None
-
-
 def test_full_size_tensor_equals_the_zfp_library(torch_cuda):
     """The benchmark's own 402 MB tensor (softmax(N(0,1)) [32,12,512,512], field
     512 x 512 x 384, rate 8) against the stock zfp 0.5.5 serial codec running on
@@ -622,50 +589,20 @@ def test_full_size_tensor_equals_the_zfp_library(torch_cuda):
 
 
 @pytest.mark.parametrize("kind", ["f32", "i32", "f64", "i64"])
-@pytest.mark.parametrize("shape,rate", [((33, 47, 65), 8.0), ((64, 64, 64), 16.0), ((300, 257), 12.0), ((70001,), 10.0),
-                                        ((9, 130, 130), 3.0)])
+@pytest.mark.parametrize("shape,rate", MID_SIZE_CASES)
 def test_mid_size_fields_equal_the_zfp_library(torch_cuda, kind, shape, rate):
     """Fields of a few hundred thousand values of every scalar type and
     dimensionality against the stock zfp 0.5.5 library on this machine's CPU."""
     torch = torch_cuda
-    import ctypes as C
-
     from cswap_amd._lib import check, lib
 
     Z = _libzfp()
     if Z is None:
         pytest.skip("no zfp 0.5.5 library on this machine")
-    for fn in ("zfp_field_1d", "zfp_field_2d"):
-        getattr(Z, fn).restype = C.c_void_p
-    Z.zfp_field_1d.argtypes = [C.c_void_p, C.c_int, C.c_uint]
-    Z.zfp_field_2d.argtypes = [C.c_void_p, C.c_int, C.c_uint, C.c_uint]
-    npdt, ztype = {"f32": (np.float32, 3), "i32": (np.int32, 1), "f64": (np.float64, 4), "i64": (np.int64, 2)}[kind]
-    rng = np.random.default_rng(len(shape) * 1000 + int(rate))
-    smooth = np.cumsum(rng.standard_normal(shape), axis=-1)
-    if kind[0] == "i":
-        f = np.ascontiguousarray((smooth * (1 << (20 if kind == "i32" else 40))).astype(npdt))
-    else:
-        f = np.ascontiguousarray(smooth.astype(npdt))
+    f = mid_size_field(kind, shape, rate)
+    maxbits, stream, dec = libzfp_round_trip(Z, f, rate)
     dims = f.ndim
     nz, ny, nx = (1,) * (3 - dims) + f.shape
-
-    def field(arr):
-        if dims == 3:
-            return Z.zfp_field_3d(arr.ctypes.data, ztype, nx, ny, nz)
-        if dims == 2:
-            return Z.zfp_field_2d(arr.ctypes.data, ztype, nx, ny)
-        return Z.zfp_field_1d(arr.ctypes.data, ztype, nx)
-
-    buf = np.zeros(f.nbytes + 4096, dtype=np.uint8)
-    bs = Z.stream_open(buf.ctypes.data, buf.size)
-    zs = Z.zfp_stream_open(bs)
-    Z.zfp_stream_set_rate(zs, rate, ztype, dims, 0)
-    maxbits = int((C.c_uint * 4).from_address(zs)[1])           # zfp_stream: minbits, maxbits, maxprec, minexp
-    fi = field(f)
-    Z.zfp_stream_rewind(zs)
-    n = Z.zfp_compress(zs, fi)
-    assert n > 0
-
     L = lib()
     t = torch.from_numpy(f).cuda()
     cap = L.cswap_zfp_stream_capacity_nd(dims, nx, ny, nz, maxbits)
@@ -673,19 +610,11 @@ def test_mid_size_fields_equal_the_zfp_library(torch_cuda, kind, shape, rate):
     check(getattr(L, f"cswap_zfp_compress_{kind}_nd")(t.data_ptr(), dims, nx, ny, nz, 0, 0, 0, maxbits,
                                                         s.data_ptr(), None), "compress")
     got = s.cpu().numpy()
-    k = min(n, cap)
-    assert np.array_equal(got[:k], buf[:k]), (kind, shape, maxbits)
-    assert not got[k:].any() and not buf[k:n].any()
+    k = min(stream.size, cap)
+    assert np.array_equal(got[:k], stream[:k]), (kind, shape, maxbits)
+    assert not got[k:].any() and not stream[k:].any()
     o = torch.zeros_like(t)
     check(getattr(L, f"cswap_zfp_decompress_{kind}_nd")(s.data_ptr(), dims, nx, ny, nz, 0, 0, 0, maxbits,
                                                           o.data_ptr(), None), "decompress")
     torch.cuda.synchronize()
-    out = np.empty_like(f)
-    fo = field(out)
-    Z.zfp_stream_rewind(zs)
-    Z.zfp_decompress(zs, fo)
-    assert np.array_equal(o.cpu().numpy().view(np.uint8), out.view(np.uint8)), (kind, shape, maxbits)
-    Z.zfp_field_free(fi)
-    Z.zfp_field_free(fo)
-    Z.zfp_stream_close(zs)
-    Z.stream_close(bs)
+    assert np.array_equal(o.cpu().numpy().view(np.uint8), dec.view(np.uint8)), (kind, shape, maxbits)

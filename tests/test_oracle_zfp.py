@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import oracle
-from conftest import golden_cases
+from conftest import MID_SIZE_CASES, golden_cases, libzfp, libzfp_round_trip, mid_size_field
 from cswap_amd.workloads import config1_field, config3_fields
 
 
@@ -349,3 +349,32 @@ def test_int32_high_rate_is_nearly_lossless():
     s = oracle.zfp_encode_i32(z, 512)
     assert not s.any()                       # zeros code as zero bits: every plane is a negative group test
     assert not oracle.zfp_decode_i32(s, z.shape, 512).any()
+
+
+@pytest.mark.parametrize("kind", ["f32", "i32", "f64", "i64"])
+@pytest.mark.parametrize("shape,rate", MID_SIZE_CASES)
+def test_checker_equals_the_zfp_library_on_mid_size_fields(kind, shape, rate):
+    """The checker against the stock zfp 0.5.5 library (where this machine has
+    it) on fields of a few hundred thousand values of every scalar type and
+    dimensionality: stream bytes and decoded values."""
+    import oracle
+
+    Z = libzfp()
+    if Z is None:
+        pytest.skip("no zfp 0.5.5 library on this machine")
+    f = mid_size_field(kind, shape, rate)
+    maxbits, stream, dec = libzfp_round_trip(Z, f, rate)
+    if kind == "f32":
+        s = oracle.zfp_encode_nd(f, maxbits)
+        d = oracle.zfp_decode_nd(s, f.shape, maxbits)
+    elif kind == "i32":
+        s = oracle.zfp_encode_i32(f, maxbits)
+        d = oracle.zfp_decode_i32(s, f.shape, maxbits)
+    else:
+        s = oracle.zfp_encode_64(f, maxbits)
+        d = oracle.zfp_decode_64(s, f.shape, maxbits, f.dtype)
+    sb = s.view(np.uint8)
+    k = min(sb.size, stream.size)
+    assert np.array_equal(sb[:k], stream[:k]), (kind, shape, maxbits)
+    assert not sb[k:].any() and not stream[k:].any()
+    assert np.array_equal(d.view(np.uint8), dec.view(np.uint8)), (kind, shape, maxbits)
