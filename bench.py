@@ -13,7 +13,8 @@ uncompressed fp32 pushed through the compress+decompress pair:
 The single JSON line also carries
   roofline      HBM-roofline figures of the dominant (slower) ZFP kernel, from
                 HIP-event timing of that kernel inside the timed region
-  cpu_baseline  the CPU checker (a port of the reference algorithm) timed on a
+  cpu_baseline  the CPU checker (a port of the reference algorithm; and the stock
+                zfp 0.5.5 library where the machine has it) timed on a
                 bounded sample of the same tensor on this host
   extra         the other kernels of the path (ZVC compact/expand, probe, other
                 rates, swap latency) -- reported, not the headline.
@@ -166,10 +167,72 @@ def cpu_baseline(x, maxbits):
     ser = pair(False)
     par = pair(True)
     threads = oracle.lib(True).orc_threads()
-    return {"value": round(nbytes / ser[0] / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "first 4 of 32 batch entries (50.3 MB) of the same tensor, compress+decompress, best of 3",
-            "compress_GBs": round(nbytes / ser[1] / 1e9, 4), "decompress_GBs": round(nbytes / ser[2] / 1e9, 4),
-            "all_cores": {"value": round(nbytes / par[0] / 1e9, 4), "cores": threads}}
+    res = {"value": round(nbytes / ser[0] / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+           "sample": "first 4 of 32 batch entries (50.3 MB) of the same tensor, compress+decompress, best of 3",
+           "compress_GBs": round(nbytes / ser[1] / 1e9, 4), "decompress_GBs": round(nbytes / ser[2] / 1e9, 4),
+           "all_cores": {"value": round(nbytes / par[0] / 1e9, 4), "cores": threads}}
+    z = zfp_library_pair(sample, maxbits)
+    if z is not None:
+        res["zfp_0_5_5_library"] = {"value": round(nbytes / z[0] / 1e9, 4), "cores": 1,
+                                    "compress_GBs": round(nbytes / z[1] / 1e9, 4),
+                                    "decompress_GBs": round(nbytes / z[2] / 1e9, 4),
+                                    "note": "stock serial codec of the image, same sample, best of 3"}
+    return res
+
+
+def zfp_library_pair(sample, maxbits):
+    """The stock zfp 0.5.5 serial codec (the version the reference snapshots), if
+    this machine has the library: (pair, compress, decompress) seconds, best of 3."""
+    import ctypes as C
+
+    import numpy as np
+
+    path = "/opt/conda/lib/libzfp.so.0.5.5"
+    if not os.path.exists(path):
+        return None
+    try:
+        Z = C.CDLL(path)
+    except OSError:
+        return None
+    vp = C.c_void_p
+    Z.stream_open.restype = vp; Z.stream_open.argtypes = [vp, C.c_size_t]
+    Z.stream_close.argtypes = [vp]
+    Z.zfp_stream_open.restype = vp; Z.zfp_stream_open.argtypes = [vp]
+    Z.zfp_stream_close.argtypes = [vp]
+    Z.zfp_stream_set_rate.restype = C.c_double
+    Z.zfp_stream_set_rate.argtypes = [vp, C.c_double, C.c_int, C.c_uint, C.c_int]
+    Z.zfp_stream_rewind.argtypes = [vp]
+    Z.zfp_field_3d.restype = vp; Z.zfp_field_3d.argtypes = [vp, C.c_int, C.c_uint, C.c_uint, C.c_uint]
+    Z.zfp_field_free.argtypes = [vp]
+    Z.zfp_compress.restype = C.c_size_t; Z.zfp_compress.argtypes = [vp, vp]
+    Z.zfp_decompress.restype = C.c_size_t; Z.zfp_decompress.argtypes = [vp, vp]
+    nz, ny, nx = sample.shape
+    buf = np.zeros(sample.nbytes + 4096, dtype=np.uint8)
+    out = np.empty_like(sample)
+    bs = Z.stream_open(buf.ctypes.data, buf.size)
+    zs = Z.zfp_stream_open(bs)
+    Z.zfp_stream_set_rate(zs, maxbits / 64.0, 3, 3, 0)
+    fi = Z.zfp_field_3d(sample.ctypes.data, 3, nx, ny, nz)
+    fo = Z.zfp_field_3d(out.ctypes.data, 3, nx, ny, nz)
+    best = None
+    for _ in range(3):
+        Z.zfp_stream_rewind(zs)
+        t0 = time.perf_counter()
+        n = Z.zfp_compress(zs, fi)
+        t1 = time.perf_counter()
+        Z.zfp_stream_rewind(zs)
+        Z.zfp_decompress(zs, fo)
+        t2 = time.perf_counter()
+        if n == 0:
+            best = None
+            break
+        cur = (t2 - t0, t1 - t0, t2 - t1)
+        best = cur if best is None or cur[0] < best[0] else best
+    for f in (fi, fo):
+        Z.zfp_field_free(f)
+    Z.zfp_stream_close(zs)
+    Z.stream_close(bs)
+    return best
 
 
 def extras(torch, api, dev):
