@@ -351,8 +351,7 @@ def test_reference_named_entry_points(torch_cuda):
     xf = x.cpu().numpy().reshape(-1, 32, 32)
     wantx = oracle.zfp_decode3(oracle.zfp_encode3(xf, 512), xf.shape, 512)
     assert np.array_equal(y.cpu().numpy().reshape(xf.shape).view(np.uint32), wantx.view(np.uint32))
-    import ctypes
-    hip = ctypes.CDLL("libamdhip64.so")
+    hip = C.CDLL("libamdhip64.so")                           # the default allocator is hipMalloc / hipFree
     hip.hipFree.argtypes = [ctypes.c_void_p]
     assert hip.hipFree(buf) == 0
 
@@ -533,6 +532,78 @@ def test_random_ticket_traffic_with_small_pools(torch_cuda):
     # both pools are whole again: one allocation of (almost) the full size fits
     big = torch.zeros(64, 64, (6 << 20) // 4 // 4096 - 1, device="cuda")       # 6 MiB less 16 KiB
     tk = eng.pre(big, swap.NONE)
+    eng.post(tk)
+    eng.release(tk)
+    eng.close()
+
+
+def test_compat_allocator_field_hint_and_copy_stream(torch_cuda):
+    """The knobs around the reference-named compress()/decompress(): a caller's
+    allocator receives the stream buffer request (the reference allocates through
+    c10, Execution.h:113-114), the field hint changes how a flat tensor is cut into
+    blocks, the engine's copy stream can be handed to torch, and the last HIP error
+    of a clean sequence is hipSuccess."""
+    torch = torch_cuda
+    import oracle
+    from cswap_amd import api, swap
+    from cswap_amd._lib import lib
+
+    L = lib()
+    calls = {"alloc": [], "free": []}
+    keep = {}
+    ALLOC = C.CFUNCTYPE(C.c_void_p, C.c_size_t)
+    FREE = C.CFUNCTYPE(None, C.c_void_p)
+
+    def my_alloc(nbytes):
+        t = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        keep[t.data_ptr()] = t
+        calls["alloc"].append(nbytes)
+        return t.data_ptr()
+
+    def my_free(p):
+        calls["free"].append(p)
+        keep.pop(p, None)
+
+    a, f = ALLOC(my_alloc), FREE(my_free)
+    x = torch.randn(64 * 64 * 32, device="cuda")
+    L.setRatio(128)
+    try:
+        L.cswap_set_allocator(C.cast(a, C.c_void_p), C.cast(f, C.c_void_p))
+        L.cswap_compat_set_field(64, 64)
+        nbytes = C.c_size_t(0)
+        buf = L.compress(x.data_ptr(), x.numel(), C.byref(nbytes))
+        assert buf in keep and calls["alloc"] == [nbytes.value] and nbytes.value == x.numel()
+        want = oracle.zfp_encode3(x.cpu().numpy().reshape(32, 64, 64), 512)
+        got = keep[buf].cpu().numpy().view(np.uint64)
+        assert np.array_equal(got, want)                      # blocks cut from the (64, 64, 32) field, not 32 x 32 rows
+        y = torch.empty_like(x)
+        assert L.decompress(buf, x.numel(), y.data_ptr()) == 0
+        torch.cuda.synchronize()
+        assert np.array_equal(y.cpu().numpy().view(np.uint32),
+                              oracle.zfp_decode3(want, (32, 64, 64), 512).reshape(-1).view(np.uint32))
+    finally:
+        L.cswap_compat_set_field(0, 0)
+        L.cswap_set_allocator(None, None)
+    # default layout again: 32 x 32 rows
+    nbytes = C.c_size_t(0)
+    buf2 = L.compress(x.data_ptr(), x.numel(), C.byref(nbytes))
+    assert buf2 and calls["alloc"] == [x.numel()]             # the default allocator served this one
+    s2 = api.cuda_compress(x.view(-1, 32, 32), 512)
+    torch.cuda.synchronize()
+    view = torch.empty(nbytes.value, dtype=torch.uint8, device="cuda")
+    hip = C.CDLL("libamdhip64.so")                           # the default allocator is hipMalloc / hipFree
+    assert hip.hipMemcpy(C.c_void_p(view.data_ptr()), C.c_void_p(buf2), C.c_size_t(nbytes.value), 3) == 0
+    assert torch.equal(view, s2[: nbytes.value])
+    assert hip.hipFree(C.c_void_p(buf2)) == 0
+    assert L.cswap_last_hip_error() == 0
+
+    eng = swap.SwapEngine(pinned_bytes=16 << 20, device_bytes=16 << 20)
+    h = L.cswap_engine_copy_stream(eng._h)
+    assert h
+    ext = torch.cuda.ExternalStream(h)
+    tk = eng.pre(x.view(64, 64, 32), swap.NONE)
+    ext.synchronize()                                         # the copy went onto that stream
+    assert eng.info(tk).state in (1, 2)
     eng.post(tk)
     eng.release(tk)
     eng.close()
