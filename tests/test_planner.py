@@ -235,3 +235,24 @@ def test_policy_maker_header_compiles_and_plans():
                                "-Wl,-rpath," + os.path.dirname(lib), "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib",
                                "-lamdhip64", "-o", exe])
         subprocess.check_call([exe])
+
+
+def test_backward_factor_scales_the_base_time_and_the_room_to_hide_copies():
+    """set_backward_factor: backward of op i takes factor x its forward time.  The
+    base time is (1 + factor) x the forward time, and a longer backward hides more
+    of every inbound copy, so the planned overhead cannot grow with it."""
+    from cswap_amd.planner import PolicyMaker
+
+    over = []
+    for factor in (0.5, 1.0, 2.0, 4.0):
+        pm = PolicyMaker(costs())
+        pm.set_backward_factor(factor)
+        vgg_like(pm, comptime=200.0)
+        pm.init(0.5)
+        pol, t = pm.make_policy(20)
+        s = pm.summary
+        assert s.base_time_us == pytest.approx(20 * 200.0 * (1.0 + factor))
+        assert s.target_met
+        over.append(t - s.base_time_us)
+    assert all(b <= a + 1e-6 for a, b in zip(over, over[1:])), over
+    assert over[0] > over[-1]
