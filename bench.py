@@ -58,6 +58,8 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain copy kernel of the same tensor (known traffic: 4N read, 4N "
                          "written) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE can be scaled")
+    ap.add_argument("--zvc-only", action="store_true",
+                    help="run only the 256 MiB ReLU zero-value-compaction case (for profiling); prints its figures")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; run with --gpus 1 "
@@ -73,6 +75,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.zvc_only:
+        print(json.dumps(extras(torch, api, dev, zvc_only=True)))
+        return
 
     rate = 8
     maxbits = 64 * rate
@@ -235,12 +240,88 @@ def zfp_library_pair(sample, maxbits):
     return best
 
 
-def extras(torch, api, dev):
+def zvc_extras(torch, api, dev, ex, config2_tensor, only_256=False):
+    # ---- ZVC compact / expand / probe
+    def zvc_case(label, t):
+        n = t.numel()
+        values, mask, begin, nnz = api.zvc_compress(t)
+        o = torch.empty_like(t)
+        api.GPUdecompression(values, o, mask, begin)
+        torch.cuda.synchronize()
+        k = int(nnz.item())
+        dens = k / n
+        reps = 10 if n > 1 << 24 else 50
+        from cswap_amd._lib import lib
+        L = lib()
+        st = torch.cuda.current_stream().cuda_stream
+        full = ev_ms(torch, lambda: L.cswap_zvc_compress(t.data_ptr(), n, api.PROCESS, begin.data_ptr(),
+                                                         nnz.data_ptr(), values.data_ptr(), mask.data_ptr(), st), reps)
+        ws = torch.empty(L.cswap_zvc_workspace_bytes(api.PROCESS), dtype=torch.uint8, device=dev)
+        fused = ev_ms(torch, lambda: L.cswap_zvc_compress_fused(t.data_ptr(), n, api.PROCESS, ws.data_ptr(),
+                                                                begin.data_ptr(), nnz.data_ptr(),
+                                                                values.data_ptr(), mask.data_ptr(), st), reps)
+        cnt = torch.zeros(api.PROCESS, dtype=torch.int32, device=dev)
+        count = ev_ms(torch, lambda: L.cswap_zvc_count(t.data_ptr(), n, api.PROCESS, cnt.data_ptr(), st), reps)
+        compact = ev_ms(torch, lambda: L.cswap_zvc_compact(t.data_ptr(), n, api.PROCESS, begin.data_ptr(),
+                                                           values.data_ptr(), mask.data_ptr(), st), reps)
+        expand = ev_ms(torch, lambda: api.GPUdecompression(values, o, mask, begin), reps)
+        pr = torch.zeros(1, dtype=torch.int64, device=dev)
+        probe = ev_ms(torch, lambda: api.probe_nnz(t, out=pr), reps)
+        bpv = 4 + 1 / 8 + 4 * dens
+        ex[f"zvc_{label}"] = {
+            "density": round(dens, 4), "ratio": round((4 * k + n / 8 + 4 * api.PROCESS) / (4 * n), 4),
+            "count_ms": round(count, 4), "compact_ms": round(compact, 4), "compress_total_ms": round(full, 4),
+            "compress_fused_ms": round(fused, 4),
+            "compress_fused_hbm_frac": round(bpv * n / fused / 1e6 / HBM_PEAK_GBS, 4),
+            "expand_ms": round(expand, 4), "probe_ms": round(probe, 4),
+            "compact_GBs_fp32": round(4 * n / compact / 1e6, 1), "expand_GBs_fp32": round(4 * n / expand / 1e6, 1),
+            "compact_hbm_frac": round(bpv * n / compact / 1e6 / HBM_PEAK_GBS, 4),
+            "compress_total_hbm_frac": round(bpv * n / full / 1e6 / HBM_PEAK_GBS, 4),
+            "expand_hbm_frac": round(bpv * n / expand / 1e6 / HBM_PEAK_GBS, 4),
+            "probe_hbm_frac": round(4 * n / probe / 1e6 / HBM_PEAK_GBS, 4)}
+
+    if not only_256:
+        for pct in (30, 50, 70, 90):
+            zvc_case(f"config2_s{pct}", torch.from_numpy(config2_tensor(pct)).to(dev))
+
+    # ---- ZVC chunk count: the reference's 512*32 against the size rule the engine uses
+    def geometry_case(mib):
+        from cswap_amd._lib import lib
+        L = lib()
+        n = mib * 1024 * 1024 // 4
+        t = torch.relu(torch.randn(n, device=dev))
+        o = torch.empty_like(t)
+        st = torch.cuda.current_stream().cuda_stream
+        row = {}
+        for label, process in (("reference_16384", api.PROCESS), ("size_rule", L.cswap_zvc_pick_process(n))):
+            _, W, _ = api.zvc_geometry(n, process)
+            values = torch.empty(n, device=dev)
+            mask = torch.empty(W * process, dtype=torch.int32, device=dev)
+            begin = torch.zeros(process, dtype=torch.int32, device=dev)
+            nnz = torch.zeros(1, dtype=torch.int32, device=dev)
+            c = ev_ms(torch, lambda: L.cswap_zvc_compress(t.data_ptr(), n, process, begin.data_ptr(), nnz.data_ptr(),
+                                                          values.data_ptr(), mask.data_ptr(), st), 30)
+            e = ev_ms(torch, lambda: L.cswap_zvc_expand(values.data_ptr(), mask.data_ptr(), begin.data_ptr(), n,
+                                                        process, o.data_ptr(), st), 30)
+            row[label] = {"process": process, "compress_ms": round(c, 4), "expand_ms": round(e, 4)}
+        ex[f"zvc_geometry_{mib}MiB"] = row
+
+    if not only_256:
+        for mib in (1, 4, 16, 32, 128):
+            geometry_case(mib)
+    g = torch.Generator(device=dev); g.manual_seed(1)
+    zvc_case("relu_256MiB", torch.relu(torch.randn(64 * 1024 * 1024, generator=g, device=dev)))
+    return ex
+
+
+def extras(torch, api, dev, zvc_only=False):
     import numpy as np
 
     from cswap_amd.workloads import config1_field, config2_tensor, field_dims
 
     ex = {}
+    if zvc_only:
+        return zvc_extras(torch, api, dev, ex, config2_tensor, only_256=True)
     # ---- ZFP at other rates and on configuration 1
     g = torch.Generator(device=dev); g.manual_seed(0)
     big = torch.softmax(torch.randn((32, 12, 512, 512), generator=g, device=dev), dim=-1).contiguous()
@@ -315,74 +396,7 @@ def extras(torch, api, dev):
             "decompress_hbm_frac": round(bpv * n / d / 1e6 / HBM_PEAK_GBS, 4)}
     del base
 
-    # ---- ZVC compact / expand / probe
-    def zvc_case(label, t):
-        n = t.numel()
-        values, mask, begin, nnz = api.zvc_compress(t)
-        o = torch.empty_like(t)
-        api.GPUdecompression(values, o, mask, begin)
-        torch.cuda.synchronize()
-        k = int(nnz.item())
-        dens = k / n
-        reps = 10 if n > 1 << 24 else 50
-        from cswap_amd._lib import lib
-        L = lib()
-        st = torch.cuda.current_stream().cuda_stream
-        full = ev_ms(torch, lambda: L.cswap_zvc_compress(t.data_ptr(), n, api.PROCESS, begin.data_ptr(),
-                                                         nnz.data_ptr(), values.data_ptr(), mask.data_ptr(), st), reps)
-        ws = torch.empty(L.cswap_zvc_workspace_bytes(api.PROCESS), dtype=torch.uint8, device=dev)
-        fused = ev_ms(torch, lambda: L.cswap_zvc_compress_fused(t.data_ptr(), n, api.PROCESS, ws.data_ptr(),
-                                                                begin.data_ptr(), nnz.data_ptr(),
-                                                                values.data_ptr(), mask.data_ptr(), st), reps)
-        cnt = torch.zeros(api.PROCESS, dtype=torch.int32, device=dev)
-        count = ev_ms(torch, lambda: L.cswap_zvc_count(t.data_ptr(), n, api.PROCESS, cnt.data_ptr(), st), reps)
-        compact = ev_ms(torch, lambda: L.cswap_zvc_compact(t.data_ptr(), n, api.PROCESS, begin.data_ptr(),
-                                                           values.data_ptr(), mask.data_ptr(), st), reps)
-        expand = ev_ms(torch, lambda: api.GPUdecompression(values, o, mask, begin), reps)
-        pr = torch.zeros(1, dtype=torch.int64, device=dev)
-        probe = ev_ms(torch, lambda: api.probe_nnz(t, out=pr), reps)
-        bpv = 4 + 1 / 8 + 4 * dens
-        ex[f"zvc_{label}"] = {
-            "density": round(dens, 4), "ratio": round((4 * k + n / 8 + 4 * api.PROCESS) / (4 * n), 4),
-            "count_ms": round(count, 4), "compact_ms": round(compact, 4), "compress_total_ms": round(full, 4),
-            "compress_fused_ms": round(fused, 4),
-            "compress_fused_hbm_frac": round(bpv * n / fused / 1e6 / HBM_PEAK_GBS, 4),
-            "expand_ms": round(expand, 4), "probe_ms": round(probe, 4),
-            "compact_GBs_fp32": round(4 * n / compact / 1e6, 1), "expand_GBs_fp32": round(4 * n / expand / 1e6, 1),
-            "compact_hbm_frac": round(bpv * n / compact / 1e6 / HBM_PEAK_GBS, 4),
-            "compress_total_hbm_frac": round(bpv * n / full / 1e6 / HBM_PEAK_GBS, 4),
-            "expand_hbm_frac": round(bpv * n / expand / 1e6 / HBM_PEAK_GBS, 4),
-            "probe_hbm_frac": round(4 * n / probe / 1e6 / HBM_PEAK_GBS, 4)}
-
-    for pct in (30, 50, 70, 90):
-        zvc_case(f"config2_s{pct}", torch.from_numpy(config2_tensor(pct)).to(dev))
-
-    # ---- ZVC chunk count: the reference's 512*32 against the size rule the engine uses
-    def geometry_case(mib):
-        from cswap_amd._lib import lib
-        L = lib()
-        n = mib * 1024 * 1024 // 4
-        t = torch.relu(torch.randn(n, device=dev))
-        o = torch.empty_like(t)
-        st = torch.cuda.current_stream().cuda_stream
-        row = {}
-        for label, process in (("reference_16384", api.PROCESS), ("size_rule", L.cswap_zvc_pick_process(n))):
-            _, W, _ = api.zvc_geometry(n, process)
-            values = torch.empty(n, device=dev)
-            mask = torch.empty(W * process, dtype=torch.int32, device=dev)
-            begin = torch.zeros(process, dtype=torch.int32, device=dev)
-            nnz = torch.zeros(1, dtype=torch.int32, device=dev)
-            c = ev_ms(torch, lambda: L.cswap_zvc_compress(t.data_ptr(), n, process, begin.data_ptr(), nnz.data_ptr(),
-                                                          values.data_ptr(), mask.data_ptr(), st), 30)
-            e = ev_ms(torch, lambda: L.cswap_zvc_expand(values.data_ptr(), mask.data_ptr(), begin.data_ptr(), n,
-                                                        process, o.data_ptr(), st), 30)
-            row[label] = {"process": process, "compress_ms": round(c, 4), "expand_ms": round(e, 4)}
-        ex[f"zvc_geometry_{mib}MiB"] = row
-
-    for mib in (1, 4, 16, 32, 128):
-        geometry_case(mib)
-    g = torch.Generator(device=dev); g.manual_seed(1)
-    zvc_case("relu_256MiB", torch.relu(torch.randn(64 * 1024 * 1024, generator=g, device=dev)))
+    zvc_extras(torch, api, dev, ex, config2_tensor)
 
     try:
         from cswap_amd import swap
