@@ -58,6 +58,8 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain copy kernel of the same tensor (known traffic: 4N read, 4N "
                          "written) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE can be scaled")
+    ap.add_argument("--swap-only", action="store_true",
+                    help="run only the swap schedule of configuration 4 and its backward walk (for profiling)")
     ap.add_argument("--zvc-only", action="store_true",
                     help="run only the 256 MiB ReLU zero-value-compaction case (for profiling); prints its figures")
     args = ap.parse_args()
@@ -77,6 +79,10 @@ def main():
     torch.cuda.set_device(dev)
     if args.zvc_only:
         print(json.dumps(extras(torch, api, dev, zvc_only=True)))
+        return
+    if args.swap_only:
+        from cswap_amd import swap
+        print(json.dumps({"swap": swap.bench_schedule(dev), "swap_backward": swap.bench_backward(dev)}))
         return
 
     rate = 8
