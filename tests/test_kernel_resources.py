@@ -21,10 +21,11 @@ HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 def test_zfp_fp32_kernels_fit_five_waves_without_scratch():
     src = os.path.join(ROOT, "cswap_amd", "csrc", "zfp_kernels.hip")
     with tempfile.TemporaryDirectory() as d:
+        from cswap_amd.build import HIPCC_FLAGS      # the flags the shipped library is built with
+
         out = subprocess.run(
-            [HIPCC, "-O3", "-std=c++17", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
-             "-packed-fp32-ops", "-Rpass-analysis=kernel-resource-usage", "--cuda-device-only", "-c", src,
-             "-o", os.path.join(d, "k.o")],
+            [HIPCC, *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", "--cuda-device-only", "-x", "hip",
+             "-c", src, "-o", os.path.join(d, "k.o")],
             capture_output=True, text=True, timeout=600)
     assert out.returncode == 0, out.stderr[-2000:]
     kernels = {}
