@@ -73,6 +73,11 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         self.stats = {"swapped": 0, "bytes_in": 0, "bytes_out": 0, "kept": 0, "shared": 0}
         super().__init__(self._pack, self._unpack)
 
+    def __exit__(self, *exc):
+        r = super().__exit__(*exc)
+        self._settle()     # forward is over: wait for the last outbound copies and let their device tensors go
+        return r
+
     # -- forward side
     def _settle(self, keep_in_flight: int = 0):
         """Wait for the oldest outbound copies until at most ``keep_in_flight`` are left."""
