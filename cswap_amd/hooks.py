@@ -102,7 +102,13 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
             return h
         self._settle(self.depth - 1)
         self._drain()
-        ticket = self.engine.pre(t.detach(), self.policy)
+        try:
+            ticket = self.engine.pre(t.detach(), self.policy)
+        except CswapError as err:
+            if err.code != E_NOMEM:
+                raise
+            self.stats["kept_no_room"] = self.stats.get("kept_no_room", 0) + 1
+            return t                     # pinned pool, staging pool or tickets exhausted: the tensor stays on the device
         info = self.engine.info(ticket)
         self.stats["swapped"] += 1
         self.stats["bytes_in"] += info.bytes_in

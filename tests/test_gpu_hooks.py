@@ -103,6 +103,24 @@ def test_tensor_saved_by_two_nodes_is_swapped_once(torch_cuda):
     eng.close()
 
 
+def test_full_pools_leave_tensors_on_the_device(torch_cuda):
+    """A pinned pool that holds only part of the activations: what does not fit
+    stays on the device, the step still runs and gradients stay bit-identical."""
+    torch = torch_cuda
+    from cswap_amd import swap
+    from cswap_amd.hooks import swap_saved_tensors
+
+    net = make_mlp(torch)
+    x = torch.randn(2048, 512, device="cuda")
+    loss0, g0 = grads(torch, net, x)
+    eng = swap.SwapEngine(pinned_bytes=12 << 20, device_bytes=64 << 20)       # the 8 MiB activations: one fits, not two
+    ctx = swap_saved_tensors(eng, policy=swap.NONE, min_bytes=1 << 16)
+    loss1, g1 = grads(torch, net, x, ctx)
+    assert loss1 == loss0 and all(torch.equal(a, b) for a, b in zip(g0, g1))
+    assert ctx.stats["swapped"] >= 1 and ctx.stats.get("kept_no_room", 0) >= 1, ctx.stats
+    eng.close()
+
+
 def test_conv_net_round_trip_close(torch_cuda):
     """Convolution backward is not bit-reproducible run to run, so compare with a
     tolerance; the swapped activations themselves are restored exactly."""
