@@ -238,6 +238,108 @@ static void abandon_device(cswap_engine* e, Ticket& t, hipStream_t compute)
   drop_device(e, t);
 }
 
+// ---- the four steps of a swap-out.  Each leaves the ticket consistent on failure:
+// whatever it holds is given back by abandon_device / the caller.
+
+// Counts the non-zeros of the tensor (one host round trip, Execution.h:92) and
+// leaves the per-chunk counts, scanned into offsets, in the ticket's probe block.
+// Without room for that block: CSWAP_E_NOMEM if the probe is required, else the
+// tensor is taken as dense.
+static int probe_tensor(cswap_engine* e, Ticket& t, const float* d_in, hipStream_t compute, bool required)
+{
+  const size_t cnt_bytes = 4 * (size_t)t.process;
+  size_t off;
+  if (!e->dpool.alloc(cnt_bytes, &off)) {
+    if (required) return CSWAP_E_NOMEM;
+    t.nnz = t.n;
+    return CSWAP_OK;
+  }
+  t.probe_off = off; t.probe_bytes = cnt_bytes; t.probe_held = true;
+  int* d_counts = (int*)(e->d_base + off);
+  int rc = cswap_zvc_count(d_in, (int)t.n, t.process, d_counts, compute);
+  if (!rc) rc = cswap_zvc_scan(d_counts, cswap_zvc_active_chunks((int)t.n, t.process), e->d_nnz, compute);
+  if (rc) { abandon_device(e, t, compute); return rc; }
+  hipError_t err = hipMemcpyAsync(e->h_nnz, e->d_nnz, sizeof(int), hipMemcpyDeviceToHost, compute);
+  if (err == hipSuccess) err = hipEventRecord(e->ev_probe, compute);
+  if (err == hipSuccess) err = hipEventSynchronize(e->ev_probe);
+  if (err != hipSuccess) { abandon_device(e, t, compute); return hip_fail(err); }
+  t.nnz = (size_t)*e->h_nnz;
+  return CSWAP_OK;
+}
+
+// Sizes the payload for t.policy and reserves its staging block (compressed
+// policies) and its host block.  A selector's request that finds no staging room
+// degrades to the raw swap; everything else that does not fit is CSWAP_E_NOMEM.
+static int reserve_blocks(cswap_engine* e, Ticket& t, int requested)
+{
+  if (t.policy == CSWAP_POLICY_ZFP && t.probe_held) {  // the counts are of no further use
+    e->dpool.free(t.probe_off, t.probe_bytes);         // (their kernels finished before the host read nnz)
+    t.probe_held = false;
+  }
+  if (t.policy == CSWAP_POLICY_SPARSE || t.policy == CSWAP_POLICY_ZFP) {
+    t.bytes_out = t.policy == CSWAP_POLICY_SPARSE ? zvc_header_bytes((int)t.n, t.process) + 4 * t.nnz
+                                                  : cswap_zfp_stream_capacity(t.nx, t.ny, t.nz, e->maxbits);
+    size_t off;
+    if (e->dpool.alloc(t.bytes_out, &off)) {
+      t.dev_off = off; t.dev_bytes = t.bytes_out; t.dev_held = true;
+    } else if (requested == CSWAP_POLICY_AUTO) {
+      t.policy = CSWAP_POLICY_NONE;
+    } else {
+      drop_device(e, t);
+      return CSWAP_E_NOMEM;
+    }
+  }
+  if (t.policy == CSWAP_POLICY_NONE) {
+    drop_device(e, t);  // a probe's block, if any
+    t.bytes_out = 4 * t.n;
+  }
+  size_t hoff;
+  if (!e->hpool.alloc(t.bytes_out, &hoff)) {
+    drop_device(e, t);
+    return CSWAP_E_NOMEM;
+  }
+  t.host_off = hoff; t.host_bytes = t.bytes_out;
+  return CSWAP_OK;
+}
+
+// Launches the compression of t.policy on the compute stream; *src is what the copy will read.
+static int compress_tensor(cswap_engine* e, Ticket& t, const float* d_in, hipStream_t compute, const void** src)
+{
+  int rc = CSWAP_OK;
+  if (t.policy == CSWAP_POLICY_SPARSE) {
+    // layout of the payload: [begin: process ints][mask][values: nnz floats]
+    const size_t hdr = zvc_header_bytes((int)t.n, t.process);
+    char* base = e->d_base + t.dev_off;
+    int* d_begin = (int*)base;
+    // the scanned counts become the payload's offset table; the probe's block stays
+    // allocated until the ticket lets go of its staging, so nothing can reuse it under this copy
+    hipError_t err = hipMemcpyAsync(d_begin, e->d_base + t.probe_off, 4 * (size_t)t.process,
+                                    hipMemcpyDeviceToDevice, compute);
+    if (err != hipSuccess) return hip_fail(err);
+    rc = cswap_zvc_compact(d_in, (int)t.n, t.process, d_begin, (float*)(base + hdr),
+                           (uint32_t*)(base + 4 * (size_t)t.process), compute);
+    *src = base;
+  } else if (t.policy == CSWAP_POLICY_ZFP) {
+    uint64_t* d_stream = (uint64_t*)(e->d_base + t.dev_off);
+    rc = cswap_zfp_compress_f32(d_in, t.nx, t.ny, t.nz, 0, 0, 0, e->maxbits, d_stream, compute);
+    *src = d_stream;
+  } else {
+    *src = d_in;
+  }
+  return rc;
+}
+
+// Device-to-host copy on the copy stream, ordered after the compression by an event.
+static int start_outbound_copy(cswap_engine* e, Ticket& t, const void* src, hipStream_t compute)
+{
+  hipError_t err = hipEventRecord(t.ev_ready, compute);
+  if (err == hipSuccess) err = hipStreamWaitEvent(e->copy, t.ev_ready, 0);
+  if (err == hipSuccess)
+    err = hipMemcpyAsync(e->h_base + t.host_off, src, t.bytes_out, hipMemcpyDeviceToHost, e->copy);
+  if (err == hipSuccess) err = hipEventRecord(t.ev_copy, e->copy);
+  return err == hipSuccess ? CSWAP_OK : hip_fail(err);
+}
+
 extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, size_t ny, size_t nz, int policy,
                               cswap_stream_t compute_, int* ticket)
 {
@@ -258,7 +360,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   if (id < 0) return CSWAP_E_NOMEM;
   Ticket& t = e->tickets[(size_t)id];
   const int requested = policy;
-  t.policy = policy; t.n = n; t.nnz = 0; t.nx = nx; t.ny = ny; t.nz = nz;
+  t.policy = policy; t.n = n; t.nnz = n; t.nx = nx; t.ny = ny; t.nz = nz;
   t.dev_held = false;
   t.probe_held = false;
   t.process = zvc_ok ? process_for(e, n) : 0;
@@ -274,113 +376,29 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     cswap_choice best_case;
     if ((rc = cswap_select_field(nx, ny, nz, 0, e->maxbits, &costs, &best_case))) return rc;
     if (best_case.policy == CSWAP_POLICY_NONE) {
-      policy = t.policy = CSWAP_POLICY_NONE;
+      t.policy = CSWAP_POLICY_NONE;
       want_probe = false;
     }
   }
-  if (want_probe) {
-    // The probe needs room for the chunk counts only; the payload is allocated
-    // once nnz is known, at its exact size.
-    const size_t cnt_bytes = 4 * (size_t)t.process;
-    size_t off;
-    if (e->dpool.alloc(cnt_bytes, &off)) {
-      t.probe_off = off; t.probe_bytes = cnt_bytes; t.probe_held = true;
-      int* d_counts = (int*)(e->d_base + off);
-      if ((rc = cswap_zvc_count(d_in, (int)n, t.process, d_counts, compute))) { abandon_device(e, t, compute); return rc; }
-      if ((rc = cswap_zvc_scan(d_counts, cswap_zvc_active_chunks((int)n, t.process), e->d_nnz, compute))) {
-        abandon_device(e, t, compute); return rc;
-      }
-      hipError_t err = hipMemcpyAsync(e->h_nnz, e->d_nnz, sizeof(int), hipMemcpyDeviceToHost, compute);
-      if (err == hipSuccess) err = hipEventRecord(e->ev_probe, compute);
-      if (err == hipSuccess) err = hipEventSynchronize(e->ev_probe);  // the one host round trip (Execution.h:92)
-      if (err != hipSuccess) { abandon_device(e, t, compute); return hip_fail(err); }
-      t.nnz = (size_t)*e->h_nnz;
-    } else if (policy == CSWAP_POLICY_SPARSE) {
-      return CSWAP_E_NOMEM;
-    } else {
-      t.nnz = n;  // no room to probe: treat as dense
-    }
-  } else {
-    t.nnz = n;
-  }
-
-  if (policy == CSWAP_POLICY_AUTO) {
+  if (want_probe && (rc = probe_tensor(e, t, d_in, compute, policy == CSWAP_POLICY_SPARSE))) return rc;
+  if (t.policy == CSWAP_POLICY_AUTO) {
     cswap_choice ch;
-    cswap_costs c = costs;
-    if (!t.probe_held) c.sparse_max_ratio = 0.0;  // not probed: ZVC is not an option
-    if ((rc = cswap_select_field(nx, ny, nz, t.nnz, e->maxbits, &c, &ch))) { drop_device(e, t); return rc; }
+    if (!t.probe_held) costs.sparse_max_ratio = 0.0;  // not probed: ZVC is not an option
+    if ((rc = cswap_select_field(nx, ny, nz, t.nnz, e->maxbits, &costs, &ch))) { drop_device(e, t); return rc; }
     t.policy = ch.policy;
   }
 
-  // ---- compress on the compute stream into a staging block of the exact size
+  if ((rc = reserve_blocks(e, t, requested))) return rc;
   const void* src = nullptr;
-  if (t.policy == CSWAP_POLICY_SPARSE) {
-    t.bytes_out = zvc_header_bytes((int)n, t.process) + 4 * t.nnz;
-  } else if (t.policy == CSWAP_POLICY_ZFP) {
-    t.bytes_out = cswap_zfp_stream_capacity(nx, ny, nz, e->maxbits);
-    if (t.probe_held) {  // the counts are of no further use (their kernels finished before the host read nnz)
-      e->dpool.free(t.probe_off, t.probe_bytes);
-      t.probe_held = false;
-    }
-  }
-  if (t.policy == CSWAP_POLICY_SPARSE || t.policy == CSWAP_POLICY_ZFP) {
-    size_t off;
-    if (e->dpool.alloc(t.bytes_out, &off)) {
-      t.dev_off = off; t.dev_bytes = t.bytes_out; t.dev_held = true;
-    } else if (requested == CSWAP_POLICY_AUTO) {
-      t.policy = CSWAP_POLICY_NONE;  // no staging room: the selector's choice degrades to the raw swap
-    } else {
-      abandon_device(e, t, compute);
-      return CSWAP_E_NOMEM;
-    }
-  }
-  if (t.policy == CSWAP_POLICY_SPARSE) {
-    const size_t hdr = zvc_header_bytes((int)n, t.process);
-    char* base = e->d_base + t.dev_off;
-    int* d_begin = (int*)base;
-    uint32_t* d_mask = (uint32_t*)(base + 4 * (size_t)t.process);
-    float* d_values = (float*)(base + hdr);
-    // the scanned counts become the payload's offset table; the probe's block stays
-    // allocated until the ticket lets go of its staging, so nothing can reuse it under this copy
-    hipError_t err = hipMemcpyAsync(d_begin, e->d_base + t.probe_off, 4 * (size_t)t.process,
-                                    hipMemcpyDeviceToDevice, compute);
-    if (err != hipSuccess) { abandon_device(e, t, compute); return hip_fail(err); }
-    if ((rc = cswap_zvc_compact(d_in, (int)n, t.process, d_begin, d_values, d_mask, compute))) {
-      abandon_device(e, t, compute); return rc;
-    }
-    src = base;
-  } else if (t.policy == CSWAP_POLICY_ZFP) {
-    uint64_t* d_stream = (uint64_t*)(e->d_base + t.dev_off);
-    if ((rc = cswap_zfp_compress_f32(d_in, nx, ny, nz, 0, 0, 0, e->maxbits, d_stream, compute))) {
-      abandon_device(e, t, compute); return rc;
-    }
-    src = d_stream;
-  } else {
-    drop_device(e, t);  // a probe's block, if any: its kernels finished before the host read nnz
-    t.bytes_out = 4 * n;
-    src = d_in;
-  }
-
-  size_t hoff;
-  if (!e->hpool.alloc(t.bytes_out, &hoff)) {
-    // the compression kernel may still be writing the staging block: let it finish before the block is reused
-    (void)hipStreamSynchronize(compute);
-    drop_device(e, t);
-    return CSWAP_E_NOMEM;
-  }
-  t.host_off = hoff; t.host_bytes = t.bytes_out;
-
-  // ---- copy on the copy stream, ordered after the compression by an event
-  hipError_t err = hipEventRecord(t.ev_ready, compute);
-  if (err == hipSuccess) err = hipStreamWaitEvent(e->copy, t.ev_ready, 0);
-  if (err == hipSuccess) err = hipMemcpyAsync(e->h_base + hoff, src, t.bytes_out, hipMemcpyDeviceToHost, e->copy);
-  if (err == hipSuccess) err = hipEventRecord(t.ev_copy, e->copy);
-  if (err != hipSuccess) {
+  rc = compress_tensor(e, t, d_in, compute, &src);
+  if (!rc) rc = start_outbound_copy(e, t, src, compute);
+  if (rc) {
+    // kernels or the copy may already be queued on blocks that are about to be given back
     (void)hipStreamSynchronize(compute);
     (void)hipStreamSynchronize(e->copy);
     drop_device(e, t);
     e->hpool.free(t.host_off, t.host_bytes);
-    return hip_fail(err);
+    return rc;
   }
   t.state = kOutInFlight;
   *ticket = id;

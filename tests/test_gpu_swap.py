@@ -352,7 +352,7 @@ def test_reference_named_entry_points(torch_cuda):
     wantx = oracle.zfp_decode3(oracle.zfp_encode3(xf, 512), xf.shape, 512)
     assert np.array_equal(y.cpu().numpy().reshape(xf.shape).view(np.uint32), wantx.view(np.uint32))
     hip = C.CDLL("libamdhip64.so")                           # the default allocator is hipMalloc / hipFree
-    hip.hipFree.argtypes = [ctypes.c_void_p]
+    hip.hipFree.argtypes = [C.c_void_p]
     assert hip.hipFree(buf) == 0
 
     # ZVC launchers in the reference's order
