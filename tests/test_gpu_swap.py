@@ -607,3 +607,50 @@ def test_compat_allocator_field_hint_and_copy_stream(torch_cuda):
     eng.post(tk)
     eng.release(tk)
     eng.close()
+
+
+def test_two_threads_share_one_engine(torch_cuda):
+    """Engine calls are serialised by a mutex (the probe's pinned nnz slot and its
+    event are shared): two host threads, each on its own compute stream, swap
+    different tensors in and out through one engine and get their own data back."""
+    torch = torch_cuda
+    import threading
+
+    from cswap_amd import api, swap
+
+    eng = swap.SwapEngine(pinned_bytes=64 << 20, device_bytes=32 << 20)
+    errors = []
+
+    def worker(k):
+        try:
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                xs = [relu_tensor(torch, (64, 64, 8 + 8 * j), 0.3 + 0.3 * ((j + k) % 3), 50 * k + j) for j in range(4)]
+                zf = [api.cuda_decompress(api.cuda_compress(x, 512), x.shape, 512) for x in xs]
+                st.synchronize()
+                for it in range(60):
+                    j = (it + k) % 4
+                    pol = (swap.NONE, swap.SPARSE, swap.ZFP, swap.AUTO)[(it + 2 * k) % 4]
+                    tk = eng.pre(xs[j], pol)
+                    if it % 3 == 0:
+                        eng.post(tk)
+                    if it % 2:
+                        eng.prefetch(tk)
+                    out = torch.full_like(xs[j], -3.0)
+                    eng.swap_in(tk, out)
+                    st.synchronize()
+                    want = zf[j] if eng.info(tk).policy == swap.ZFP else xs[j]
+                    if not torch.equal(out.view(torch.int32), want.view(torch.int32)):
+                        errors.append((k, it, j, pol))
+                    eng.release(tk)
+        except Exception as exc:  # noqa: BLE001
+            errors.append((k, repr(exc)))
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads)
+    assert not errors, errors[:5]
+    eng.close()
