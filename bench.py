@@ -412,6 +412,7 @@ def extras(torch, api, dev, zvc_only=False):
         ex["planner"] = planner.bench_planner(dev)
         from cswap_amd import hooks
         ex["train_step"] = hooks.bench_training_step(dev)
+        ex["train_step_transformer"] = hooks.bench_transformer_step(dev)
     except ImportError:
         pass
     return ex

@@ -31,6 +31,15 @@ class _Handle:
         self.out = None      # the swapped-in tensor while further nodes still have to ask for it
 
 
+class _Ref:
+    """What autograd holds for one saved tensor: the swapped tensor and the shape
+    this node saw it in (a matmul saves a [b, h, s, s] tensor as [b*h, s, s])."""
+    __slots__ = ("handle", "shape")
+
+    def __init__(self, handle, shape):
+        self.handle, self.shape = handle, shape
+
+
 class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
     """Swap eligible saved activations (contiguous fp32 device tensors of at
     least ``min_bytes``) through ``engine``; everything else is saved as usual.
@@ -43,10 +52,11 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
     link, so the link does not idle between tensors.
 
     A tensor that several nodes save (the output of a ReLU is saved by the ReLU
-    and by the convolution or pooling that consumes it) is swapped once: while its
-    device copy is still held, packing the same storage, shape and version again
-    returns the same handle, and backward hands the one swapped-in tensor to
-    every node that asks for it.
+    and by the convolution or pooling that consumes it; attention probabilities by
+    the softmax and by the matmul, there reshaped) is swapped once: while its
+    device copy is still held, packing the same contiguous bytes (address, element
+    count, version) again refers to the same swap, and backward hands the one
+    swapped-in tensor, viewed in each node's shape, to every node that asks for it.
 
     Backward asks for the tensors in roughly the reverse of the order they were
     packed in, so each unpack also starts the inbound copy of the ``prefetch``
@@ -94,12 +104,12 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         if not eligible:
             self.stats["kept"] += 1
             return t
-        key = (t.data_ptr(), tuple(t.shape), t._version)
+        key = (t.data_ptr(), t.numel(), t._version)
         h = self._live.get(key)
         if h is not None:                # same tensor saved by another node: one swap serves both
             h.refs += 1
             self.stats["shared"] += 1
-            return h
+            return _Ref(h, tuple(t.shape))
         self._settle(self.depth - 1)
         self._drain()
         try:
@@ -120,7 +130,7 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         self._pending.append(h)
         self._live[key] = h
         self._order.append(h)
-        return h
+        return _Ref(h, tuple(t.shape))
 
     # -- backward side
     def _drain(self):
@@ -129,15 +139,16 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
             self._released.add(h.ticket)
         self._to_release.clear()
 
-    def _unpack(self, h):
-        if not isinstance(h, _Handle):
-            return h
+    def _unpack(self, ref):
+        if not isinstance(ref, _Ref):
+            return ref
+        h = ref.handle
         if h.out is not None:            # another node already had it swapped in
             out = h.out
             h.refs -= 1
             if h.refs <= 0:
                 h.out = None
-            return out
+            return out.view(ref.shape)
         self._settle()
         self._drain()
         out = torch.empty(h.shape, dtype=torch.float32, device="cuda")
@@ -148,7 +159,7 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         if h.refs > 0:
             h.out = out
         self._prefetch_before(h)
-        return out
+        return out.view(ref.shape)
 
     def _prefetch_before(self, h):
         """Start the inbound copies of the tensors packed just before ``h``."""
@@ -249,3 +260,87 @@ def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int =
                       "prefetched": st.get("prefetched", 0)}
     eng.close()
     return res
+
+
+def bench_transformer_step(dev, layers: int = 4, batch: int = 32, seq: int = 512, hidden: int = 768, heads: int = 12,
+                           min_bytes: int = 8 << 20) -> dict:
+    """Forward + backward of a BERT-base-shaped encoder stack (attention written
+    out, so the [batch, heads, seq, seq] probabilities are saved as in
+    configuration 5; GELU feed-forward of 4 x hidden) with and without swapping
+    through the saved-tensor hooks.  No ReLU anywhere: the selector has only ZFP
+    and raw to choose from."""
+    import math
+    import time
+
+    torch.manual_seed(0)
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.qkv = torch.nn.Linear(hidden, 3 * hidden)
+            self.proj = torch.nn.Linear(hidden, hidden)
+            self.ln1 = torch.nn.LayerNorm(hidden)
+            self.ln2 = torch.nn.LayerNorm(hidden)
+            self.fc1 = torch.nn.Linear(hidden, 4 * hidden)
+            self.fc2 = torch.nn.Linear(4 * hidden, hidden)
+
+        def forward(self, x):
+            b, s, h = x.shape
+            q, k, v = self.qkv(self.ln1(x)).view(b, s, 3, heads, h // heads).permute(2, 0, 3, 1, 4)
+            p = torch.softmax(q @ k.transpose(-1, -2) / math.sqrt(h // heads), dim=-1)
+            x = x + self.proj((p @ v).transpose(1, 2).reshape(b, s, h))
+            return x + self.fc2(torch.nn.functional.gelu(self.fc1(self.ln2(x))))
+
+    net = torch.nn.Sequential(*[Block() for _ in range(layers)]).to(dev)
+    x = torch.randn(batch, seq, hidden, device=dev)
+    params = list(net.parameters())
+
+    def step(ctx):
+        for p in params:
+            p.grad = None
+        if ctx is None:
+            loss = net(x).square().mean()
+        else:
+            with ctx:
+                loss = net(x).square().mean()
+        loss.backward()
+        if ctx is not None:
+            ctx.close()
+
+    def measure(make_ctx, reps=4):
+        for _ in range(2):
+            step(make_ctx())
+        for p in params:
+            p.grad = None
+        torch.cuda.synchronize()
+        base = torch.cuda.memory_allocated()
+        torch.cuda.reset_peak_memory_stats()
+        best, stats = None, None
+        for _ in range(reps):
+            ctx = make_ctx()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            step(ctx)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+            stats = ctx.stats if ctx is not None else None
+        return best * 1e3, (torch.cuda.max_memory_allocated() - base) / 1e6, stats
+
+    res = {"model": f"{layers} encoder blocks, batch {batch}, seq {seq}, hidden {hidden}, {heads} heads",
+           "min_bytes": min_bytes}
+    ms, mb, _ = measure(lambda: None)
+    res["no_swap"] = {"step_ms": round(ms, 2), "step_peak_MB": round(mb, 1)}
+    staging = 768 << 20
+    eng = swap.SwapEngine(pinned_bytes=12 << 30, device_bytes=staging)
+    eng.calibrate()
+    res["staging_pool_MB"] = round(staging / 1e6, 1)
+    for label, pol in (("raw_swap", swap.NONE), ("selector", swap.AUTO)):
+        ms, mb, st = measure(lambda: swap_saved_tensors(eng, policy=pol, min_bytes=min_bytes))
+        res[label] = {"step_ms": round(ms, 2), "step_peak_MB": round(mb, 1), "swapped_tensors": st["swapped"],
+                      "swapped_MB": round(st["bytes_in"] / 1e6, 1), "link_MB": round(st["bytes_out"] / 1e6, 1),
+                      "shared": st["shared"], "by_policy": dict(st.get("by_policy", {})),
+                      "kept_no_room": st.get("kept_no_room", 0)}
+    eng.close()
+    return res
+

@@ -103,6 +103,46 @@ def test_tensor_saved_by_two_nodes_is_swapped_once(torch_cuda):
     eng.close()
 
 
+def test_tensor_saved_under_two_shapes_is_swapped_once(torch_cuda):
+    """Attention probabilities are saved by the softmax as [b, h, s, s] and by the
+    matmul that consumes them as [b*h, s, s]: the same bytes, one swap, each node
+    gets its own shape back."""
+    torch = torch_cuda
+    from cswap_amd import swap
+    from cswap_amd.hooks import swap_saved_tensors
+
+    torch.manual_seed(0)
+    b, h, s, d = 4, 8, 128, 32
+    wq = torch.randn(h * d, h * d, device="cuda", requires_grad=True)
+    x = torch.randn(b, s, h * d, device="cuda")
+
+    def run(ctx):
+        wq.grad = None
+        def fwd():
+            q = (x @ wq).view(b, s, h, d).transpose(1, 2)
+            p = torch.softmax(q @ q.transpose(-1, -2) / d ** 0.5, dim=-1)
+            return (p @ q).square().mean()
+        if ctx is None:
+            loss = fwd()
+        else:
+            with ctx:
+                loss = fwd()
+        loss.backward()
+        if ctx is not None:
+            ctx.close()
+        return float(loss.detach()), wq.grad.clone()
+
+    l0, g0 = run(None)
+    l0b, g0b = run(None)
+    assert l0 == l0b and torch.equal(g0, g0b), "baseline is not deterministic"
+    eng = swap.SwapEngine(pinned_bytes=64 << 20, device_bytes=64 << 20)
+    ctx = swap_saved_tensors(eng, policy=swap.NONE, min_bytes=b * h * s * s * 4)    # only the probabilities are big enough
+    l1, g1 = run(ctx)
+    assert ctx.stats["swapped"] == 1 and ctx.stats["shared"] == 1, ctx.stats
+    assert l1 == l0 and torch.equal(g0, g1)
+    eng.close()
+
+
 def test_full_pools_leave_tensors_on_the_device(torch_cuda):
     """A pinned pool that holds only part of the activations: what does not fit
     stays on the device, the step still runs and gradients stay bit-identical."""
