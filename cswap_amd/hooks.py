@@ -58,6 +58,10 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
     count, version) again refers to the same swap, and backward hands the one
     swapped-in tensor, viewed in each node's shape, to every node that asks for it.
 
+    The last ``depth`` tensors of the forward pass are still on the device when it
+    ends (their copies are the ones in flight) and are the first that backward
+    asks for: they are handed back as they are, without a transfer.
+
     Backward asks for the tensors in roughly the reverse of the order they were
     packed in, so each unpack also starts the inbound copy of the ``prefetch``
     tensors packed just before the one it returns (one context serves one forward
@@ -82,11 +86,6 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         self._to_release = []      # handles whose swap-in has been launched
         self.stats = {"swapped": 0, "bytes_in": 0, "bytes_out": 0, "kept": 0, "shared": 0}
         super().__init__(self._pack, self._unpack)
-
-    def __exit__(self, *exc):
-        r = super().__exit__(*exc)
-        self._settle()     # forward is over: wait for the last outbound copies and let their device tensors go
-        return r
 
     # -- forward side
     def _settle(self, keep_in_flight: int = 0):
@@ -149,10 +148,16 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
             if h.refs <= 0:
                 h.out = None
             return out.view(ref.shape)
-        self._settle()
         self._drain()
-        out = torch.empty(h.shape, dtype=torch.float32, device="cuda")
-        self.engine.swap_in(h.ticket, out)
+        if h.keep is not None:           # still on the device: its outbound copy was one of the last in flight
+            out = h.keep.detach()
+            h.keep = None
+            self._pending.remove(h)
+            self._live.pop(h.key, None)
+            self.stats["resident"] = self.stats.get("resident", 0) + 1
+        else:
+            out = torch.empty(h.shape, dtype=torch.float32, device="cuda")
+            self.engine.swap_in(h.ticket, out)
         self._fetched.add(h.ticket)
         self._to_release.append(h)       # released once the next swap-in is issued (or at close)
         h.refs -= 1
@@ -170,7 +175,7 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         for g in reversed(self._order[:i]):
             if started >= self.prefetch:
                 break
-            if g.ticket in self._fetched:
+            if g.ticket in self._fetched or g.keep is not None:
                 continue
             try:
                 self.engine.prefetch(g.ticket)
