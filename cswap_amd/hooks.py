@@ -200,12 +200,48 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         self._order.clear()
 
 
+def _measure_step(step, params, make_ctx, reps=5):
+    """Best wall time of ``step(ctx)`` over ``reps`` runs after two warm-up runs, the
+    step's peak in torch's allocator above what is allocated before it, and the
+    hook statistics of the last run."""
+    import time
+
+    for _ in range(2):
+        step(make_ctx())
+    for p in params:
+        p.grad = None
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()     # weights, input and whatever else the process holds
+    torch.cuda.reset_peak_memory_stats()
+    best = None
+    stats = None
+    for _ in range(reps):
+        ctx = make_ctx()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        step(ctx)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+        stats = ctx.stats if ctx is not None else None
+    return best * 1e3, (torch.cuda.max_memory_allocated() - base) / 1e6, stats
+
+
+def _swap_rows(res, eng, step, params, min_bytes, reps):
+    for label, pol in (("raw_swap", swap.NONE), ("selector", swap.AUTO)):
+        ms, mb, st = _measure_step(step, params, lambda: swap_saved_tensors(eng, policy=pol, min_bytes=min_bytes), reps)
+        res[label] = {"step_ms": round(ms, 2), "step_peak_MB": round(mb, 1), "swapped_tensors": st["swapped"],
+                      "swapped_MB": round(st["bytes_in"] / 1e6, 1), "link_MB": round(st["bytes_out"] / 1e6, 1),
+                      "shared": st["shared"], "by_policy": dict(st.get("by_policy", {})),
+                      "prefetched": st.get("prefetched", 0), "resident": st.get("resident", 0),
+                      "kept_no_room": st.get("kept_no_room", 0)}
+
+
 def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int = 8 << 20) -> dict:
     """Forward + backward of a VGG-16 (conv/BN/ReLU x13, 5 pools, linear head) on
     random data with and without activation swapping through the saved-tensor
     hooks: step time and peak device memory of the step (torch's allocator, above
     what is allocated before the step).  Stock autograd, nothing patched."""
-    import time
 
     from .planner import _vgg_modules
 
@@ -228,41 +264,14 @@ def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int =
             ctx.close()
         return loss
 
-    def measure(make_ctx, reps=5):
-        for _ in range(2):
-            step(make_ctx())
-        for p in params:
-            p.grad = None
-        torch.cuda.synchronize()
-        base = torch.cuda.memory_allocated()     # weights, input and whatever else the process holds
-        torch.cuda.reset_peak_memory_stats()
-        best = None
-        stats = None
-        for _ in range(reps):
-            ctx = make_ctx()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            step(ctx)
-            torch.cuda.synchronize()
-            dt = time.perf_counter() - t0
-            best = dt if best is None else min(best, dt)
-            stats = ctx.stats if ctx is not None else None
-        return best * 1e3, (torch.cuda.max_memory_allocated() - base) / 1e6, stats
-
     res = {"model": f"VGG-16 BN, batch {batch}, 3x{image}x{image}", "min_bytes": min_bytes}
-    base_ms, base_mb, _ = measure(lambda: None)
+    base_ms, base_mb, _ = _measure_step(step, params, lambda: None)
     res["no_swap"] = {"step_ms": round(base_ms, 2), "step_peak_MB": round(base_mb, 1)}
     staging = 192 << 20
     eng = swap.SwapEngine(pinned_bytes=4 << 30, device_bytes=staging)
     eng.calibrate()
     res["staging_pool_MB"] = round(staging / 1e6, 1)    # device memory the engine holds besides torch's allocator
-    for label, pol in (("raw_swap", swap.NONE), ("selector", swap.AUTO)):
-        ms, mb, st = measure(lambda: swap_saved_tensors(eng, policy=pol, min_bytes=min_bytes, prefetch=2, depth=2))
-        res[label] = {"step_ms": round(ms, 2), "step_peak_MB": round(mb, 1),
-                      "swapped_tensors": st["swapped"], "swapped_MB": round(st["bytes_in"] / 1e6, 1),
-                      "link_MB": round(st["bytes_out"] / 1e6, 1), "shared": st["shared"],
-                      "by_policy": dict(st.get("by_policy", {})),
-                      "prefetched": st.get("prefetched", 0)}
+    _swap_rows(res, eng, step, params, min_bytes, 5)
     eng.close()
     return res
 
@@ -275,7 +284,6 @@ def bench_transformer_step(dev, layers: int = 4, batch: int = 32, seq: int = 512
     through the saved-tensor hooks.  No ReLU anywhere: the selector has only ZFP
     and raw to choose from."""
     import math
-    import time
 
     torch.manual_seed(0)
 
@@ -312,40 +320,14 @@ def bench_transformer_step(dev, layers: int = 4, batch: int = 32, seq: int = 512
         if ctx is not None:
             ctx.close()
 
-    def measure(make_ctx, reps=4):
-        for _ in range(2):
-            step(make_ctx())
-        for p in params:
-            p.grad = None
-        torch.cuda.synchronize()
-        base = torch.cuda.memory_allocated()
-        torch.cuda.reset_peak_memory_stats()
-        best, stats = None, None
-        for _ in range(reps):
-            ctx = make_ctx()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            step(ctx)
-            torch.cuda.synchronize()
-            dt = time.perf_counter() - t0
-            best = dt if best is None else min(best, dt)
-            stats = ctx.stats if ctx is not None else None
-        return best * 1e3, (torch.cuda.max_memory_allocated() - base) / 1e6, stats
-
     res = {"model": f"{layers} encoder blocks, batch {batch}, seq {seq}, hidden {hidden}, {heads} heads",
            "min_bytes": min_bytes}
-    ms, mb, _ = measure(lambda: None)
+    ms, mb, _ = _measure_step(step, params, lambda: None, 4)
     res["no_swap"] = {"step_ms": round(ms, 2), "step_peak_MB": round(mb, 1)}
     staging = 768 << 20
     eng = swap.SwapEngine(pinned_bytes=12 << 30, device_bytes=staging)
     eng.calibrate()
     res["staging_pool_MB"] = round(staging / 1e6, 1)
-    for label, pol in (("raw_swap", swap.NONE), ("selector", swap.AUTO)):
-        ms, mb, st = measure(lambda: swap_saved_tensors(eng, policy=pol, min_bytes=min_bytes))
-        res[label] = {"step_ms": round(ms, 2), "step_peak_MB": round(mb, 1), "swapped_tensors": st["swapped"],
-                      "swapped_MB": round(st["bytes_in"] / 1e6, 1), "link_MB": round(st["bytes_out"] / 1e6, 1),
-                      "shared": st["shared"], "by_policy": dict(st.get("by_policy", {})),
-                      "kept_no_room": st.get("kept_no_room", 0)}
+    _swap_rows(res, eng, step, params, min_bytes, 4)
     eng.close()
     return res
-
