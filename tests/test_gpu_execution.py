@@ -160,3 +160,29 @@ def test_planned_iteration_restores_every_swapped_tensor():
     assert sorted(seen) == [i for i, p in enumerate(pol) if p]
     eng.close()
     pm.close()
+
+
+def test_cpp_driver_with_policy_maker_and_execution():
+    """tests/cpp_schedule_walk.cpp: a driver in the style of the reference's model
+    files, written against the two header-only mirrors and the C ABI only (no
+    Python, no torch): calibrate, plan half of the activation bytes with
+    cswap::PolicyMaker, walk forward with cswap::Execution::pre/post, walk backward
+    with prefetch/fetch, and compare every tensor that comes back byte for byte."""
+    import os
+    import subprocess
+    import tempfile
+
+    from conftest import ROOT
+
+    src = os.path.join(ROOT, "tests", "cpp_schedule_walk.cpp")
+    lib = os.path.join(ROOT, "cswap_amd", "libcswap_hip.so")
+    with tempfile.TemporaryDirectory() as d:
+        exe = os.path.join(d, "walk")
+        subprocess.check_call(["g++", "-std=c++17", "-O1", "-Wall", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROOT, "include"),
+                               "-I/opt/rocm/include", src, lib, "-Wl,-rpath," + os.path.dirname(lib),
+                               "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib", "-lamdhip64", "-o", exe])
+        out = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    print(out.stdout, out.stderr, flush=True)
+    assert out.returncode == 0, out.stdout
+    tag, swapped, link = out.stdout.split()[-3:]
+    assert tag == "OK" and int(swapped) >= 3 and int(link) > 0
