@@ -165,7 +165,7 @@ def test_planned_iteration_restores_every_swapped_tensor():
 def test_cpp_driver_with_policy_maker_and_execution():
     """tests/cpp_schedule_walk.cpp: a driver in the style of the reference's model
     files, written against the two header-only mirrors and the C ABI only (no
-    Python, no torch): calibrate, plan half of the activation bytes with
+    Python, no torch): calibrate, plan most of the activation bytes with
     cswap::PolicyMaker, walk forward with cswap::Execution::pre/post, walk backward
     with prefetch/fetch, and compare every tensor that comes back byte for byte."""
     import os
@@ -186,3 +186,5 @@ def test_cpp_driver_with_policy_maker_and_execution():
     assert out.returncode == 0, out.stdout
     tag, swapped, link = out.stdout.split()[-3:]
     assert tag == "OK" and int(swapped) >= 3 and int(link) > 0
+    policy = [int(v) for v in out.stdout.split("policy:")[1].split("OK")[0].split()]
+    assert 3 in policy and 2 in policy                       # ZVC for the ReLU-like tensors, raw for the (de-ZFP-ed) dense ones
