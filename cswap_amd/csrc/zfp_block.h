@@ -461,19 +461,31 @@ struct BlockEncoder {
     uint64_t rest = n < 64 ? x >> n : 0;
     put(n < 64 ? x ^ (rest << n) : x, n);
     if (n < SIZE) {
-      while (rest != 0 && n < SIZE && pos < limit) {
-        unsigned t = (unsigned)ctz64(rest);  // zeros before the next one-bit
-        unsigned nt = n + t;
-        bool more = nt < SIZE - 1;           // a one-bit at the last position is implied, not written
-        unsigned q = pos + t + 1;
+      bool more = true;
+      while (rest != 0 && more && pos < limit) {
+        unsigned t1 = (unsigned)ctz64(rest) + 1;  // zeros before the next one-bit, and that bit
+        unsigned q = pos + t1;
+        n += t1;
+        more = n < SIZE;                     // a one-bit at the last position is implied, not written
         set_bit(pos, true);                  // positive group test
-        set_bit(q, more);                    // t zeros, then the one-bit
+        set_bit(q, more);                    // the zeros, then the one-bit
         pos = q + (more ? 1u : 0u);
-        n = nt + 1;
-        rest = (rest >> t) >> 1;
+        rest >>= t1 & 63;                    // t1 = 64 only for the last coefficient: more is false, rest is not used again
       }
       if (rest == 0 && n < SIZE && pos < limit) pos++;  // negative group test: a zero bit
     }
+  }
+
+  // One of the leading planes.  While no block of the wavefront has found a
+  // significant coefficient and the plane is empty in all of them, the plane
+  // costs every block one zero bit and nothing else.
+  CSWAP_HD void leading_plane(uint64_t x)
+  {
+    if (!CSWAP_ANY(x != 0 || n != 0)) {
+      if (active()) pos++;
+      return;
+    }
+    plane(x);
   }
 };
 
@@ -508,7 +520,9 @@ CSWAP_HD void encode_planes32(uint32_t (&lo)[32], uint32_t (&hi)[32], Enc& enc, 
   tr_stage<1, 16, 32, kNotOut>(lo);
   tr_stage<1, 16, 32, kNotOut>(hi);
 #pragma unroll
-  for (int k = 31; k >= 16; k--) enc.plane(((uint64_t)hi[k] << 32) | lo[k]);
+  for (int k = 31; k >= 28; k--) enc.leading_plane(((uint64_t)hi[k] << 32) | lo[k]);
+#pragma unroll
+  for (int k = 27; k >= 16; k--) enc.plane(((uint64_t)hi[k] << 32) | lo[k]);
   if (CSWAP_ANY(enc.active())) {
     tr_half<0, kNotOut>(lo);
     tr_half<0, kNotOut>(hi);
