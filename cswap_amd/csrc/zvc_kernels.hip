@@ -35,6 +35,14 @@ __device__ __forceinline__ int wave_sum(int v)
   return v;
 }
 
+// 16-byte store with the nontemporal hint, for output that is written once in whole lines
+typedef float stream_f4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void st_stream4(float4* p, float4 v)
+{
+  stream_f4 t = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(t, reinterpret_cast<stream_f4*>(p));
+}
+
 struct Geometry {
   int n;        // elements
   int E;        // elements per chunk
@@ -232,7 +240,10 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand_kernel(
   }
 }
 
-// Same expansion with one lane = four consecutive elements and 16-byte stores:
+// Same expansion with one lane = four consecutive elements and 16-byte stores
+// (with the nontemporal hint: 256 MiB expand in 63 instead of 88 us, 32 MiB in
+// 10.9 instead of 12.3 us, a reader of the result right after it no slower;
+// the same hint on the loads of the counting and compacting passes gains nothing):
 // the per-element form above issues one 4-byte store per lane and is bound by
 // that instruction stream, not by bytes.  A row is 256 elements = 8 mask words;
 // lane l keeps mask word 64*(row/8) + l of the chunk, together with the number
@@ -297,7 +308,7 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand4_kernel(
     for (int j = 0; j < kRowsInFlight; j++) {
       const int k = (r0 + j) * 256 + 4 * (int)lane;
       if (k + 4 <= len) {
-        *reinterpret_cast<float4*>(q + k) = x[j];
+        st_stream4(reinterpret_cast<float4*>(q + k), x[j]);
       } else {  // ragged end of the last chunk
         if (k < len) q[k] = x[j].x;
         if (k + 1 < len) q[k + 1] = x[j].y;

@@ -40,7 +40,7 @@ def test_zfp_fp32_kernels_fit_five_waves_without_scratch():
         if m and name:
             kernels[name][m.group(1).split()[0]] = int(m.group(2))
     f32 = {k: v for k, v in kernels.items() if "zfp_encode3_f32_kernel" in k or "zfp_decode3_f32_kernel" in k}
-    assert len(f32) == 8, sorted(kernels)
+    assert len(f32) == 10, sorted(kernels)     # 4 decoders, 4 encoders, 2 encoders that load with the nontemporal hint
     for k, v in f32.items():
         assert v["ScratchSize"] == 0, (k, v)
         assert v["VGPRs"] <= 96 and v["Occupancy"] >= 5, (k, v)
