@@ -472,7 +472,9 @@ struct BlockEncoder {
         pos = q + (more ? 1u : 0u);
         rest >>= t1 & 63;                    // t1 = 64 only for the last coefficient: more is false, rest is not used again
       }
-      if (rest == 0 && n < SIZE && pos < limit) pos++;  // negative group test: a zero bit
+      // negative group test: a zero bit.  Without the guard a position past the end is
+      // harmless (nothing is written there and the next plane sees the block as full)
+      if (rest == 0 && n < SIZE && (!GUARD || pos < limit)) pos++;
     }
   }
 

@@ -29,6 +29,12 @@ struct Field3 {
   Div31 by_mx, by_my;      // block index -> block coordinates without a hardware divide
 };
 
+// Fields of at least this many bytes are loaded with the nontemporal hint (make_field)
+#ifndef CSWAP_READ_ONCE_BYTES
+#define CSWAP_READ_ONCE_BYTES (128ull << 20)
+#endif
+constexpr unsigned long long kReadOnceBytes = CSWAP_READ_ONCE_BYTES;
+
 // 16 bytes of the field as the compiler's own vector type (what the nontemporal builtins take)
 typedef float stream_f4 __attribute__((ext_vector_type(4)));
 
@@ -641,12 +647,13 @@ static int make_field(Field3& fd, const void* base, const void* stream, size_t n
   // instead of 117 us, and the kernel that runs next no longer waits behind those lines
   // draining from the memory-side cache (33.6 MB: decode 14.5 instead of 17.6 us, and a
   // reader of the result right after it is no slower).  The encoder loads with the hint
-  // only when the field is larger than that cache (256 MB): a smaller tensor may still be
-  // cached from the kernel that produced it, and hinted loads of cached lines are slower
-  // (16.8 MB right after its producer: 25.0 against 23.1 us).  The stream keeps the
+  // only when the field is large against that cache (256 MB): a smaller tensor is still
+  // cached from the kernel that produced it, and hinted loads of cached lines are slower.
+  // Producer kernel + encoder, hinted / plain loads: 402.7 MB 205 / 220 us, 201.3 MB
+  // 95 / 109 us, 100.7 MB 43.6 / 43.2 us, 50.3 MB 26.1 / 24.5 us.  The stream keeps the
   // default policy: a lane's piece of it is not a whole line, and the decoder or the copy
   // engine reads it next.
-  fd.read_once = (unsigned long long)nx * ny * nz * elem >= (256ull << 20);
+  fd.read_once = (unsigned long long)nx * ny * nz * elem >= kReadOnceBytes;
   return CSWAP_OK;
 }
 
