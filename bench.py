@@ -126,7 +126,7 @@ def main():
         torch.cuda.synchronize()
     # the events of the timed region exist before the GPU is brought to its steady
     # clocks, so that nothing but a synchronize separates the warm-up from the timed steps
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(args.steps + 1)]
     settle(torch, step, CLOCK_SETTLE_S)
     for _ in range(args.warmup):
         step()
@@ -134,17 +134,17 @@ def main():
     # ---- timed region: exactly K steps, per-kernel HIP events inside it
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for k in range(args.steps):
+    for k in range(args.steps):          # two events per step: the end of a decompress is the start of the next step
         evs[k][0].record()
         api.cuda_compress(x, maxbits, out=stream)
         evs[k][1].record()
         api.cuda_decompress(stream, x.shape, maxbits, out=out)
-        evs[k][2].record()
+    evs[args.steps][0].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    enc_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
-    dec_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps
+    enc_ms = sum(evs[k][0].elapsed_time(evs[k][1]) for k in range(args.steps)) / args.steps
+    dec_ms = sum(evs[k][1].elapsed_time(evs[k + 1][0]) for k in range(args.steps)) / args.steps
     value = 4.0 * n / (ms_per_step * 1e-3) / 1e9
 
     bytes_per_value = 4.0 + rate / 8.0          # read 4 B, write rate/8 B (or the reverse)
