@@ -95,6 +95,7 @@ _SIGNATURES = {
     "cswap_zvc_active_chunks": (i32, [i32, i32]),
     "cswap_zvc_mask_bytes": (sz, [i32, i32]),
     "cswap_zvc_pick_process": (i32, [sz]),
+    "cswap_zvc_set_staged_compact_bytes": (sz, [sz]),
     "cswap_zvc_count": (i32, [vp, i32, i32, vp, vp]),
     "cswap_zvc_scan": (i32, [vp, i32, vp, vp]),
     "cswap_zvc_compact": (i32, [vp, i32, i32, vp, vp, vp, vp]),

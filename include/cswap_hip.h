@@ -124,6 +124,14 @@ size_t cswap_zvc_mask_bytes(int n, int process);    /* W*process*4, Execution.h:
  * always passes 512*32): about 1024 elements per chunk, a power of two in
  * [1024, 16384].  Both directions must use the same value. */
 int    cswap_zvc_pick_process(size_t n);
+/* No counterpart in the reference: cswap_zvc_compact has two forms, one that
+ * stores each 64-element row's non-zeros straight from the lanes that hold them
+ * and one that stages them in LDS and writes whole aligned 1 KB runs with the
+ * nontemporal hint; the second is faster for tensors larger than the GPU's
+ * memory-side cache and runs for tensors of at least this many bytes (default
+ * 192 MiB; 0 = always, SIZE_MAX = never).  Same output either way.  Returns the
+ * previous value.  Process-wide; not meant to be changed while kernels are being launched. */
+size_t cswap_zvc_set_staged_compact_bytes(size_t bytes);
 
 /* Replaces PreGPUcompression (zfp/compression.cu:134-165, launcher :334-341):
  * d_count[i] = number of elements != 0 in chunk i, for the active chunks. */

@@ -15,6 +15,22 @@ def torch_cuda():
     return torch
 
 
+@pytest.fixture(params=["by_size", "staged"])
+def compact_form(request):
+    """Both forms of cswap_zvc_compact: the one its size rule picks (row-wise stores at
+    these sizes) and the LDS-staged one, forced for inputs of any size."""
+    from cswap_amd._lib import lib
+
+    if request.param == "by_size":
+        yield request.param
+        return
+    before = lib().cswap_zvc_set_staged_compact_bytes(0)
+    try:
+        yield request.param
+    finally:
+        lib().cswap_zvc_set_staged_compact_bytes(before)
+
+
 def run_gpu(torch, x, process=P, fused=False):
     from cswap_amd import api
 
@@ -44,7 +60,7 @@ def check_against_oracle(x, got, process=P):
 
 
 @pytest.mark.parametrize("pct", [30, 50, 70, 90])
-def test_config2_sparsity_sweep(torch_cuda, pct):
+def test_config2_sparsity_sweep(torch_cuda, compact_form, pct):
     from cswap_amd.workloads import config2_tensor
 
     x = config2_tensor(pct).reshape(-1)
@@ -54,7 +70,7 @@ def test_config2_sparsity_sweep(torch_cuda, pct):
 
 
 @pytest.mark.parametrize("n", [1, 31, 33, 64, 1000, P - 1, P, P + 1, 1_000_003, P * 62 + 17, P * 64, P * 96 + 5])
-def test_ragged_sizes(torch_cuda, n):
+def test_ragged_sizes(torch_cuda, compact_form, n):
     rng = np.random.default_rng(n)
     x = (rng.standard_normal(n) * (rng.random(n) < 0.4)).astype(np.float32)
     print("n", n, flush=True)
@@ -62,7 +78,7 @@ def test_ragged_sizes(torch_cuda, n):
 
 
 @pytest.mark.parametrize("process", [1, 7, 64, 4096])
-def test_other_chunk_counts(torch_cuda, process):
+def test_other_chunk_counts(torch_cuda, compact_form, process):
     rng = np.random.default_rng(process)
     x = np.maximum(rng.standard_normal(300_001), 0).astype(np.float32)
     check_against_oracle(x, run_gpu(torch_cuda, x, process), process)
@@ -138,7 +154,7 @@ def test_fused_repeated_calls_share_a_workspace(torch_cuda):
         assert int(ws.view(torch.int32)[1].item()) == 0      # no bounded wait ran out
 
 
-def test_special_values_and_extremes(torch_cuda):
+def test_special_values_and_extremes(torch_cuda, compact_form):
     n = P * 64
     x = np.zeros(n, dtype=np.float32)
     x[[3, 10, 11, 12, 13, 70]] = [-0.0, np.nan, np.inf, -np.inf, 1e-45, -2.5]
@@ -206,7 +222,7 @@ def test_full_size_round_trip(torch_cuda):
     assert torch.equal(values[:k], t[t != 0])
 
 
-def test_random_sizes_chunk_counts_and_sparsities(torch_cuda):
+def test_random_sizes_chunk_counts_and_sparsities(torch_cuda, compact_form):
     """120 seeded cases: n from 1 to 400 000, chunk counts from 1 to 65 536 (more
     chunks than elements included), zero fractions from 0 to 1 with special values
     mixed in, plain and single-pass compaction, and a destination that is not
@@ -241,3 +257,34 @@ def test_random_sizes_chunk_counts_and_sparsities(torch_cuda):
         want = np.where(x != 0, x, np.float32(0))
         assert np.array_equal(b[shift:shift + n].view(np.uint32), want.view(np.uint32)), tag
         assert (b[:shift] == -1).all() and (b[shift + n:] == -1).all(), tag
+
+
+@pytest.mark.parametrize("nnz_per_chunk", [0, 1, 3, 255, 256, 257, 511, 512, 513, 1000])
+def test_staged_compaction_ring_boundaries(torch_cuda, nnz_per_chunk):
+    """The staged form writes a wave's ring out 256 values at a time: chunks whose
+    counts sit on either side of one and two ring halves, so that every alignment of
+    a chunk's first value (begin % 4) meets every fill level at the end of a chunk."""
+    from cswap_amd._lib import lib
+
+    E, chunks = 1024, 48
+    rng = np.random.default_rng(nnz_per_chunk)
+    x = np.zeros(E * chunks, dtype=np.float32)
+    for c in range(chunks):
+        k = min(E, max(0, nnz_per_chunk + (c % 5) - 2)) if nnz_per_chunk else 0
+        idx = rng.choice(E, size=k, replace=False)
+        x[c * E + idx] = rng.standard_normal(k).astype(np.float32) + 3.0
+    before = lib().cswap_zvc_set_staged_compact_bytes(0)
+    try:
+        got = run_gpu(torch_cuda, x, chunks)
+    finally:
+        lib().cswap_zvc_set_staged_compact_bytes(before)
+    check_against_oracle(x, got, chunks)
+
+
+def test_staged_threshold_is_reported_and_restored(torch_cuda):
+    from cswap_amd._lib import lib
+
+    L = lib()
+    default = L.cswap_zvc_set_staged_compact_bytes(12345)
+    assert default == 192 << 20
+    assert L.cswap_zvc_set_staged_compact_bytes(default) == 12345
