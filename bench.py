@@ -16,7 +16,8 @@ return to its steady clocks, and a training loop never leaves it idle.
 
 The single JSON line also carries
   roofline      HBM-roofline figures of the dominant (slower) ZFP kernel, from
-                HIP-event timing of that kernel inside the timed region
+                HIP-event timing of that kernel inside the timed region (events
+                around both kernels of every tenth step)
   cpu_baseline  the CPU checker (a port of the reference algorithm; and the stock
                 zfp 0.5.5 library where the machine has it) timed on a
                 bounded sample of the same tensor on this host
