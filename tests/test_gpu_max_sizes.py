@@ -153,6 +153,35 @@ def test_zfp_f64_field_beyond_2_32_elements(torch_cuda):
     _free(torch)
 
 
+def test_zfp_i32_field_loaded_with_the_nontemporal_hint(torch_cuda):
+    """An int32 field of 160 MiB: above the size from which the encoder loads its
+    rows with the nontemporal hint (a separate instantiation per element kind).
+    First, middle and last slab against the checker, every block against pieces."""
+    torch = torch_cuda
+    import oracle
+    from cswap_amd import api
+
+    nz, ny, nx = 640, 256, 256
+    g = torch.Generator(device="cuda"); g.manual_seed(8)
+    x = torch.randint(-(1 << 28), 1 << 28, (nz, ny, nx), generator=g, device="cuda", dtype=torch.int32)
+    x[300:304].zero_()
+    s = api.cuda_compress(x, 512)
+    d = api.cuda_decompress(s, x.shape, 512, dtype=torch.int32)
+    torch.cuda.synchronize()
+    layer = (nx // 4) * (ny // 4) * 64
+    for z in (0, 296, 632):
+        slab = x[z:z + 8].cpu().numpy()
+        got = s[(z // 4) * layer:(z // 4 + 2) * layer].cpu().numpy().view(np.uint64)
+        want = oracle.zfp_encode_i32(slab, 512)
+        assert np.array_equal(got, want[:got.size]), z
+        back = d[z:z + 8].cpu().numpy()
+        assert np.array_equal(back, oracle.zfp_decode_i32(got, slab.shape, 512)), z
+    assert not d[300:304].any().item()
+    _pieces_agree(torch, x, s, d, 512, 128, layer)       # pieces of 32 MiB: plain loads
+    del x, s, d
+    _free(torch)
+
+
 def test_zfp_rejects_fields_beyond_its_block_index_range(torch_cuda):
     """2^31 blocks or more, or an extent above 2^31 - 1, are refused before any launch."""
     torch = torch_cuda
