@@ -69,15 +69,27 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
     it and its host copy is released right after): their transfer then runs on
     the copy stream under the backward kernels of the current layer.  (VGG-16 at
     batch 128 on one MI355X: looking two tensors ahead keeps the link busy through
-    layers whose backward is short; deeper look-ahead gains nothing more.)"""
+    layers whose backward is short; deeper look-ahead gains nothing more.)
+
+    ``memo``: a dict the caller keeps from one training iteration to the next.  With
+    ``policy=AUTO`` the selector probes every tensor (a counting pass and a host
+    round trip, CSWAP+/Execution.h:92 has the same one); the k-th swapped tensor of
+    an iteration is the same activation every time, so its decision is remembered
+    under (k, element count).  A remembered "ZFP" or "raw" is passed to the engine
+    as an explicit policy and costs no probe; "ZVC" needs the non-zero count anyway
+    and is probed as before.  After ``recheck`` uses an entry is probed again, so a
+    layer whose sparsity drifts is noticed."""
 
     def __init__(self, engine: "swap.SwapEngine", policy: int = swap.AUTO, min_bytes: int = 1 << 20,
-                 prefetch: int = 2, depth: int = 2):
+                 prefetch: int = 2, depth: int = 2, memo: dict | None = None, recheck: int = 16):
         self.engine = engine
         self.policy = policy
         self.min_bytes = min_bytes
         self.prefetch = prefetch
         self.depth = max(1, depth)
+        self.memo = memo
+        self.recheck = max(1, recheck)
+        self._position = 0         # swaps attempted so far in this context
         self._order = []           # handles in pack order
         self._fetched = set()      # tickets already swapped in or being prefetched
         self._released = set()
@@ -111,14 +123,30 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
             return _Ref(h, tuple(t.shape))
         self._settle(self.depth - 1)
         self._drain()
+        policy, slot = self.policy, (self._position, t.numel())
+        self._position += 1
+        if self.memo is not None and self.policy == swap.AUTO:
+            known = self.memo.get(slot)
+            if known is not None and known[0] in (swap.ZFP, swap.NONE) and known[1] < self.recheck:
+                policy = known[0]
+                self.memo[slot] = (known[0], known[1] + 1)
+                self.stats["memo_hits"] = self.stats.get("memo_hits", 0) + 1
         try:
-            ticket = self.engine.pre(t.detach(), self.policy)
+            try:
+                ticket = self.engine.pre(t.detach(), policy)
+            except CswapError as err:
+                if err.code != E_NOMEM or policy == self.policy:
+                    raise
+                policy = self.policy     # no staging room for the remembered codec: let the selector degrade it
+                ticket = self.engine.pre(t.detach(), policy)
         except CswapError as err:
             if err.code != E_NOMEM:
                 raise
             self.stats["kept_no_room"] = self.stats.get("kept_no_room", 0) + 1
             return t                     # pinned pool, staging pool or tickets exhausted: the tensor stays on the device
         info = self.engine.info(ticket)
+        if self.memo is not None and policy == swap.AUTO:
+            self.memo[slot] = (info.policy, 0)
         self.stats["swapped"] += 1
         self.stats["bytes_in"] += info.bytes_in
         self.stats["bytes_out"] += info.bytes_out
@@ -228,13 +256,16 @@ def _measure_step(step, params, make_ctx, reps=5):
 
 
 def _swap_rows(res, eng, step, params, min_bytes, reps):
-    for label, pol in (("raw_swap", swap.NONE), ("selector", swap.AUTO)):
-        ms, mb, st = _measure_step(step, params, lambda: swap_saved_tensors(eng, policy=pol, min_bytes=min_bytes), reps)
+    memo = {}        # the selector's decisions, kept across the iterations of the last row
+    for label, pol, kw in (("raw_swap", swap.NONE, {}), ("selector", swap.AUTO, {}),
+                           ("selector_remembered", swap.AUTO, {"memo": memo})):
+        ms, mb, st = _measure_step(step, params,
+                                   lambda: swap_saved_tensors(eng, policy=pol, min_bytes=min_bytes, **kw), reps)
         res[label] = {"step_ms": round(ms, 2), "step_peak_MB": round(mb, 1), "swapped_tensors": st["swapped"],
                       "swapped_MB": round(st["bytes_in"] / 1e6, 1), "link_MB": round(st["bytes_out"] / 1e6, 1),
                       "shared": st["shared"], "by_policy": dict(st.get("by_policy", {})),
                       "prefetched": st.get("prefetched", 0), "resident": st.get("resident", 0),
-                      "kept_no_room": st.get("kept_no_room", 0)}
+                      "kept_no_room": st.get("kept_no_room", 0), "memo_hits": st.get("memo_hits", 0)}
 
 
 def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int = 8 << 20) -> dict:

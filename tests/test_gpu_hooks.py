@@ -205,3 +205,40 @@ def test_zfp_policy_keeps_gradients_close(torch_cuda):
     for a, b in zip(g0, g1):
         assert float((a - b).norm()) <= 2e-2 * float(a.norm()) + 1e-8
     eng.close()
+
+
+def test_decisions_are_remembered_across_iterations(torch_cuda):
+    """memo: the selector's choice for the k-th swapped tensor is kept from one
+    iteration to the next; remembered ZFP / raw choices skip the probe, ZVC is
+    probed as before, and after `recheck` uses an entry is probed again."""
+    torch = torch_cuda
+    from cswap_amd import swap
+    from cswap_amd.hooks import swap_saved_tensors
+
+    net = make_mlp(torch)
+    x = torch.randn(2048, 512, device="cuda")
+    eng = swap.SwapEngine(pinned_bytes=256 << 20, device_bytes=256 << 20)
+    eng.calibrate()
+    memo = {}
+    runs = []
+    for it in range(5):
+        ctx = swap_saved_tensors(eng, policy=swap.AUTO, min_bytes=1 << 16, memo=memo, recheck=2)
+        loss, g = grads(torch, net, x, ctx)
+        runs.append((loss, g, dict(ctx.stats)))
+    first = runs[0][2]
+    assert first.get("memo_hits", 0) == 0 and first["swapped"] >= 3
+    dense = sum(v for k, v in first["by_policy"].items() if k in ("zfp", "raw"))
+    assert dense >= 1, first                         # the Linear inputs / GELU input are dense
+    # iterations 2 and 3 use the remembered decisions, iteration 4 probes again (recheck = 2), 5 remembers again
+    assert [r[2].get("memo_hits", 0) for r in runs] == [0, dense, dense, 0, dense], [r[2] for r in runs]
+    for loss, g, st in runs[1:]:
+        assert st["by_policy"] == first["by_policy"] and st["swapped"] == first["swapped"]
+        assert loss == runs[0][0]
+        for a, b in zip(runs[0][1], g):
+            assert torch.equal(a, b)                 # same codecs, same inputs: the same gradients
+    # a position whose size changed is not trusted
+    memo2 = {k: v for k, v in memo.items()}
+    ctx = swap_saved_tensors(eng, policy=swap.AUTO, min_bytes=1 << 16, memo=memo2)
+    grads(torch, net, torch.randn(1024, 512, device="cuda"), ctx)
+    assert ctx.stats.get("memo_hits", 0) == 0
+    eng.close()
