@@ -26,6 +26,7 @@ struct Field3 {
                            //    planes inside the volume, and any 64 consecutive blocks lie within 4 GiB
   int stream16;            // 1: the stream pointer is 16-byte aligned
   int read_once;           // 1: the encoder should load the field with the nontemporal hint (see make_field)
+  int once64;              // 1: the decoder of 64-bit elements should store its rows with the hint (see make_field)
   Div31 by_mx, by_my;      // block index -> block coordinates without a hardware divide
 };
 
@@ -37,6 +38,7 @@ constexpr unsigned long long kReadOnceBytes = CSWAP_READ_ONCE_BYTES;
 
 // 16 bytes of the field as the compiler's own vector type (what the nontemporal builtins take)
 typedef float stream_f4 __attribute__((ext_vector_type(4)));
+typedef unsigned long long stream_u2 __attribute__((ext_vector_type(2)));
 
 // ------------------------------------------------------------- LDS adapter
 // The bit region the block codec ORs into / reads from is LDS, addressed in
@@ -358,6 +360,7 @@ __device__ __forceinline__ void load_block_w64(const uint64_t* __restrict__ in, 
   }
 }
 
+template <bool ONCE>
 __device__ __forceinline__ void store_block_w64(uint64_t* __restrict__ out, const Field3& fd, uint32_t b,
                                                 const uint64_t (&q)[64])
 {
@@ -370,9 +373,16 @@ __device__ __forceinline__ void store_block_w64(uint64_t* __restrict__ out, cons
     for (int z = 0; z < 4; z++)
 #pragma unroll
       for (int y = 0; y < 4; y++) {
-        ulonglong2* r = reinterpret_cast<ulonglong2*>(p + y * fd.sy + z * fd.sz);
-        r[0] = make_ulonglong2(q[16 * z + 4 * y + 0], q[16 * z + 4 * y + 1]);
-        r[1] = make_ulonglong2(q[16 * z + 4 * y + 2], q[16 * z + 4 * y + 3]);
+        stream_u2* r = reinterpret_cast<stream_u2*>(p + y * fd.sy + z * fd.sz);
+        const stream_u2 a = {q[16 * z + 4 * y + 0], q[16 * z + 4 * y + 1]};
+        const stream_u2 c = {q[16 * z + 4 * y + 2], q[16 * z + 4 * y + 3]};
+        if (ONCE) {
+          __builtin_nontemporal_store(a, r);
+          __builtin_nontemporal_store(c, r + 1);
+        } else {
+          r[0] = a;
+          r[1] = c;
+        }
       }
   } else {
 #pragma unroll
@@ -407,7 +417,8 @@ __global__ __launch_bounds__(64) void zfp_encode3_w64_kernel(const uint64_t* __r
   store_region<WHOLE>(lds, lane, first, valid, maxbits, fd.stream16, stream);
 }
 
-template <bool WHOLE, bool INT>
+// ONCE: rows stored with the nontemporal hint (Field3::once64)
+template <bool WHOLE, bool INT, bool ONCE = false>
 __global__ __launch_bounds__(64) void zfp_decode3_w64_kernel(const uint64_t* __restrict__ stream, Field3 fd,
                                                              unsigned maxbits, uint64_t* __restrict__ out)
 {
@@ -422,7 +433,7 @@ __global__ __launch_bounds__(64) void zfp_decode3_w64_kernel(const uint64_t* __r
     uint64_t q[64];
     LdsBits mem{lds};
     decode_block_w64<INT, WHOLE>(mem, lane * slot_bits(maxbits), maxbits, q);
-    store_block_w64(out, fd, first + lane, q);
+    store_block_w64<ONCE>(out, fd, first + lane, q);
   }
 }
 
@@ -654,6 +665,10 @@ static int make_field(Field3& fd, const void* base, const void* stream, size_t n
   // default policy: a lane's piece of it is not a whole line, and the decoder or the copy
   // engine reads it next.
   fd.read_once = (unsigned long long)nx * ny * nz * elem >= kReadOnceBytes;
+  // 64-bit elements: a lane's row is two 16-byte pieces, half a line per store instruction.  The
+  // hint on those stores gains 15 % at 537 MB and loses 20 % at 134 MB: only for fields of 256 MiB
+  // and more (the memory-side cache's size).
+  fd.once64 = elem == 8 && (unsigned long long)nx * ny * nz * elem >= (256ull << 20);
   return CSWAP_OK;
 }
 
@@ -735,7 +750,14 @@ static int decompress3(const uint64_t* d_stream, Elem elem, size_t nx, size_t ny
     CSWAP_LAUNCH3(zfp_decode3_f32_kernel, float, d_stream, out);
   } else {
     uint64_t* out = static_cast<uint64_t*>(d_out);
-    CSWAP_LAUNCH3(zfp_decode3_w64_kernel, uint64_t, d_stream, out);
+    if (fd.once64 && fd.rows16 && whole && !is_int)
+      hipLaunchKernelGGL((zfp_decode3_w64_kernel<true, false, true>), dim3(grid), dim3(64), lds_bytes, st, d_stream,
+                         fd, maxbits, out);
+    else if (fd.once64 && fd.rows16 && whole)
+      hipLaunchKernelGGL((zfp_decode3_w64_kernel<true, true, true>), dim3(grid), dim3(64), lds_bytes, st, d_stream,
+                         fd, maxbits, out);
+    else
+      CSWAP_LAUNCH3(zfp_decode3_w64_kernel, uint64_t, d_stream, out);
   }
   return check_launch();
 }
