@@ -264,12 +264,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void
   const uint32_t valid = min(64u, fd.nblocks - first);
   const unsigned slot = slot_bits(maxbits);
 
+  float f[64];
+  if (lane < valid) load_block<ONCE>(in, fd, first, first + lane, f);  // in flight while the region is cleared
   zero_region(lds_raw, lane, maxbits);
   __syncthreads();
 
   if (lane < valid) {
-    float f[64];
-    load_block<ONCE>(in, fd, first, first + lane, f);
     LdsBits mem{lds};
     if (INT) {
       int32_t v[64];
@@ -405,11 +405,11 @@ __global__ __launch_bounds__(64) void zfp_encode3_w64_kernel(const uint64_t* __r
   const unsigned lane = threadIdx.x;
   const uint32_t first = blockIdx.x * 64u;
   const uint32_t valid = min(64u, fd.nblocks - first);
+  uint64_t q[64];
+  if (lane < valid) load_block_w64(in, fd, first + lane, q);  // in flight while the region is cleared
   zero_region(lds_raw, lane, maxbits);
   __syncthreads();
   if (lane < valid) {
-    uint64_t q[64];
-    load_block_w64(in, fd, first + lane, q);
     LdsBits mem{lds};
     encode_block_w64<!WHOLE, INT>(q, lane * slot_bits(maxbits), maxbits, mem);
   }
