@@ -14,15 +14,18 @@ Before the W warm-up steps the same step runs, untimed, for CLOCK_SETTLE_S
 seconds: after an idle gap the GPU needs about 25 ms of continuous work to
 return to its steady clocks, and a training loop never leaves it idle.
 
-The single JSON line also carries
+The last line of stdout is ONE short JSON object (under 1500 characters) that
+also carries
   roofline      HBM-roofline figures of the dominant (slower) ZFP kernel, from
                 HIP-event timing of that kernel inside the timed region (events
-                around both kernels of every tenth step)
-  cpu_baseline  the CPU checker (a port of the reference algorithm; and the stock
-                zfp 0.5.5 library where the machine has it) timed on a
+                around both kernels of every few steps)
+  cpu_baseline  the CPU checker (a port of the reference algorithm) timed on a
                 bounded sample of the same tensor on this host
-  extra         the other kernels of the path (ZVC compact/expand, probe, other
-                rates, swap latency) -- reported, not the headline.
+  also          a handful of roofline fractions of the other kernels of the path.
+Everything else that is measured (ZVC compact/expand, probe, other rates and
+tensors, swap latency, the training steps, the per-kernel details of the two
+objects above) goes to the file named by ``extra_file`` -- reported, not the
+headline.
 """
 from __future__ import annotations
 
@@ -78,6 +81,8 @@ def main():
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
+    ap.add_argument("--extra-file", default=os.path.join(ROOT, "gpurun_out", "bench_extra.json"),
+                    help="where the figures beyond the headline line are written")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain copy kernel of the same tensor (known traffic: 4N read, 4N "
@@ -129,7 +134,7 @@ def main():
     # clocks, so that nothing but a synchronize separates the warm-up from the timed steps
     # an event record costs about 4 us of GPU time between two launches, so only every
     # `stride`-th step of the timed region carries the events that time its two kernels
-    stride = max(1, args.steps // 100)
+    stride = max(1, min(10, args.steps // 5))
     sampled = list(range(0, args.steps, stride))
     evs = {k: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for k in sampled}
     settle(torch, step, CLOCK_SETTLE_S)
@@ -161,61 +166,103 @@ def main():
     dom = "zfp_encode3_f32_kernel" if enc_ms >= dec_ms else "zfp_decode3_f32_kernel"
     dom_ms = max(enc_ms, dec_ms)
     achieved = bytes_per_value * n / (dom_ms * 1e-3) / 1e9
+
+    def frac(ms):
+        return round(bytes_per_value * n / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+
     roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                "algorithmic_bytes_per_launch": int(bytes_per_value * n),
-                "avg_launch_ms": round(dom_ms, 4),
-                "compress_ms": round(enc_ms, 4), "decompress_ms": round(dec_ms, 4),
-                "compress_frac": round(bytes_per_value * n / (enc_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                "decompress_frac": round(bytes_per_value * n / (dec_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
-    roofline["traffic"] = HBM_TRAFFIC_BYTES_PER_LAUNCH.get(dom)
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": HBM_TRAFFIC_BYTES_PER_LAUNCH.get(dom),
+                "algorithmic_bytes_per_launch": int(bytes_per_value * n), "avg_launch_ms": round(dom_ms, 4),
+                "compress_frac": frac(enc_ms), "decompress_frac": frac(dec_ms)}
 
     result = {
         "metric": "compress+decompress GB/s (fp32 in), ZFP fixed-rate 8 bits/value, 1xMI355X",
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "clock_settle_s": CLOCK_SETTLE_S, "kernel_event_samples": len(evs),
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "i32", "data": "synthetic",
+        "vs_baseline": None, "dtype": "fp32", "data": "synthetic",
         "config": {"workload": "config5 attention probabilities fp32 [32,12,512,512] = softmax(N(0,1)), "
-                               "zfp field nx=512 ny=512 nz=384, rate 8 (maxbits 512), compress then decompress",
+                               "zfp field nx=512 ny=512 nz=384, rate 8, compress then decompress",
                    "bytes_in": 4 * n, "rate_bits_per_value": rate},
         "roofline": roofline,
     }
+    detail = {"clock_settle_s": CLOCK_SETTLE_S, "kernel_event_samples": len(evs),
+              "compress_ms": round(enc_ms, 4), "decompress_ms": round(dec_ms, 4)}
 
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(x, maxbits)
+        cb = cpu_baseline(x, maxbits)
+        detail["cpu_baseline"] = cb
+        result["cpu_baseline"] = {k: cb[k] for k in ("value", "unit", "cores", "kind", "sample")}
     if not args.no_extra:
-        result["extra"] = extras(torch, api, dev)
+        ex = extras(torch, api, dev)
+        detail["extra"] = ex
+        result["also"] = headline_fractions(ex)
+    if not args.no_extra or not args.no_cpu:
+        try:
+            os.makedirs(os.path.dirname(os.path.abspath(args.extra_file)), exist_ok=True)
+            with open(args.extra_file, "w") as fh:
+                json.dump(dict(result, **detail), fh, indent=1)
+            result["extra_file"] = os.path.relpath(args.extra_file, ROOT)
+        except OSError as err:      # a read-only tree: the figures above are still printed
+            print(f"bench.py: could not write {args.extra_file}: {err}", file=sys.stderr)
     print(json.dumps(result))
 
 
-def cpu_baseline(x, maxbits):
-    """The CPU checker (port of the reference algorithm) on a bounded sample:
-    the first 4 of the 32 batch entries (50 MB) of the same tensor."""
-    import numpy as np
+def headline_fractions(ex):
+    """A few fractions of the 8 TB/s HBM roofline (algorithmic bytes) picked from
+    the extra figures, short enough for the one-line record:
+    [compress, decompress] for ZFP, [count+scan+compact, expand] for ZVC."""
+    def pick(key, a, b):
+        row = ex.get(key)
+        return [row[a], row[b]] if row else None
 
+    also = {
+        "zfp_r16_attn402MB": pick("zfp_attn_402MB_r16", "compress_hbm_frac", "decompress_hbm_frac"),
+        "zfp_r8_ffn201MB": pick("zfp_config5_ffn_gelu_r8", "compress_hbm_frac", "decompress_hbm_frac"),
+        "zfp_r8_hidden50MB": pick("zfp_config5_hidden_gelu_r8", "compress_hbm_frac", "decompress_hbm_frac"),
+        "zfp_r8_config3_34MB": pick("zfp_config3_64x32x32_r8", "compress_hbm_frac", "decompress_hbm_frac"),
+        "zfp_r8_config1_16MB": pick("zfp_config1_16MB_r8", "compress_hbm_frac", "decompress_hbm_frac"),
+        "zvc_256MiB": pick("zvc_relu_256MiB", "compress_total_hbm_frac", "expand_hbm_frac"),
+        "zvc_512MiB": pick("zvc_relu_512MiB", "compress_total_hbm_frac", "expand_hbm_frac"),
+        "zvc_config2_50pct": pick("zvc_config2_s50", "compress_total_hbm_frac", "expand_hbm_frac"),
+    }
+    sw = ex.get("swap")
+    if sw and "total_none_ms" in sw:
+        also["swap_config4_ms"] = {"raw": sw["total_none_ms"], "selector": sw["total_auto_ms"]}
+    return {k: v for k, v in also.items() if v is not None}
+
+
+def median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def cpu_baseline(x, maxbits):
+    """The CPU checker (port of the reference algorithm) on the whole tensor of
+    the workload: compress + decompress, one warm-up and the median of five runs
+    (about 15 s of CPU work on one core), then the same on all cores."""
     import oracle
 
-    sample = x[:4].cpu().numpy().reshape(-1, x.shape[-2], x.shape[-1])
+    sample = x.cpu().numpy().reshape(-1, x.shape[-2], x.shape[-1])
     nbytes = sample.nbytes
 
-    def pair(omp):
-        best = None
-        for _ in range(3):
+    def pair(omp, runs):
+        times = []
+        for i in range(runs + 1):
             t0 = time.perf_counter()
             s = oracle.zfp_encode3(sample, maxbits, omp=omp)
             t1 = time.perf_counter()
             oracle.zfp_decode3(s, sample.shape, maxbits, omp=omp)
             t2 = time.perf_counter()
-            cur = (t2 - t0, t1 - t0, t2 - t1)
-            best = cur if best is None or cur[0] < best[0] else best
-        return best
+            if i:                                  # the first run is the warm-up
+                times.append((t2 - t0, t1 - t0, t2 - t1))
+        return tuple(median([t[j] for t in times]) for j in range(3))
 
-    ser = pair(False)
-    par = pair(True)
+    ser = pair(False, 5)
+    par = pair(True, 5)
     threads = oracle.lib(True).orc_threads()
     res = {"value": round(nbytes / ser[0] / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-           "sample": "first 4 of 32 batch entries (50.3 MB) of the same tensor, compress+decompress, best of 3",
+           "sample": "the whole 402.7 MB tensor, compress+decompress, 1 warm-up + median of 5",
            "compress_GBs": round(nbytes / ser[1] / 1e9, 4), "decompress_GBs": round(nbytes / ser[2] / 1e9, 4),
            "all_cores": {"value": round(nbytes / par[0] / 1e9, 4), "cores": threads}}
     z = zfp_library_pair(sample, maxbits)
@@ -223,7 +270,7 @@ def cpu_baseline(x, maxbits):
         res["zfp_0_5_5_library"] = {"value": round(nbytes / z[0] / 1e9, 4), "cores": 1,
                                     "compress_GBs": round(nbytes / z[1] / 1e9, 4),
                                     "decompress_GBs": round(nbytes / z[2] / 1e9, 4),
-                                    "note": "stock serial codec of the image, same sample, best of 3"}
+                                    "note": "stock serial codec of the image, same tensor, best of 3"}
     return res
 
 

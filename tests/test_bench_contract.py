@@ -30,22 +30,49 @@ def test_defaults_are_one_gpu_and_a_run_of_minutes_at_most():
         assert flag in out.stdout
 
 
-@pytest.mark.gpu
-def test_json_line_on_the_gpu():
-    out = subprocess.run([sys.executable, BENCH, "--steps", "5", "--warmup", "2", "--no-extra"],
-                         capture_output=True, text=True, timeout=280)
-    assert out.returncode == 0, out.stderr[-2000:]
-    lines = [l for l in out.stdout.splitlines() if l.strip()]
-    assert len(lines) == 1
-    r = json.loads(lines[0])
-    assert r["n_gpus"] == 1 and r["steps"] == 5 and r["warmup"] == 2
+def _check_line(r, steps, warmup):
+    assert r["n_gpus"] == 1 and r["steps"] == steps and r["warmup"] == warmup
     assert r["unit"] == "GB/s" and r["higher_is_better"] is True and r["vs_baseline"] is None
-    assert r["data"] == "synthetic" and r["dtype"] == "i32" and "workload" in r["config"]
+    assert r["data"] == "synthetic" and r["dtype"] == "fp32" and "workload" in r["config"]
     assert abs(r["value"] - r["config"]["bytes_in"] / (r["ms_per_step"] * 1e-3) / 1e9) < 0.01 * r["value"]
     rf = r["roofline"]
     assert rf["bound"] == "hbm" and rf["peak"] == 8000.0 and rf["unit"] == "GB/s"
     assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-3
     assert abs(rf["achieved"] - rf["algorithmic_bytes_per_launch"] / (rf["avg_launch_ms"] * 1e-3) / 1e9) < 0.01 * rf["achieved"]
     assert 0.9 < rf["traffic"] / rf["algorithmic_bytes_per_launch"] < 1.1
+    # one kernel cannot take longer than the step that contains it
+    assert rf["avg_launch_ms"] < r["ms_per_step"]
     cb = r["cpu_baseline"]
     assert cb["kind"] == "port" and cb["cores"] == 1 and cb["unit"] == "GB/s" and cb["value"] > 0 and cb["sample"]
+
+
+@pytest.mark.gpu
+def test_json_line_on_the_gpu(tmp_path):
+    out = subprocess.run([sys.executable, BENCH, "--steps", "5", "--warmup", "2", "--no-extra",
+                          "--extra-file", str(tmp_path / "extra.json")],
+                         capture_output=True, text=True, timeout=280)
+    assert out.returncode == 0, out.stderr[-2000:]
+    lines = [l for l in out.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1 and len(lines[0]) < 1500
+    _check_line(json.loads(lines[0]), 5, 2)
+
+
+@pytest.mark.gpu
+def test_the_drivers_command_prints_a_short_last_line(tmp_path):
+    """`python bench.py --gpus 1 --steps 20 --warmup 5`, everything switched on: the
+    last line of stdout is one JSON object short enough for a 2000-character tail,
+    and the rest of the figures are in the file it names."""
+    extra = tmp_path / "extra.json"
+    out = subprocess.run([sys.executable, BENCH, "--gpus", "1", "--steps", "20", "--warmup", "5",
+                          "--extra-file", str(extra)], capture_output=True, text=True, timeout=900)
+    assert out.returncode == 0, out.stderr[-2000:]
+    last = [l for l in out.stdout.splitlines() if l.strip()][-1]
+    assert len(last) < 1500, len(last)
+    r = json.loads(last)
+    _check_line(r, 20, 5)
+    assert "extra" not in r and r["also"]
+    for pair in r["also"].values():
+        vals = pair.values() if isinstance(pair, dict) else pair
+        assert all(v > 0 for v in vals)
+    full = json.loads(extra.read_text())
+    assert full["value"] == r["value"] and "zvc_relu_512MiB" in full["extra"] and "swap" in full["extra"]
