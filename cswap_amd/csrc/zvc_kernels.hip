@@ -444,16 +444,23 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand4_kernel(
 //   ws[0]  ticket counter: tiles are handed out in the order workgroups start,
 //          so every tile a workgroup waits for belongs to a workgroup that is
 //          already running (no dependence on the dispatch order)
-//   ws[1]  error flag: set if a bounded wait ran out (never in a healthy run)
+//   ws[1]  error flag: set if a bounded wait ran out (never in a healthy run);
+//          the same event stores -1 in *nnz, which is what the caller sees
 //   ws[16 + t]  status of tile t: bits 31..30 = 0 nothing yet, 1 = count of the
 //          tile alone, 2 = inclusive prefix; bits 29..0 = the value
 constexpr uint32_t kFlagAgg = 1u << 30, kFlagPre = 2u << 30, kValMask = (1u << 30) - 1u;
 constexpr unsigned kSpinLimit = 1u << 22;
+// cswap_zvc_debug_set_lookback: the bound of the wait and the first ticket handed out
+static unsigned g_spin_limit = kSpinLimit, g_first_ticket = 0;
 
-__global__ void zvc_ws_zero_kernel(uint32_t* ws, int words)
+// Clears the workspace, sets the ticket counter and arms *nnz: the tile that ends
+// the tensor lowers it to the total with atomicMin, a wait that ran out lowers it to -1,
+// so -1 wins whichever comes first.
+__global__ void zvc_ws_zero_kernel(uint32_t* ws, int words, uint32_t first_ticket, int* nnz)
 {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < words) ws[i] = 0;
+  if (i < words) ws[i] = i == 0 ? first_ticket : 0u;
+  if (i == 0) *nnz = 0x7fffffff;
 }
 
 __device__ __forceinline__ uint32_t ld_status(const uint32_t* p)
@@ -468,7 +475,7 @@ __device__ __forceinline__ void st_status(uint32_t* p, uint32_t v)
 template <int IT, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void zvc_fused_kernel(
     const float* __restrict__ in, Geometry g, uint32_t* __restrict__ ws, int* __restrict__ begin,
-    int* __restrict__ nnz, float* __restrict__ values, uint32_t* __restrict__ mask)
+    int* __restrict__ nnz, float* __restrict__ values, uint32_t* __restrict__ mask, unsigned spin_limit)
 {
   __shared__ unsigned s_agg[WAVES];
   __shared__ unsigned s_tile;   // ticket, then the tile's exclusive offset
@@ -478,6 +485,7 @@ __global__ __launch_bounds__(64 * WAVES) void zvc_fused_kernel(
   if (threadIdx.x == 0) s_tile = atomicAdd(&ws[0], 1u);
   __syncthreads();
   const int tile = (int)s_tile;
+  if (tile >= (int)gridDim.x) return;  // only when the ticket counter did not start at zero
   const int c = tile * WAVES + wv;
   const bool in_layout = c < g.process;
   const bool has_data = c < g.active;
@@ -525,8 +533,14 @@ __global__ __launch_bounds__(64 * WAVES) void zvc_fused_kernel(
             missing |= (v[r] >> 30) == 0u;
           }
           if (__ballot(missing) == 0ull) break;
-          if (++spins > kSpinLimit) {  // give up: flag the error and let the grid drain
-            if (lane == 0) atomicOr(&ws[1], 1u);
+          if (++spins > spin_limit) {
+            // give up: report it through *nnz, then go on with what is there so that
+            // the grid drains (offsets stay below n, the output is garbage)
+            if (lane == 0) {
+              atomicOr(&ws[1], 1u);
+              atomicMin(nnz, -1);
+              __threadfence();
+            }
 #pragma unroll
             for (int r = 0; r < 4; r++) v[r] |= kFlagPre;
             break;
@@ -562,7 +576,7 @@ __global__ __launch_bounds__(64 * WAVES) void zvc_fused_kernel(
   }
   if (lane == 0) {
     begin[c] = (int)off;
-    if (c == g.active - 1) *nnz = (int)(off + agg);
+    if (c == g.active - 1) atomicMin(nnz, (int)(off + agg));
   }
 
   // ---- phase 2: mask words and packed values from the registers
@@ -756,6 +770,12 @@ extern "C" size_t cswap_zvc_workspace_bytes(int process)
   return process > 0 ? ((size_t)process + 16) * sizeof(uint32_t) : 0;
 }
 
+extern "C" void cswap_zvc_debug_set_lookback(unsigned spin_limit, unsigned first_ticket)
+{
+  g_spin_limit = spin_limit ? spin_limit : kSpinLimit;
+  g_first_ticket = first_ticket;
+}
+
 extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, void* d_ws, int* d_begin,
                                         int* d_nnz, float* d_values, uint32_t* d_mask, cswap_stream_t stream)
 {
@@ -768,11 +788,13 @@ extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, v
   if (g.E > 64 * 128 || n >= (1 << 30)) return cswap_zvc_compress(d_in, n, process, d_begin, d_nnz, d_values, d_mask, stream);
   uint32_t* ws = (uint32_t*)d_ws;
   const int words = process + 16;
-  hipLaunchKernelGGL(zvc_ws_zero_kernel, dim3((words + 255) / 256), dim3(256), 0, (hipStream_t)stream, ws, words);
+  hipLaunchKernelGGL(zvc_ws_zero_kernel, dim3((words + 255) / 256), dim3(256), 0, (hipStream_t)stream, ws, words,
+                     (uint32_t)g_first_ticket, d_nnz);
   const int iters = (g.E + 63) >> 6;
 #define CSWAP_FUSED(IT_, WAVES_)                                                                          \
   hipLaunchKernelGGL((zvc_fused_kernel<IT_, WAVES_>), dim3((g.process + WAVES_ - 1) / WAVES_),            \
-                     dim3(64 * WAVES_), 0, (hipStream_t)stream, d_in, g, ws, d_begin, d_nnz, d_values, d_mask)
+                     dim3(64 * WAVES_), 0, (hipStream_t)stream, d_in, g, ws, d_begin, d_nnz, d_values, d_mask,   \
+                     g_spin_limit)
   if (iters <= 8) CSWAP_FUSED(8, 16);
   else if (iters <= 16) CSWAP_FUSED(16, 16);
   else if (iters <= 32) CSWAP_FUSED(32, 16);

@@ -154,6 +154,42 @@ def test_fused_repeated_calls_share_a_workspace(torch_cuda):
         assert int(ws.view(torch.int32)[1].item()) == 0      # no bounded wait ran out
 
 
+def test_fused_reports_a_wait_that_ran_out(torch_cuda):
+    """The single-pass kernel's wait for the chunks before it is bounded.  Forced
+    from the host: the first piece of work is never handed out and the bound is a
+    few re-reads, so every later piece gives up at once, every kernel still exits
+    normally, and the caller sees nnz == -1 instead of made-up offsets.  The next
+    call, with the defaults back, is correct again."""
+    torch = torch_cuda
+    from cswap_amd import api
+    from cswap_amd._lib import check, lib
+
+    L = lib()
+    n = P * 256
+    x = np.maximum(np.random.default_rng(5).standard_normal(n), 0).astype(np.float32)
+    t = torch.from_numpy(x).cuda()
+    ws = torch.empty(L.cswap_zvc_workspace_bytes(P), dtype=torch.uint8, device="cuda")
+    values = torch.empty(n, device="cuda"); mask = torch.empty(n // 32, dtype=torch.int32, device="cuda")
+    begin = torch.zeros(P, dtype=torch.int32, device="cuda"); nnz = torch.zeros(1, dtype=torch.int32, device="cuda")
+    L.cswap_zvc_debug_set_lookback(4, 1)
+    try:
+        print("forced give-up", flush=True)
+        check(L.cswap_zvc_compress_fused(t.data_ptr(), n, P, ws.data_ptr(), begin.data_ptr(), nnz.data_ptr(),
+                                         values.data_ptr(), mask.data_ptr(), None), "fused")
+        torch.cuda.synchronize()
+    finally:
+        L.cswap_zvc_debug_set_lookback(0, 0)
+    assert int(nnz.item()) == -1
+    assert int(ws.view(torch.int32)[1].item()) == 1
+    check(L.cswap_zvc_compress_fused(t.data_ptr(), n, P, ws.data_ptr(), begin.data_ptr(), nnz.data_ptr(),
+                                     values.data_ptr(), mask.data_ptr(), None), "fused")
+    torch.cuda.synchronize()
+    k = int(nnz.item())
+    assert k == np.count_nonzero(x)
+    assert np.array_equal(values[:k].cpu().numpy(), x[x != 0])
+    check_against_oracle(x, run_gpu(torch, x, fused=True))
+
+
 def test_special_values_and_extremes(torch_cuda, compact_form):
     n = P * 64
     x = np.zeros(n, dtype=np.float32)
