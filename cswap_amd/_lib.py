@@ -103,6 +103,7 @@ _SIGNATURES = {
     "cswap_zvc_compress": (i32, [vp, i32, i32, vp, vp, vp, vp, vp]),
     "cswap_zvc_workspace_bytes": (sz, [i32]),
     "cswap_zvc_compress_fused": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp]),
+    "cswap_zvc_debug_set_lookback": (None, [u, u]),
     "cswap_probe_nnz": (i32, [vp, sz, vp, vp]),
     "cswap_costs_default": (None, [C.POINTER(Costs)]),
     "cswap_policy_bytes": (sz, [i32, sz, sz, u, i32, sz, sz, sz]),
@@ -117,6 +118,7 @@ _SIGNATURES = {
     "cswap_swap_prefetch": (i32, [vp, i32]),
     "cswap_swap_release": (i32, [vp, i32]),
     "cswap_swap_info": (i32, [vp, i32, C.POINTER(TicketInfo)]),
+    "cswap_engine_probe_count": (C.c_ulonglong, [vp]),
     "cswap_engine_calibrate": (i32, [vp, C.POINTER(Costs)]),
     "cswap_engine_copy_stream": (vp, [vp]),
     "cswap_engine_tune": (i32, [vp, sz, C.POINTER(i32)]),

@@ -121,10 +121,18 @@ struct cswap_engine {
   int* d_nnz = nullptr;
   hipEvent_t ev_probe = nullptr;
   int device = 0;
+  unsigned long long probes = 0;  // counting passes with a host round trip so far
 };
 
 // layout of a ZVC payload: [begin: process ints][mask][values: nnz floats]
 static size_t zvc_header_bytes(int n, int process) { return 4 * (size_t)process + cswap_zvc_mask_bytes(n, process); }
+
+extern "C" unsigned long long cswap_engine_probe_count(cswap_engine* e)
+{
+  if (!e) return 0;
+  std::lock_guard<std::mutex> lock(e->mu);
+  return e->probes;
+}
 
 extern "C" void cswap_engine_config_default(cswap_engine_config* cfg)
 {
@@ -264,6 +272,7 @@ static int probe_tensor(cswap_engine* e, Ticket& t, const float* d_in, hipStream
   if (err == hipSuccess) err = hipEventSynchronize(e->ev_probe);
   if (err != hipSuccess) { abandon_device(e, t, compute); return hip_fail(err); }
   t.nnz = (size_t)*e->h_nnz;
+  e->probes++;
   return CSWAP_OK;
 }
 

@@ -97,6 +97,10 @@ class SwapEngine:
         check(lib().cswap_engine_tune(self._h, numel, C.byref(best)), "cswap_engine_tune")
         return best.value
 
+    def probe_count(self) -> int:
+        """Counting passes with a host round trip the engine has run so far."""
+        return lib().cswap_engine_probe_count(self._h)
+
     def process_for(self, numel: int) -> int:
         return lib().cswap_engine_process_for(self._h, numel)
 

@@ -83,4 +83,15 @@ void cswap_compat_set_field(size_t nx, size_t ny);
 #ifdef __cplusplus
 }
 #endif
+
+#if defined(__cplusplus) && !defined(CSWAP_COMPAT_NO_PROTOTYPES)
+/* The form the reference's call sites use,
+ *   buffer = compress(pre.data_ptr(), pre.numel(), buffersize);
+ * (CSWAP+/Execution.h:113,201: the size comes back through a size_t lvalue), so
+ * that those lines compile unchanged. */
+inline void* compress(void* dev_ptr, long long numel, size_t& out_bytes)
+{
+  return compress(dev_ptr, numel, &out_bytes);
+}
+#endif
 #endif /* CSWAP_COMPAT_H */

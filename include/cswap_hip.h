@@ -164,10 +164,20 @@ int cswap_zvc_compress(const float* d_in, int n, int process, int* d_begin, int*
  * traffic is the algorithmic 4 + 1/8 + 4*density bytes per element.  d_ws is
  * scratch of cswap_zvc_workspace_bytes(process) bytes, cleared by the call
  * itself; calls that share a workspace must not overlap.  Tensors whose chunks
- * exceed 8192 elements (n > 8192*process) fall back to the three-kernel path. */
+ * exceed 8192 elements (n > 8192*process) fall back to the three-kernel path.
+ * A wavefront waits for the offsets of the chunks before its own; that wait is
+ * bounded, and if it ever runs out the kernel still finishes but *d_nnz is -1
+ * and the other outputs are undefined: a caller must treat a negative count as
+ * failure (the return value cannot tell, the call does not synchronise). */
 size_t cswap_zvc_workspace_bytes(int process);
 int cswap_zvc_compress_fused(const float* d_in, int n, int process, void* d_ws, int* d_begin,
                              int* d_nnz, float* d_values, uint32_t* d_mask, cswap_stream_t stream);
+/* For tests of that failure path only.  spin_limit: how many times a wavefront
+ * re-reads the status words it waits for before it gives up (0 = the default,
+ * about four million); first_ticket: the first piece of work handed out, so that
+ * with 1 the first piece is never done and every later one waits in vain.
+ * Process-wide; (0, 0) restores normal operation. */
+void cswap_zvc_debug_set_lookback(unsigned spin_limit, unsigned first_ticket);
 
 /* ---------------------------------------------------------------- probe -----
  * One fused read pass: *d_nnz = number of elements != 0 (the quantity the
@@ -293,6 +303,10 @@ int cswap_swap_prefetch(cswap_engine* e, int ticket);
  * work of the ticket that is still in flight. */
 int cswap_swap_release(cswap_engine* e, int ticket);
 int cswap_swap_info(cswap_engine* e, int ticket, cswap_ticket_info* info);
+/* Number of probes so far: counting passes followed by the host round trip for
+ * the non-zero count (the one at Execution.h:92), which a selector-driven or ZVC
+ * swap-out pays and an explicit raw or ZFP request does not. */
+unsigned long long cswap_engine_probe_count(cswap_engine* e);
 /* Measure link bandwidth and kernel throughput on this box and store them in
  * the engine's cost model (allocates temporaries; call once after create). */
 int cswap_engine_calibrate(cswap_engine* e, cswap_costs* out_costs);

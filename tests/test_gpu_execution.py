@@ -168,23 +168,96 @@ def test_cpp_driver_with_policy_maker_and_execution():
     Python, no torch): calibrate, plan most of the activation bytes with
     cswap::PolicyMaker, walk forward with cswap::Execution::pre/post, walk backward
     with prefetch/fetch, and compare every tensor that comes back byte for byte."""
+    out = _build_and_run_cpp("cpp_schedule_walk")
+    assert out.returncode == 0, out.stdout
+    tag, swapped, link = out.stdout.split()[-3:]
+    assert tag == "OK" and int(swapped) >= 3 and int(link) > 0
+    policy = [int(v) for v in out.stdout.split("policy:")[1].split("OK")[0].split()]
+    assert 3 in policy and 2 in policy                       # ZVC for the ReLU-like tensors, raw for the (de-ZFP-ed) dense ones
+
+
+def _build_and_run_cpp(name, timeout=100):
     import os
     import subprocess
     import tempfile
 
     from conftest import ROOT
 
-    src = os.path.join(ROOT, "tests", "cpp_schedule_walk.cpp")
+    src = os.path.join(ROOT, "tests", name + ".cpp")
     lib = os.path.join(ROOT, "cswap_amd", "libcswap_hip.so")
     with tempfile.TemporaryDirectory() as d:
-        exe = os.path.join(d, "walk")
+        exe = os.path.join(d, name)
         subprocess.check_call(["g++", "-std=c++17", "-O1", "-Wall", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROOT, "include"),
                                "-I/opt/rocm/include", src, lib, "-Wl,-rpath," + os.path.dirname(lib),
                                "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib", "-lamdhip64", "-o", exe])
-        out = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+        out = subprocess.run([exe], capture_output=True, text=True, timeout=timeout)
     print(out.stdout, out.stderr, flush=True)
+    return out
+
+
+def test_cpp_selector_memo_skips_the_probe_for_remembered_decisions():
+    """tests/cpp_selector_memo.cpp: with policy[] = -1 the C++ mirror asks the
+    selector in the first iteration and reuses a ZFP or raw decision afterwards
+    without the counting pass and its host round trip (Execution.h:89-92), until
+    `recheck` reuses are spent; a ZVC tensor is probed every time."""
+    out = _build_and_run_cpp("cpp_selector_memo")
     assert out.returncode == 0, out.stdout
-    tag, swapped, link = out.stdout.split()[-3:]
-    assert tag == "OK" and int(swapped) >= 3 and int(link) > 0
-    policy = [int(v) for v in out.stdout.split("policy:")[1].split("OK")[0].split()]
-    assert 3 in policy and 2 in policy                       # ZVC for the ReLU-like tensors, raw for the (de-ZFP-ed) dense ones
+    assert out.stdout.split()[-6:] == ["OK", "2", "1", "1", "2", "1"]
+
+
+def test_python_mirror_selector_memo_and_global_modes():
+    """The Python twin: the same memo, and the reference's global modes -- under
+    policy_ = 3 (vDNN) every input of a convolution goes out raw whatever its
+    entry says, under policy_ = 4 (SuperNeurons) everything else is dropped
+    (Execution.h:70,243)."""
+    import torch
+
+    from cswap_amd import swap
+    from cswap_amd.execution import ACT, CONV, Execution
+
+    eng = swap.SwapEngine(pinned_bytes=256 << 20, device_bytes=256 << 20)
+    dense = torch.randn(64, 64, 32, 32, device="cuda")
+    relu = torch.relu(torch.randn(64, 64, 32, 32, device="cuda") - 0.6)
+    exe = Execution(eng)
+    exe.init_(4)
+    exe.policy = [-1, -1, 0, 0]
+    exe.recheck = 3
+    per_iter = []
+    for _ in range(3):
+        before = eng.probe_count()
+        exe.preforward()
+        exe.pre(dense, -1); exe.post()
+        exe.pre(dense, 0); exe.post()
+        exe.pre(relu, 1); exe.post()
+        exe.postforward()
+        per_iter.append(eng.probe_count() - before)
+        assert exe.com_and_tran(0) == swap.ZFP and exe.com_and_tran(1) == swap.SPARSE
+        back = exe.fetch(1)
+        assert torch.equal(back, relu)
+        assert float((exe.fetch(0) - dense).abs().max()) < 0.5
+    assert per_iter == [2, 1, 1] and exe.memo_hits == 2
+
+    # global modes
+    exe = Execution(eng)
+    exe.init_(4)
+    exe.policy = [3, 6, 2, 0]
+    exe.policy_ = 3
+    exe.preforward()
+    exe.pre(dense, -1, CONV); exe.post()
+    exe.pre(relu, 0, CONV); exe.post()          # entry 3, but a convolution consumes it under vDNN: raw
+    exe.pre(dense, 1, ACT); exe.post()          # entry 6, consumer is not a convolution: ZFP as written
+    assert exe.com_and_tran(0) == 2 and exe.com_and_tran(1) == 6
+    assert torch.equal(exe.fetch(0), relu)
+    exe.fetch(1)
+    exe.policy_ = 4
+    exe.preforward()
+    exe.pre(dense, -1, CONV); exe.post()
+    exe.pre(relu, 0, ACT); exe.post()           # SuperNeurons: not a convolution input -> dropped
+    exe.pre(dense, 1, CONV); exe.post()         # convolution input -> raw swap
+    exe.pre(relu, 2, ACT); exe.post()           # entry 2, still dropped: the drop branch comes first
+    assert exe.com_and_tran(0) == 1 and exe.dropped(0) and not exe.swapped(0)
+    assert exe.com_and_tran(1) == 2 and exe.com_and_tran(2) == 1
+    assert torch.equal(exe.fetch(1), dense)
+    with pytest.raises(KeyError):
+        exe.fetch(0)                            # nothing to bring back: the caller recomputes it
+    eng.close()
