@@ -13,6 +13,9 @@
 // format carries anyway (`begin`) is the device-wide scan; no finer scan is
 // needed.
 #include <hip/hip_runtime.h>
+
+#include <mutex>
+
 #include "../../include/cswap_hip.h"
 #include "common.h"
 
@@ -802,6 +805,39 @@ extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, v
   else CSWAP_FUSED(128, 8);
 #undef CSWAP_FUSED
   return check_launch();
+}
+
+// ------------------------------------------------------------------ no allocation
+// The single-pass compression once more, for callers that cannot bring a workspace
+// because they cannot allocate one: the status words live in this array, one copy
+// per GPU, held until the process ends.
+constexpr int kStaticProcessMax = 65536;
+static __device__ __align__(256) uint32_t scratch[kStaticProcessMax + 16];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+uint32_t* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, once looked up
+}  // namespace
+
+extern "C" int cswap_zvc_compress_fused_static(const float* d_in, int n, int process, int* d_begin, int* d_nnz,
+                                               float* d_values, uint32_t* d_mask, cswap_stream_t stream)
+{
+  if (process > kStaticProcessMax) return CSWAP_E_NOMEM;
+  int dev = -1;
+  CSWAP_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return CSWAP_E_UNSUPPORTED;
+  uint32_t* ws;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {  // first call on this GPU: where its copy of the array lives
+      void* p = nullptr;
+      CSWAP_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+      g_scratch_ptr[dev] = static_cast<uint32_t*>(p);
+    }
+    ws = g_scratch_ptr[dev];
+  }
+  return cswap_zvc_compress_fused(d_in, n, process, ws, d_begin, d_nnz, d_values, d_mask, stream);
 }
 
 extern "C" int cswap_probe_nnz(const float* d_in, size_t n, unsigned long long* d_nnz, cswap_stream_t stream)

@@ -178,6 +178,15 @@ int cswap_zvc_compress_fused(const float* d_in, int n, int process, void* d_ws, 
  * with 1 the first piece is never done and every later one waits in vain.
  * Process-wide; (0, 0) restores normal operation. */
 void cswap_zvc_debug_set_lookback(unsigned spin_limit, unsigned first_ticket);
+/* No counterpart in the reference.  cswap_zvc_compress_fused for callers that
+ * cannot allocate a workspace (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc): the status words live in a static device
+ * array of the library (256 KiB per GPU, held until the process ends), so the
+ * call takes no workspace and allocates nothing.  process <= 65536, otherwise
+ * CSWAP_E_NOMEM.  Every call on a GPU uses that GPU's one array: calls that
+ * overlap on one GPU (different streams, different threads) race. */
+int cswap_zvc_compress_fused_static(const float* d_in, int n, int process, int* d_begin, int* d_nnz,
+                                    float* d_values, uint32_t* d_mask, cswap_stream_t stream);
 
 /* ---------------------------------------------------------------- probe -----
  * One fused read pass: *d_nnz = number of elements != 0 (the quantity the
