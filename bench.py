@@ -343,12 +343,15 @@ def zvc_extras(torch, api, dev, ex, config2_tensor, only_256=False):
         from cswap_amd._lib import lib
         L = lib()
         st = torch.cuda.current_stream().cuda_stream
-        full = ev_ms(torch, lambda: L.cswap_zvc_compress(t.data_ptr(), n, api.PROCESS, begin.data_ptr(),
-                                                         nnz.data_ptr(), values.data_ptr(), mask.data_ptr(), st), reps)
+        three = ev_ms(torch, lambda: L.cswap_zvc_compress(t.data_ptr(), n, api.PROCESS, begin.data_ptr(),
+                                                          nnz.data_ptr(), values.data_ptr(), mask.data_ptr(), st), reps)
         ws = torch.empty(L.cswap_zvc_workspace_bytes(api.PROCESS), dtype=torch.uint8, device=dev)
-        fused = ev_ms(torch, lambda: L.cswap_zvc_compress_fused(t.data_ptr(), n, api.PROCESS, ws.data_ptr(),
-                                                                begin.data_ptr(), nnz.data_ptr(),
-                                                                values.data_ptr(), mask.data_ptr(), st), reps)
+        # count + scan + compact as one operation, as the swap engine runs it for a ZVC request: the
+        # single pass from 128 MiB on, the three kernels below
+        full = ev_ms(torch, lambda: L.cswap_zvc_compress_fused(t.data_ptr(), n, api.PROCESS, ws.data_ptr(),
+                                                               begin.data_ptr(), nnz.data_ptr(),
+                                                               values.data_ptr(), mask.data_ptr(), st), reps)
+        single = bool(L.cswap_zvc_takes_single_pass(n, api.PROCESS))
         cnt = torch.zeros(api.PROCESS, dtype=torch.int32, device=dev)
         count = ev_ms(torch, lambda: L.cswap_zvc_count(t.data_ptr(), n, api.PROCESS, cnt.data_ptr(), st), reps)
         compact = ev_ms(torch, lambda: L.cswap_zvc_compact(t.data_ptr(), n, api.PROCESS, begin.data_ptr(),
@@ -360,8 +363,9 @@ def zvc_extras(torch, api, dev, ex, config2_tensor, only_256=False):
         ex[f"zvc_{label}"] = {
             "density": round(dens, 4), "ratio": round((4 * k + n / 8 + 4 * api.PROCESS) / (4 * n), 4),
             "count_ms": round(count, 4), "compact_ms": round(compact, 4), "compress_total_ms": round(full, 4),
-            "compress_fused_ms": round(fused, 4),
-            "compress_fused_hbm_frac": round(bpv * n / fused / 1e6 / HBM_PEAK_GBS, 4),
+            "compress_total_is_single_pass": single,
+            "compress_three_kernels_ms": round(three, 4),
+            "compress_three_kernels_hbm_frac": round(bpv * n / three / 1e6 / HBM_PEAK_GBS, 4),
             "expand_ms": round(expand, 4), "probe_ms": round(probe, 4),
             "compact_GBs_fp32": round(4 * n / compact / 1e6, 1), "expand_GBs_fp32": round(4 * n / expand / 1e6, 1),
             "compact_hbm_frac": round(bpv * n / compact / 1e6 / HBM_PEAK_GBS, 4),

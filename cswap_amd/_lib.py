@@ -96,6 +96,8 @@ _SIGNATURES = {
     "cswap_zvc_mask_bytes": (sz, [i32, i32]),
     "cswap_zvc_pick_process": (i32, [sz]),
     "cswap_zvc_set_staged_compact_bytes": (sz, [sz]),
+    "cswap_zvc_set_single_pass_bytes": (sz, [sz]),
+    "cswap_zvc_takes_single_pass": (i32, [i32, i32]),
     "cswap_zvc_count": (i32, [vp, i32, i32, vp, vp]),
     "cswap_zvc_scan": (i32, [vp, i32, vp, vp]),
     "cswap_zvc_compact": (i32, [vp, i32, i32, vp, vp, vp, vp]),
@@ -159,6 +161,13 @@ def lib() -> C.CDLL:
             raise ImportError(
                 f"{LIB_PATH} is missing: build it with `python -m cswap_amd.build` "
                 "(there is no CPU fallback)")
+        # torch ships its own copy of the HIP runtime; if this library (linked against the
+        # system's) is the first to bring a runtime into the process and initialise it, torch
+        # afterwards reports no GPU.  Importing torch first makes both use the one torch loads.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = C.CDLL(LIB_PATH)
         for name, (res, args) in _SIGNATURES.items():
             f = getattr(L, name)  # AttributeError if the symbol is not exported

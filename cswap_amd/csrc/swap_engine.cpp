@@ -119,10 +119,13 @@ struct cswap_engine {
   unsigned maxbits = 512;
   int* h_nnz = nullptr;  // pinned, 1 int
   int* d_nnz = nullptr;
+  void* d_ws = nullptr;  // status words of the single-pass ZVC kernel (chunk counts up to kWsProcess)
   hipEvent_t ev_probe = nullptr;
   int device = 0;
   unsigned long long probes = 0;  // counting passes with a host round trip so far
 };
+
+constexpr int kWsProcess = 65536;  // the engine's single-pass workspace serves chunk counts up to this
 
 // layout of a ZVC payload: [begin: process ints][mask][values: nnz floats]
 static size_t zvc_header_bytes(int n, int process) { return 4 * (size_t)process + cswap_zvc_mask_bytes(n, process); }
@@ -157,6 +160,7 @@ extern "C" void cswap_engine_destroy(cswap_engine* e)
   if (e->ev_probe) (void)hipEventDestroy(e->ev_probe);
   if (e->h_nnz) (void)hipHostFree(e->h_nnz);
   if (e->d_nnz) (void)hipFree(e->d_nnz);
+  if (e->d_ws) (void)hipFree(e->d_ws);
   if (e->h_base) (void)hipHostFree(e->h_base);
   if (e->d_base) (void)hipFree(e->d_base);
   if (e->copy) (void)hipStreamDestroy(e->copy);
@@ -192,6 +196,7 @@ extern "C" int cswap_engine_create(cswap_engine** out, const cswap_engine_config
     if ((err = hipMalloc((void**)&e->d_base, cfg.device_pool_bytes)) != hipSuccess) { fail(err); break; }
     if ((err = hipHostMalloc((void**)&e->h_nnz, 256, hipHostMallocDefault)) != hipSuccess) { fail(err); break; }
     if ((err = hipMalloc((void**)&e->d_nnz, 256)) != hipSuccess) { fail(err); break; }
+    if ((err = hipMalloc(&e->d_ws, cswap_zvc_workspace_bytes(kWsProcess))) != hipSuccess) { fail(err); break; }
     if ((err = hipEventCreateWithFlags(&e->ev_probe, hipEventDisableTiming)) != hipSuccess) { fail(err); break; }
     e->hpool.reset(cfg.pinned_pool_bytes);
     e->dpool.reset(cfg.device_pool_bytes);
@@ -273,6 +278,45 @@ static int probe_tensor(cswap_engine* e, Ticket& t, const float* d_in, hipStream
   if (err != hipSuccess) { abandon_device(e, t, compute); return hip_fail(err); }
   t.nnz = (size_t)*e->h_nnz;
   e->probes++;
+  return CSWAP_OK;
+}
+
+// An explicit ZVC request for a large tensor: count, scan and compaction in one pass over the
+// tensor, straight into a staging block of the worst-case size that is cut back to what was
+// needed once the non-zero count is on the host (the same small round trip a probe makes).
+// Returns 1 if it did not run (no room for the worst case, a chunk count beyond the
+// workspace) or did not finish its job (the bounded wait inside the kernel ran out): the caller
+// then takes the probe path, with nothing held.  On success the ticket holds its staging block
+// and *src is the payload.
+static int single_pass_sparse(cswap_engine* e, Ticket& t, const float* d_in, hipStream_t compute, const void** src)
+{
+  if (t.process > kWsProcess || !cswap_zvc_takes_single_pass((int)t.n, t.process)) return 1;
+  const size_t hdr = zvc_header_bytes((int)t.n, t.process);
+  const size_t worst = hdr + 4 * t.n;
+  size_t off;
+  if (!e->dpool.alloc(worst, &off)) return 1;
+  char* base = e->d_base + off;
+  int rc = cswap_zvc_compress_fused(d_in, (int)t.n, t.process, e->d_ws, (int*)base, e->d_nnz, (float*)(base + hdr),
+                                    (uint32_t*)(base + 4 * (size_t)t.process), compute);
+  hipError_t err = hipSuccess;
+  if (!rc) err = hipMemcpyAsync(e->h_nnz, e->d_nnz, sizeof(int), hipMemcpyDeviceToHost, compute);
+  if (!rc && err == hipSuccess) err = hipEventRecord(e->ev_probe, compute);
+  if (!rc && err == hipSuccess) err = hipEventSynchronize(e->ev_probe);
+  if (rc || err != hipSuccess) {
+    (void)hipStreamSynchronize(compute);
+    e->dpool.free(off, worst);
+    return rc ? rc : hip_fail(err);
+  }
+  if (*e->h_nnz < 0) {  // kernels have finished (the event): the block can go back at once
+    e->dpool.free(off, worst);
+    return 1;
+  }
+  t.nnz = (size_t)*e->h_nnz;
+  t.bytes_out = hdr + 4 * t.nnz;
+  e->dpool.shrink(off, worst, t.bytes_out);
+  t.dev_off = off; t.dev_bytes = t.bytes_out; t.dev_held = true;
+  e->probes++;
+  *src = base;
   return CSWAP_OK;
 }
 
@@ -387,6 +431,31 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     if (best_case.policy == CSWAP_POLICY_NONE) {
       t.policy = CSWAP_POLICY_NONE;
       want_probe = false;
+    }
+  }
+  if (policy == CSWAP_POLICY_SPARSE) {
+    const void* payload = nullptr;
+    rc = single_pass_sparse(e, t, d_in, compute, &payload);
+    if (rc < 0) return rc;
+    if (rc == 0) {
+      size_t hoff;
+      if (!e->hpool.alloc(t.bytes_out, &hoff)) {
+        (void)hipStreamSynchronize(compute);
+        drop_device(e, t);
+        return CSWAP_E_NOMEM;
+      }
+      t.host_off = hoff; t.host_bytes = t.bytes_out;
+      rc = start_outbound_copy(e, t, payload, compute);
+      if (rc) {
+        (void)hipStreamSynchronize(compute);
+        (void)hipStreamSynchronize(e->copy);
+        drop_device(e, t);
+        e->hpool.free(t.host_off, t.host_bytes);
+        return rc;
+      }
+      t.state = kOutInFlight;
+      *ticket = id;
+      return CSWAP_OK;
     }
   }
   if (want_probe && (rc = probe_tensor(e, t, d_in, compute, policy == CSWAP_POLICY_SPARSE))) return rc;

@@ -433,36 +433,20 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand4_kernel(
   }
 }
 
-// ------------------------------------------------------------------ fused
-// count + scan + compact in ONE pass over the tensor: a wavefront keeps its whole
-// chunk in registers (IT values per lane) and counts it; the WAVES chunks of a
-// workgroup form a tile whose exclusive offset comes from a decoupled look-back
-// over tile-granular status words; then every wave writes mask and packed values
-// from its registers.  HBM traffic is the algorithmic 4 + 1/8 + 4d bytes per
-// element.  Tiles (not chunks) are the unit of the look-back, and one memory
-// round trip covers a window of 256 tiles, because a workgroup that starts while
-// thousands of others are in flight has to walk back over all of them.
-//
-// Workspace (zeroed by zvc_ws_zero_kernel before every launch):
-//   ws[0]  ticket counter: tiles are handed out in the order workgroups start,
-//          so every tile a workgroup waits for belongs to a workgroup that is
-//          already running (no dependence on the dispatch order)
-//   ws[1]  error flag: set if a bounded wait ran out (never in a healthy run);
-//          the same event stores -1 in *nnz, which is what the caller sees
-//   ws[16 + t]  status of tile t: bits 31..30 = 0 nothing yet, 1 = count of the
-//          tile alone, 2 = inclusive prefix; bits 29..0 = the value
-constexpr uint32_t kFlagAgg = 1u << 30, kFlagPre = 2u << 30, kValMask = (1u << 30) - 1u;
-constexpr unsigned kSpinLimit = 1u << 22;
-// cswap_zvc_debug_set_lookback: the bound of the wait and the first ticket handed out
-static unsigned g_spin_limit = kSpinLimit, g_first_ticket = 0;
+// ------------------------------------------------------------------ status words
+// The single-pass kernel below exchanges counts between workgroups through status words
+// in global memory, read and written with relaxed atomics of agent scope (they travel past
+// the per-XCD L2 caches, which are not coherent with each other).
+constexpr unsigned kSpinLimit = 1u << 20;
+// cswap_zvc_debug_set_lookback: the bound of the waits, and whether tile 0 is never published
+static unsigned g_spin_limit = kSpinLimit, g_skip_first = 0;
 
-// Clears the workspace, sets the ticket counter and arms *nnz: the tile that ends
-// the tensor lowers it to the total with atomicMin, a wait that ran out lowers it to -1,
-// so -1 wins whichever comes first.
-__global__ void zvc_ws_zero_kernel(uint32_t* ws, int words, uint32_t first_ticket, int* nnz)
+// Clears the workspace and arms *nnz: the scanner lowers it to the total with atomicMin, a
+// wait that ran out lowers it to -1, so -1 wins whichever comes first.
+__global__ void zvc_ws_zero_kernel(uint32_t* ws, int words, int* nnz)
 {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < words) ws[i] = i == 0 ? first_ticket : 0u;
+  if (i < words) ws[i] = 0u;
   if (i == 0) *nnz = 0x7fffffff;
 }
 
@@ -475,133 +459,317 @@ __device__ __forceinline__ void st_status(uint32_t* p, uint32_t v)
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int IT, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void zvc_fused_kernel(
-    const float* __restrict__ in, Geometry g, uint32_t* __restrict__ ws, int* __restrict__ begin,
-    int* __restrict__ nnz, float* __restrict__ values, uint32_t* __restrict__ mask, unsigned spin_limit)
+// ------------------------------------------------------------------ stream
+// count + scan + compact in one pass, as a pipeline that never holds data while it
+// waits.  The tensor is cut into tiles of 192 rows (a row = 64 elements = two mask
+// words); a grid of G resident workgroups (one per compute unit) walks them round
+// robin: workgroup w takes tiles w, w+G, w+2G, ...  Each of its sixteen wavefronts keeps
+// 12 rows of five consecutive tiles of the workgroup in registers: while tile i is
+// compacted, tiles i+1 and i+2 wait counted, tile i+3 is counted and its count published,
+// and the loads of tile i+4 are issued one row at a time between the rows of tile i, so
+// that memory sees a steady stream of requests instead of bursts.  One more workgroup,
+// the scanner, reads the published counts in tile order and publishes each tile's offset;
+// a count is published two stages before its tile's offset is needed, which covers the two
+// trips through memory (count to the scanner, offset back) that take about a stage each on
+// this part, so a workgroup that asks for the offset of its next tile at the start of a
+// stage has it when the stage ends, and nobody waits for anybody's latest step.  The
+// compacted values go through an LDS stage per tile and leave as whole 16-byte groups
+// aligned in the values array.
+//
+// Needs: chunk length a multiple of 32 (the mask is then the flat bit mask and a chunk
+// starts on a half row), two status words per tile in the workspace, a 16-byte aligned
+// values pointer, and all G+1 workgroups resident at once (the waits are bounded).
+// Workspace, zero before the launch: ws[16 + t] = kTileReady | count of tile t,
+// ws[16 + tiles + t] = kTileReady | number of non-zeros before tile t.
+//
+// Measured on one MI355X, half of the elements zero (this kernel / count + scan + compact):
+// 512 MiB 0.191 / 0.240 ms, 256 MiB 0.097 / 0.115 ms, 32 MiB 0.024 / 0.020 ms (a tensor of
+// a few rounds of the grid does not fill the pipeline).
+constexpr int kSWaves = 16, kSRows = 12;
+constexpr int kSTileRows = kSWaves * kSRows, kSTileElems = kSTileRows * 64;
+constexpr int kSSlots = 5;   // tiles of a workgroup in registers
+constexpr int kSAhead = kSSlots - 1;  // the loads run this many tiles ahead of the compaction
+constexpr uint32_t kTileReady = 1u << 31;
+
+struct StreamGeometry {
+  int n, E, process, active;
+  int rows;    // rows that exist in the mask layout: process * E / 64 rounded up
+  int tiles;   // ceil(rows / 256)
+  int mask_words;
+};
+
+// Inclusive prefix sum over the 64 lanes of a wavefront with data-parallel-primitive
+// moves (row shifts inside rows of 16 lanes, then the row broadcasts): six additions, no
+// trip through the LDS crossbar that a shuffle takes.
+__device__ __forceinline__ unsigned wave_inclusive_scan(unsigned v)
 {
-  __shared__ unsigned s_agg[WAVES];
-  __shared__ unsigned s_tile;   // ticket, then the tile's exclusive offset
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, false);  // row_shr:1
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, false);  // row_shr:2
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, false);  // row_shr:4
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, false);  // row_shr:8
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1, 3
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2, 3
+  return v;
+}
+
+// The scanner: one wavefront turns counts into offsets, 256 tiles at a time, in tile order.
+__device__ void zvc_stream_scanner(uint32_t* ws, int tiles, int step, int* nnz, unsigned spin_limit)
+{
+  if (threadIdx.x >= 64) return;
   const unsigned lane = lane_id();
-  const int wv = (int)(threadIdx.x >> 6);
   uint32_t* status = ws + 16;
-  if (threadIdx.x == 0) s_tile = atomicAdd(&ws[0], 1u);
-  __syncthreads();
-  const int tile = (int)s_tile;
-  if (tile >= (int)gridDim.x) return;  // only when the ticket counter did not start at zero
-  const int c = tile * WAVES + wv;
-  const bool in_layout = c < g.process;
-  const bool has_data = c < g.active;
-
-  const long long b = (long long)g.E * c;
-  const int len = has_data ? (int)min((long long)g.E, (long long)g.n - b) : 0;
-  const float* p = in + b;
-  const int iters = (g.E + 63) >> 6;  // <= IT
-
-  // ---- phase 1: the chunk into registers, and its count
-  float x[IT];
+  uint32_t* offset = ws + 16 + tiles;
+  unsigned carry = 0;
+  // `step` tiles at a time (at most 256): the tiles that the data workgroups count in the same
+  // stage, so that a step never waits for a count that is published a stage later than the rest
+  for (int t0 = 0; t0 < tiles; t0 += step) {
+    // lane l owns tiles t0 + 4l .. t0 + 4l + 3
+    const int stop = t0 + step < tiles ? t0 + step : tiles;
+    uint32_t v[4];
+    unsigned spins = 0;
+    for (;;) {
+      bool missing = false;
 #pragma unroll
-  for (int t = 0; t < IT; t++) {
-    const int k = t * 64 + (int)lane;
-    x[t] = (t < iters && k < len) ? p[k] : 0.0f;
-  }
-  unsigned agg = 0;
-#pragma unroll
-  for (int t = 0; t < IT; t++) agg += popc64(__ballot(x[t] != 0.0f));
-  if (lane == 0) s_agg[wv] = agg;
-  __syncthreads();  // also orders the read of the ticket before s_tile is reused
-
-  // ---- wave 0: decoupled look-back over the tiles before this one
-  if (wv == 0) {
-    unsigned tile_agg = 0;
-#pragma unroll
-    for (int w = 0; w < WAVES; w++) tile_agg += s_agg[w];
-    unsigned excl = 0;
-    if (tile == 0) {
-      if (lane == 0) st_status(&status[0], kFlagPre | tile_agg);
-    } else {
-      if (lane == 0) st_status(&status[tile], kFlagAgg | tile_agg);
-      int idx = tile - 1;
-      bool done = false;
-      while (!done) {
-        // one round trip fetches a window of 256 predecessors (4 per lane)
-        uint32_t v[4];
-        unsigned spins = 0;
-        for (;;) {
-          bool missing = false;
-#pragma unroll
-          for (int r = 0; r < 4; r++) {
-            const int j = idx - 64 * r - (int)lane;
-            v[r] = j >= 0 ? ld_status(&status[j]) : kFlagPre;  // before the first tile: prefix 0
-            missing |= (v[r] >> 30) == 0u;
-          }
-          if (__ballot(missing) == 0ull) break;
-          if (++spins > spin_limit) {
-            // give up: report it through *nnz, then go on with what is there so that
-            // the grid drains (offsets stay below n, the output is garbage)
-            if (lane == 0) {
-              atomicOr(&ws[1], 1u);
-              atomicMin(nnz, -1);
-              __threadfence();
-            }
-#pragma unroll
-            for (int r = 0; r < 4; r++) v[r] |= kFlagPre;
-            break;
-          }
-          __builtin_amdgcn_s_sleep(1);
-        }
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          if (!done) {
-            const unsigned long long pre = __ballot((v[r] >> 30) == 2u);
-            unsigned take = 64;  // lanes 0..take-1 of this row contribute
-            if (pre) { take = (unsigned)__builtin_ctzll(pre) + 1u; done = true; }
-            unsigned contrib = lane < take ? (v[r] & kValMask) : 0u;
-            excl += (unsigned)wave_sum((int)contrib);
-          }
-        }
-        idx -= 256;
+      for (int r = 0; r < 4; r++) {
+        const int t = t0 + 4 * (int)lane + r;
+        v[r] = t < stop ? ld_status(&status[t]) : kTileReady;
+        missing |= (v[r] & kTileReady) == 0u;
       }
-      if (lane == 0) st_status(&status[tile], kFlagPre | ((excl + tile_agg) & kValMask));
+      if (__ballot(missing) == 0ull) break;
+      if (++spins > spin_limit) {  // give up: report it through *nnz; the offsets that follow are garbage below n
+        if (lane == 0) {
+          atomicOr(&ws[1], 1u);
+          atomicMin(nnz, -1);
+        }
+        break;
+      }
+      __builtin_amdgcn_s_sleep(4);
     }
-    if (lane == 0) s_tile = excl;
-  }
-  __syncthreads();
-  unsigned off = s_tile;
+    unsigned c[4], mine = 0;
 #pragma unroll
-  for (int w = 0; w < WAVES; w++) off += w < wv ? s_agg[w] : 0u;
+    for (int r = 0; r < 4; r++) {
+      c[r] = v[r] & ~kTileReady;
+      mine += c[r];
+    }
+    const unsigned incl = wave_inclusive_scan(mine);
+    unsigned run = carry + incl - mine;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int t = t0 + 4 * (int)lane + r;
+      if (t < stop) st_status(&offset[t], kTileReady | run);
+      run += c[r];
+    }
+    carry += (unsigned)__builtin_amdgcn_readlane((int)incl, 63);
+  }
+  if (lane == 0) atomicMin(nnz, (int)carry);
+}
 
-  if (!in_layout) return;
-  uint32_t* mrow = mask + (size_t)c * g.W;
-  if (!has_data) {  // chunk without data: the reference leaves these words untouched; define them
-    for (int w = lane; w < g.W; w += 64) mrow[w] = 0;
+template <bool HINT>
+__global__ __launch_bounds__(64 * kSWaves) void zvc_stream_kernel(
+    const float* __restrict__ in, StreamGeometry g, uint32_t* __restrict__ ws, int* __restrict__ begin,
+    int* __restrict__ nnz, float* __restrict__ values, uint32_t* __restrict__ mask, unsigned spin_limit,
+    unsigned skip_first)
+{
+  __shared__ __attribute__((aligned(16))) float stage[kSTileElems + 8];
+  __shared__ unsigned s_cnt[kSSlots][kSWaves];
+  const int G = (int)gridDim.x - 1, w = (int)blockIdx.x;
+  if (w == G) {
+    zvc_stream_scanner(ws, g.tiles, G, nnz, spin_limit);
     return;
   }
-  if (lane == 0) {
-    begin[c] = (int)off;
-    if (c == g.active - 1) atomicMin(nnz, (int)(off + agg));
-  }
+  const unsigned lane = lane_id();
+  const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  uint32_t* status = ws + 16;
+  const uint32_t* offset = ws + 16 + g.tiles;
+  const int iters = (g.tiles - w + G - 1) / G;  // >= 1: the grid has no more data workgroups than there are tiles
+  // chunk index = half row / W by multiply and shift (exact while half rows * W < 2^40)
+  const unsigned long long w_magic = ((1ull << 40) + (unsigned)g.E / 32u - 1) / ((unsigned)g.E / 32u);
 
-  // ---- phase 2: mask words and packed values from the registers
-  uint32_t held = 0;
+  float x[kSSlots][kSRows];
+  unsigned woff[kSSlots];   // non-zeros of the workgroup's tile in the wavefronts before mine
+  unsigned total[kSSlots];  // non-zeros of the workgroup's tile
+  // The registers of a slot hold what the loads brought, also for rows that do not exist; `have[slot]`
+  // says how many elements do, and whoever looks at the values applies it (a select right after the
+  // load would be a use of the value and would make the load's latency part of the stage that issued it).
+  int have[kSSlots];
+  uint32_t ov = 0;          // the offset word of the workgroup's next tile, once it has arrived (every
+                            // wavefront reads it for itself: one more branch-free load per stage)
+
+  // Where my rows of tile t start, as a base that is the same for the whole wavefront and
+  // the number of elements that exist from there on (0..768).  Rows that do not exist -- past
+  // the end of the tensor, tiles past the last one -- are read from the start of the tensor
+  // instead and ignored: every wavefront issues the same loads on every path, so that the
+  // compiler's count of loads in flight is exact and a wait for one tile does not also wait
+  // for the tile whose loads were issued after it.
+  auto rows_of = [&](int t, const float*& base, int& exist) {
+    const long long first = ((long long)t * kSTileRows + wv * kSRows) * 64;
+    long long left = (long long)g.n - first;
+    left = left < 0 ? 0 : (left > kSRows * 64 ? kSRows * 64 : left);
+    exist = (int)left;
+    base = in + (left > 0 ? first : 0);
+  };
+  auto count_tile = [&](const float (&src)[kSRows], int slot) {
+    unsigned cnt = 0;
+    if (have[slot] == kSRows * 64) {
 #pragma unroll
-  for (int t = 0; t < IT; t++) {
-    if (t < iters) {
-      const bool nz = x[t] != 0.0f;
-      const unsigned long long m = __ballot(nz);
-      if (nz) values[off + rank_below(m)] = x[t];
-      off += popc64(m);
-      const unsigned slot = (unsigned)(2 * t) & 63u;
-      if (lane == slot) held = (uint32_t)m;
-      if (lane == slot + 1) held = (uint32_t)(m >> 32);
-      if ((t & 31) == 31 || t == iters - 1) {
-        const int w = (t >> 5) * 64 + (int)lane;
-        const int filled = 2 * (t & 31) + 2;
-        if ((int)lane < filled && w < g.W) mrow[w] = held;
-        held = 0;
+      for (int j = 0; j < kSRows; j++) cnt += popc64(__ballot(src[j] != 0.0f));
+    } else {
+#pragma unroll
+      for (int j = 0; j < kSRows; j++) cnt += popc64(__ballot(src[j] != 0.0f && (int)lane < have[slot] - 64 * j));
+    }
+    if (lane == 0) s_cnt[slot][wv] = cnt;
+  };
+  // after the barrier that follows count_tile: my offset inside the tile and the tile's total; wave 0 publishes it
+  auto share_counts = [&](int slot, int t, bool exists) {
+    const unsigned mine = lane < (unsigned)kSWaves ? s_cnt[slot][lane] : 0u;
+    const unsigned incl = wave_inclusive_scan(mine);
+    total[slot] = (unsigned)__builtin_amdgcn_readlane((int)incl, kSWaves - 1);
+    woff[slot] = (unsigned)__builtin_amdgcn_readlane((int)(incl - mine), wv);
+    if (wv == 0 && exists && lane == 0 && !(skip_first && t == 0)) st_status(&status[t], kTileReady | total[slot]);
+  };
+  // waits (bounded) until the scanner has published the offset of tile t
+  auto await_offset = [&](int t) {
+    unsigned spins = 0;
+    while ((ov & kTileReady) == 0u) {
+      if (++spins > spin_limit) {
+        // give up: report it through *nnz and go on with what is there, so that every
+        // workgroup still reaches its end (offsets stay below n, the output is garbage)
+        if (lane == 0) {
+          atomicOr(&ws[1], 1u);
+          atomicMin(nnz, -1);
+        }
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
+      ov = ld_status(&offset[t]);
+    }
+  };
+  // what the write-out of a tile needs, kept from its scatter to the next stage
+  unsigned out_prefix = 0, out_total = 0;
+  uint32_t out_held = 0;
+  int out_begin_idx = -1, out_begin_val = 0;
+  long long out_word = 0;
+  unsigned prev_prefix = 0, prev_total = 0;
+  auto write_out = [&](unsigned tile_prefix, unsigned tile_total) {
+    const unsigned shift = tile_prefix & 3u;
+    const unsigned end = shift + tile_total;           // stage slots [shift, end) hold data
+    float* base = values + (tile_prefix - shift);      // 16-byte aligned
+    for (unsigned q = threadIdx.x; 4u * q < end; q += 64 * kSWaves) {
+      const stream_f4 v = *reinterpret_cast<const stream_f4*>(stage + 4u * q);
+      float* dst = base + 4u * q;
+      if (4u * q >= shift && 4u * q + 4u <= end) {
+        if (HINT) __builtin_nontemporal_store(v, reinterpret_cast<stream_f4*>(dst));
+        else *reinterpret_cast<stream_f4*>(dst) = v;
+      } else {  // the first and the last group of a tile are shared with its neighbours
+        if (4u * q + 0u >= shift && 4u * q + 0u < end) dst[0] = v.x;
+        if (4u * q + 1u >= shift && 4u * q + 1u < end) dst[1] = v.y;
+        if (4u * q + 2u >= shift && 4u * q + 2u < end) dst[2] = v.z;
+        if (4u * q + 3u >= shift && 4u * q + 3u < end) dst[3] = v.w;
       }
     }
+    if (lane < 2u * kSRows && out_word < (long long)g.mask_words) mask[out_word] = out_held;
+    if (out_begin_idx >= 0) begin[out_begin_idx] = out_begin_val;
+  };
+
+  // ---- fill the pipeline: four tiles on their way, the first three counted and published
+  {
+    const float* base;
+    int exist;
+#pragma unroll
+    for (int k = 0; k < kSAhead; k++) {
+      rows_of(w + k * G, base, exist);
+      have[k] = exist;
+#pragma unroll
+      for (int j = 0; j < kSRows; j++) x[k][j] = base[min(lane + 64u * j, (unsigned)max(exist - 1, 0))];
+    }
   }
+#pragma unroll
+  for (int k = 0; k < kSAhead - 1; k++) count_tile(x[k], k);
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kSAhead - 1; k++) share_counts(k, w + k * G, k < iters);
+  ov = ld_status(&offset[w]);
+
+  for (int i0 = 0; i0 < iters; i0 += kSSlots) {
+#pragma unroll
+    for (int s = 0; s < kSSlots; s++) {
+      const int i = i0 + s;
+      if (i >= iters) break;
+      const int t = i * G + w;
+      // ---- this tile's offset was asked for a stage ago; ask for the next one
+      await_offset(t);
+      out_prefix = ov & ~kTileReady;
+      out_total = total[s];
+      // ---- the previous tile leaves
+      if (i > 0) write_out(prev_prefix, prev_total);
+      prev_prefix = out_prefix;
+      prev_total = out_total;
+      __syncthreads();
+      ov = ld_status(&offset[i + 1 < iters ? t + G : t]);
+      // ---- non-zeros of this tile into the LDS stage, one row at a time, and after each row the
+      // load of the same row of the tile four ahead, so that the requests to memory are spread
+      // over the whole stage instead of arriving in a burst
+      {
+        const int r0 = t * kSTileRows + wv * kSRows;  // my first row
+        unsigned at = (out_prefix & 3u) + woff[s];    // stage slot of the next non-zero
+        const unsigned at0 = at;
+        uint32_t held = 0;
+        const float* base;
+        int exist;
+        rows_of(t + kSAhead * G, base, exist);
+        have[(s + kSAhead) % kSSlots] = exist;
+        const unsigned last = (unsigned)max(exist - 1, 0);
+        // the same loop twice: with every row of both tiles there (nearly always), and with the checks
+        // for rows that are not; both issue the same twelve loads
+        if (have[s] == kSRows * 64 && exist == kSRows * 64) {
+#pragma unroll
+          for (int j = 0; j < kSRows; j++) {
+            const float v = x[s][j];
+            const bool nz = v != 0.0f;
+            const unsigned long long m = __ballot(nz);
+            const unsigned slot =
+                __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, at));
+            if (nz) stage[slot] = v;
+            at += popc64(m);
+            if (lane == 2u * j) held = (uint32_t)m;
+            if (lane == 2u * j + 1u) held = (uint32_t)(m >> 32);
+            x[(s + kSAhead) % kSSlots][j] = base[lane + 64u * j];
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < kSRows; j++) {
+            const float v = x[s][j];
+            const bool nz = v != 0.0f && (int)lane < have[s] - 64 * j;
+            const unsigned long long m = __ballot(nz);
+            const unsigned slot =
+                __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, at));
+            if (nz) stage[slot] = v;
+            at += popc64(m);
+            if (lane == 2u * j) held = (uint32_t)m;
+            if (lane == 2u * j + 1u) held = (uint32_t)(m >> 32);
+            x[(s + kSAhead) % kSSlots][j] = base[min(lane + 64u * j, last)];
+          }
+        }
+        // lane k < 32 holds mask word k of my rows = half row 2*r0 + k; a chunk starts there
+        // if the half row index is a multiple of W
+        const unsigned in_word = (unsigned)__popc(held);
+        const unsigned before = wave_inclusive_scan(in_word) - in_word;
+        const unsigned half = 2u * (unsigned)r0 + lane;
+        const unsigned c = (unsigned)(((unsigned long long)half * w_magic) >> 40);
+        const bool starts = lane < 2u * kSRows && c * ((unsigned)g.E / 32u) == half && (int)c < g.active;
+        out_begin_idx = starts ? (int)c : -1;
+        out_begin_val = (int)(out_prefix - (out_prefix & 3u) + at0 + before);
+        out_held = held;
+        out_word = (long long)r0 * 2 + lane;
+      }
+      // ---- the tile three ahead arrived during the previous stage: count it (in the same
+      // straight line as the loads above, so that the wait for it knows which loads are younger)
+      count_tile(x[(s + kSAhead - 1) % kSSlots], (s + kSAhead - 1) % kSSlots);
+      __syncthreads();
+      share_counts((s + kSAhead - 1) % kSSlots, t + (kSAhead - 1) * G, i + kSAhead - 1 < iters);
+    }
+  }
+  write_out(prev_prefix, prev_total);
 }
 
 // ------------------------------------------------------------------ probe
@@ -768,15 +936,67 @@ extern "C" int cswap_zvc_pick_process(size_t n)
   return p;
 }
 
+constexpr int kStatusWordsMin = 65536;
+// status words of a workspace for `process` chunks: one per chunk for the look-back kernel,
+// one per tile for the pipeline kernel, never fewer than 65536
+static int status_words(int process) { return process > kStatusWordsMin ? process : kStatusWordsMin; }
+
 extern "C" size_t cswap_zvc_workspace_bytes(int process)
 {
-  return process > 0 ? ((size_t)process + 16) * sizeof(uint32_t) : 0;
+  return process > 0 ? ((size_t)status_words(process) + 16) * sizeof(uint32_t) : 0;
 }
 
-extern "C" void cswap_zvc_debug_set_lookback(unsigned spin_limit, unsigned first_ticket)
+extern "C" void cswap_zvc_debug_set_lookback(unsigned spin_limit, unsigned skip_first)
 {
   g_spin_limit = spin_limit ? spin_limit : kSpinLimit;
-  g_first_ticket = first_ticket;
+  g_skip_first = skip_first;
+}
+
+// compute units of the current device (0 if the query fails), looked up once per device
+static int device_compute_units()
+{
+  static int cus[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (!cus[dev]) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cus[dev] = v;
+  }
+  return cus[dev];
+}
+
+static int status_words(int process);
+// Tensors of at least this many bytes take the single pass in cswap_zvc_compress_fused; smaller ones
+// finish sooner with the three kernels (a few rounds of the grid do not fill the pipeline).
+static unsigned long long g_single_pass_bytes = 128ull << 20;  // cswap_zvc_set_single_pass_bytes
+
+extern "C" size_t cswap_zvc_set_single_pass_bytes(size_t bytes)
+{
+  const size_t before = (size_t)g_single_pass_bytes;
+  g_single_pass_bytes = bytes;
+  return before;
+}
+
+// whether the single pass takes a tensor of this shape; fills its geometry
+static bool single_pass_shape(const Geometry& g, int n, int process, StreamGeometry& sg)
+{
+  sg.n = n; sg.E = g.E; sg.process = process; sg.active = g.active;
+  const long long mask_words = (long long)g.W * process;
+  sg.mask_words = (int)mask_words;
+  sg.rows = (int)((mask_words + 1) / 2);
+  sg.tiles = (sg.rows + kSTileRows - 1) / kSTileRows;
+  // whole half rows per chunk, two status words per tile in the workspace, a compute unit for
+  // every workgroup, and a tensor large enough to fill the pipeline
+  return g.E % 32 == 0 && mask_words < (1ll << 31) - 64 && 2 * sg.tiles <= status_words(process) &&
+         device_compute_units() > 1 && 4ull * (unsigned long long)n >= g_single_pass_bytes;
+}
+
+extern "C" int cswap_zvc_takes_single_pass(int n, int process)
+{
+  Geometry g;
+  StreamGeometry sg;
+  return make_geometry(g, n, process) == CSWAP_OK && single_pass_shape(g, n, process, sg);
 }
 
 extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, void* d_ws, int* d_begin,
@@ -786,24 +1006,23 @@ extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, v
   Geometry g;
   int rc = make_geometry(g, n, process);
   if (rc) return rc;
-  // chunks that do not fit a wavefront's registers, or prefixes that do not fit
-  // the 30-bit status value, take the three-kernel path
-  if (g.E > 64 * 128 || n >= (1 << 30)) return cswap_zvc_compress(d_in, n, process, d_begin, d_nnz, d_values, d_mask, stream);
   uint32_t* ws = (uint32_t*)d_ws;
-  const int words = process + 16;
+  const int cus = device_compute_units();
+  StreamGeometry sg;
+  // anything the single pass does not take, or an output that is not 16-byte aligned, runs the three kernels
+  const bool single_pass = single_pass_shape(g, n, process, sg) && (reinterpret_cast<uintptr_t>(d_values) & 15u) == 0;
+  if (!single_pass) return cswap_zvc_compress(d_in, n, process, d_begin, d_nnz, d_values, d_mask, stream);
+  // one workgroup per compute unit, the last of them the scanner
+  const int data_groups = sg.tiles < cus - 1 ? sg.tiles : cus - 1;
+  const int words = 2 * sg.tiles + 16;
   hipLaunchKernelGGL(zvc_ws_zero_kernel, dim3((words + 255) / 256), dim3(256), 0, (hipStream_t)stream, ws, words,
-                     (uint32_t)g_first_ticket, d_nnz);
-  const int iters = (g.E + 63) >> 6;
-#define CSWAP_FUSED(IT_, WAVES_)                                                                          \
-  hipLaunchKernelGGL((zvc_fused_kernel<IT_, WAVES_>), dim3((g.process + WAVES_ - 1) / WAVES_),            \
-                     dim3(64 * WAVES_), 0, (hipStream_t)stream, d_in, g, ws, d_begin, d_nnz, d_values, d_mask,   \
-                     g_spin_limit)
-  if (iters <= 8) CSWAP_FUSED(8, 16);
-  else if (iters <= 16) CSWAP_FUSED(16, 16);
-  else if (iters <= 32) CSWAP_FUSED(32, 16);
-  else if (iters <= 64) CSWAP_FUSED(64, 8);
-  else CSWAP_FUSED(128, 8);
-#undef CSWAP_FUSED
+                     d_nnz);
+  if (4ull * (unsigned long long)n >= g_staged_compact_bytes)
+    hipLaunchKernelGGL(zvc_stream_kernel<true>, dim3(data_groups + 1), dim3(64 * kSWaves), 0, (hipStream_t)stream,
+                       d_in, sg, ws, d_begin, d_nnz, d_values, d_mask, g_spin_limit, g_skip_first);
+  else
+    hipLaunchKernelGGL(zvc_stream_kernel<false>, dim3(data_groups + 1), dim3(64 * kSWaves), 0, (hipStream_t)stream,
+                       d_in, sg, ws, d_begin, d_nnz, d_values, d_mask, g_spin_limit, g_skip_first);
   return check_launch();
 }
 

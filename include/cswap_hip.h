@@ -159,25 +159,37 @@ int cswap_zvc_expand(const float* d_values, const uint32_t* d_mask, const int* d
 int cswap_zvc_compress(const float* d_in, int n, int process, int* d_begin, int* d_nnz,
                        float* d_values, uint32_t* d_mask, cswap_stream_t stream);
 
-/* The same result in a single pass over the tensor (each wavefront keeps its
- * chunk in registers and finds its offset by a decoupled look-back), so HBM
- * traffic is the algorithmic 4 + 1/8 + 4*density bytes per element.  d_ws is
- * scratch of cswap_zvc_workspace_bytes(process) bytes, cleared by the call
- * itself; calls that share a workspace must not overlap.  Tensors whose chunks
- * exceed 8192 elements (n > 8192*process) fall back to the three-kernel path.
- * A wavefront waits for the offsets of the chunks before its own; that wait is
- * bounded, and if it ever runs out the kernel still finishes but *d_nnz is -1
+/* The same result in a single pass over the tensor: resident workgroups walk the
+ * tensor tile by tile, keep the tiles they have loaded in registers until a
+ * scanner workgroup has turned the published tile counts into offsets, and then
+ * write mask, offsets and packed values, so HBM traffic is the algorithmic
+ * 4 + 1/8 + 4*density bytes per element.  Smaller tensors than
+ * cswap_zvc_set_single_pass_bytes says run the three kernels, which finish sooner there.  d_ws is scratch of cswap_zvc_workspace_bytes(process) bytes (at
+ * least 256 KiB), cleared by the call itself; calls that share a workspace must
+ * not overlap.  Shapes the single pass does not take -- a chunk length that is not
+ * a multiple of 32, d_values not 16-byte aligned, more than 32768 tiles of 12288
+ * elements -- run the three kernels instead.  The workgroups wait for each other's
+ * counts; that wait is bounded, and if it ever runs out (for example because the
+ * kernel does not get the whole GPU) the kernel still finishes but *d_nnz is -1
  * and the other outputs are undefined: a caller must treat a negative count as
  * failure (the return value cannot tell, the call does not synchronise). */
 size_t cswap_zvc_workspace_bytes(int process);
 int cswap_zvc_compress_fused(const float* d_in, int n, int process, void* d_ws, int* d_begin,
                              int* d_nnz, float* d_values, uint32_t* d_mask, cswap_stream_t stream);
+/* 1 if cswap_zvc_compress_fused would run the single pass for this shape (given a
+ * 16-byte aligned d_values), 0 if it would run the three kernels.  Host only. */
+int cswap_zvc_takes_single_pass(int n, int process);
+/* No counterpart in the reference: the tensor size in bytes from which
+ * cswap_zvc_compress_fused runs the single pass (default 128 MiB: below that the
+ * three kernels finish sooner; 0 = whenever the shape allows, SIZE_MAX = never).
+ * Returns the previous value.  Process-wide. */
+size_t cswap_zvc_set_single_pass_bytes(size_t bytes);
 /* For tests of that failure path only.  spin_limit: how many times a wavefront
- * re-reads the status words it waits for before it gives up (0 = the default,
- * about four million); first_ticket: the first piece of work handed out, so that
- * with 1 the first piece is never done and every later one waits in vain.
- * Process-wide; (0, 0) restores normal operation. */
-void cswap_zvc_debug_set_lookback(unsigned spin_limit, unsigned first_ticket);
+ * asks again for a status word it waits for before it gives up (0 = the default,
+ * about a million); skip_first: if not 0 the count of the first tile is never
+ * published, so that everything after it waits in vain.  Process-wide; (0, 0)
+ * restores normal operation. */
+void cswap_zvc_debug_set_lookback(unsigned spin_limit, unsigned skip_first);
 /* No counterpart in the reference.  cswap_zvc_compress_fused for callers that
  * cannot allocate a workspace (code under HIP graph capture, serving loops and
  * harnesses that forbid hipMalloc): the status words live in a static device

@@ -654,3 +654,37 @@ def test_two_threads_share_one_engine(torch_cuda):
     assert not any(t.is_alive() for t in threads)
     assert not errors, errors[:5]
     eng.close()
+
+
+@pytest.mark.parametrize("device_pool_mib", [320, 200])
+def test_large_zvc_request_takes_the_single_pass(torch_cuda, device_pool_mib):
+    """An explicit ZVC request for a 256 MiB tensor is compressed in one pass over the
+    tensor into a staging block of the worst-case size, cut back once the count is
+    known; without room for the worst case (the 200 MiB pool) the probe path runs
+    instead.  Same payload, same round trip either way."""
+    torch = torch_cuda
+    from cswap_amd import swap
+    from cswap_amd._lib import lib
+
+    n = 64 << 20
+    g = torch.Generator(device="cuda"); g.manual_seed(21)
+    x = torch.relu(torch.randn(n, generator=g, device="cuda")).reshape(64, 64, 128, 128)
+    nnz = int((x != 0).sum().item())
+    eng = swap.SwapEngine(pinned_bytes=256 << 20, device_bytes=device_pool_mib << 20)
+    try:
+        process = eng.process_for(n)
+        assert lib().cswap_zvc_takes_single_pass(n, process) == 1
+        for rep in range(2):
+            print("pool", device_pool_mib, "rep", rep, flush=True)
+            tk = eng.pre(x, swap.SPARSE)
+            eng.post(tk)
+            info = eng.info(tk)
+            assert info.policy == swap.SPARSE and info.nnz == nnz
+            assert info.bytes_out == 4 * nnz + n // 8 + 4 * process
+            out = torch.full_like(x, -1.0)
+            eng.swap_in(tk, out)
+            torch.cuda.synchronize()
+            eng.release(tk)
+            assert torch.equal(out, x)
+    finally:
+        eng.close()

@@ -15,6 +15,32 @@ def torch_cuda():
     return torch
 
 
+@pytest.fixture(scope="module", autouse=True)
+def single_pass_at_any_size():
+    """cswap_zvc_compress_fused runs its single pass only from 128 MiB on (the three
+    kernels finish sooner below); the tests here want it on small shapes too."""
+    from cswap_amd._lib import lib
+
+    before = lib().cswap_zvc_set_single_pass_bytes(0)
+    yield
+    lib().cswap_zvc_set_single_pass_bytes(before)
+
+
+def test_size_rule_of_the_single_pass():
+    from cswap_amd._lib import lib
+
+    L = lib()
+    assert L.cswap_zvc_takes_single_pass(P * 64, P) == 1          # forced on for this module
+    mine = L.cswap_zvc_set_single_pass_bytes(128 << 20)
+    try:
+        assert L.cswap_zvc_takes_single_pass(P * 512, P) == 0      # 32 MiB: three kernels
+        assert L.cswap_zvc_takes_single_pass(P * 2048, P) == 1     # 128 MiB
+        assert L.cswap_zvc_takes_single_pass(P * 4096 + 5, P) == 0  # chunk length 4097: not whole half rows
+        assert L.cswap_zvc_takes_single_pass(1 << 30, 1024) == 0   # more tiles than the workspace has words for
+    finally:
+        L.cswap_zvc_set_single_pass_bytes(mine)
+
+
 @pytest.fixture(params=["by_size", "staged"])
 def compact_form(request):
     """Both forms of cswap_zvc_compact: the one its size rule picks (row-wise stores at
@@ -131,6 +157,31 @@ def test_fused_single_pass_ragged(torch_cuda, n, process):
     check_against_oracle(x, run_gpu(torch_cuda, x, process, fused=True), process)
 
 
+@pytest.mark.parametrize("n,process", [
+    (P * 32, P),                 # one chunk per half row, 128 tiles: fewer tiles than compute units
+    (P * 32 - 3205, P),          # the same with a hundred idle chunks and a partial row at the end
+    (P * 32 * 3 - 45, P),        # chunks of 96 elements: they start on rows and on half rows
+    (P * 512 - 1, P),            # 8 Mi elements, the last row one short
+    (P * 4128 - 5000, P),        # 4128-element chunks: more than one round of the grid
+    (P * 2048 - 10_000, P),      # several idle chunks
+    (1024 * 16384, 1024),        # one chunk = one tile
+    (999 * 160 - 37, 999),       # an odd number of mask words in all
+    (64 * 2048 - 13, 64), (992, 1), (32, 1), (4096, 8)])
+def test_single_pass_pipeline_kernel(torch_cuda, n, process):
+    """Shapes the pipeline form of the single-pass compression accepts (chunk length a
+    multiple of 32, at most 16384): grids smaller and larger than the number of tiles,
+    partial rows, chunks that start in the middle of a row, idle chunks."""
+    import oracle
+
+    E, W, K = oracle.zvc_geometry(n, process)
+    assert E % 32 == 0 and E <= 16384
+    rng = np.random.default_rng(n % 977 + process)
+    zeros = rng.uniform(0.2, 0.9)
+    x = (rng.standard_normal(n, dtype=np.float32) * (rng.random(n, dtype=np.float32) > zeros)).astype(np.float32)
+    print("n", n, "process", process, "E", E, flush=True)
+    check_against_oracle(x, run_gpu(torch_cuda, x, process, fused=True), process)
+
+
 def test_fused_repeated_calls_share_a_workspace(torch_cuda):
     """The workspace is cleared by every call: back-to-back calls on one stream
     with the same scratch buffer give the same result."""
@@ -155,11 +206,11 @@ def test_fused_repeated_calls_share_a_workspace(torch_cuda):
 
 
 def test_fused_reports_a_wait_that_ran_out(torch_cuda):
-    """The single-pass kernel's wait for the chunks before it is bounded.  Forced
-    from the host: the first piece of work is never handed out and the bound is a
-    few re-reads, so every later piece gives up at once, every kernel still exits
-    normally, and the caller sees nnz == -1 instead of made-up offsets.  The next
-    call, with the defaults back, is correct again."""
+    """The single-pass kernel's waits for the counts of other workgroups are bounded.
+    Forced from the host: the count of the first tile is never published and the bound
+    is a few re-reads, so whoever waits for it gives up at once, every kernel still
+    exits normally, and the caller sees nnz == -1 instead of made-up offsets.  The
+    next call, with the defaults back, is correct again."""
     torch = torch_cuda
     from cswap_amd import api
     from cswap_amd._lib import check, lib

@@ -38,7 +38,10 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
     assert torch.cuda.is_available(), "this test needs the GPU"
     L = lib()
     g = torch.Generator(device="cuda"); g.manual_seed(11)
-    for n, process in ((P * 512 + 77, P), (P * 40 - 3, P), (300_001, 7)):   # later calls are smaller
+    size_rule = L.cswap_zvc_set_single_pass_bytes(0)     # the single pass (the kernel that uses the scratch) at any size
+    # later calls are smaller; the last shape is one the single pass does not take
+    for n, process in ((P * 512 - 77, P), (P * 64 - 3, P), (300_001, 7)):
+        assert L.cswap_zvc_takes_single_pass(n, process) == (process == P)
         x = torch.relu(torch.randn(n, generator=g, device="cuda"))
         print("static entry point: n", n, "process", process, flush=True)
         want = _run(torch, L, x, process, static=False)
@@ -47,6 +50,7 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
         for a, b in zip(got[1:], want[1:]):
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
         assert np.array_equal(got[1], x[x != 0].cpu().numpy())
+    L.cswap_zvc_set_single_pass_bytes(size_rule)
     # beyond the static array: refused, nothing launched
     x = torch.zeros(1 << 20, device="cuda")
     big = 65536 * 2
