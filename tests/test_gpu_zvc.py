@@ -43,8 +43,9 @@ def test_size_rule_of_the_single_pass():
 
 @pytest.fixture(params=["by_size", "staged"])
 def compact_form(request):
-    """Both forms of cswap_zvc_compact: the one its size rule picks (row-wise stores at
-    these sizes) and the LDS-staged one, forced for inputs of any size."""
+    """Both forms of cswap_zvc_compact and of the 16-byte-store expansion: the one the
+    size rule picks (no LDS staging at these sizes) and the LDS-staged one, forced for
+    inputs of any size."""
     from cswap_amd._lib import lib
 
     if request.param == "by_size":
@@ -112,8 +113,10 @@ def test_other_chunk_counts(torch_cuda, compact_form, process):
 
 @pytest.mark.parametrize("n,process", [(P * 8 - 3, P), (P * 260 - 1, P), (P * 512 - 2, P), (P * 2052 - 7, P),
                                         (P * 4096 - 254, P), (28, 7), (5000, 1), (299_992, 7), (64 * 2048, 64)])
-def test_expand_four_per_lane(torch_cuda, n, process):
-    """Chunk lengths that are multiples of four take the 16-byte-store expansion;
+def test_expand_four_per_lane(torch_cuda, compact_form, n, process):
+    """Chunk lengths that are multiples of four take the 16-byte-store expansion
+    (both of its forms: values fetched straight from global memory, and staged in
+    LDS as for tensors beyond the cache size, which `compact_form` forces);
     the sizes end the last chunk inside a quad, inside a row and inside a refill
     group.  The same data is then expanded into a destination that is only
     4-byte aligned, which takes the per-element kernel: both must agree."""
