@@ -90,7 +90,8 @@ def main():
     ap.add_argument("--swap-only", action="store_true",
                     help="run only the swap schedule of configuration 4 and its backward walk (for profiling)")
     ap.add_argument("--zvc-only", action="store_true",
-                    help="run only the 256 MiB ReLU zero-value-compaction case (for profiling); prints its figures")
+                    help="run only one ReLU zero-value-compaction case (for profiling); prints its figures")
+    ap.add_argument("--zvc-mib", type=int, default=256, help="size of the --zvc-only tensor in MiB")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; run with --gpus 1 "
@@ -107,7 +108,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.zvc_only:
-        print(json.dumps(extras(torch, api, dev, zvc_only=True)))
+        print(json.dumps(extras(torch, api, dev, zvc_only=args.zvc_mib)))
         return
     if args.swap_only:
         from cswap_amd import swap
@@ -329,7 +330,8 @@ def zfp_library_pair(sample, maxbits):
     return best
 
 
-def zvc_extras(torch, api, dev, ex, config2_tensor, only_256=False):
+def zvc_extras(torch, api, dev, ex, config2_tensor, only_mib=0):
+    only_256 = bool(only_mib)
     # ---- ZVC compact / expand / probe
     def zvc_case(label, t):
         n = t.numel()
@@ -403,6 +405,9 @@ def zvc_extras(torch, api, dev, ex, config2_tensor, only_256=False):
         for mib in (1, 4, 16, 32, 128):
             geometry_case(mib)
     g = torch.Generator(device=dev); g.manual_seed(1)
+    if only_mib and only_mib != 256:
+        zvc_case(f"relu_{only_mib}MiB", torch.relu(torch.randn(only_mib << 18, generator=g, device=dev)))
+        return ex
     zvc_case("relu_256MiB", torch.relu(torch.randn(64 * 1024 * 1024, generator=g, device=dev)))
     # twice the size: mask and values (286 MB) no longer stay in the 256 MB memory-side cache
     # between the launches of a timing loop, as the 143 MB of the case above do
@@ -411,14 +416,14 @@ def zvc_extras(torch, api, dev, ex, config2_tensor, only_256=False):
     return ex
 
 
-def extras(torch, api, dev, zvc_only=False):
+def extras(torch, api, dev, zvc_only=0):
     import numpy as np
 
     from cswap_amd.workloads import config1_field, config2_tensor, field_dims
 
     ex = {}
     if zvc_only:
-        return zvc_extras(torch, api, dev, ex, config2_tensor, only_256=True)
+        return zvc_extras(torch, api, dev, ex, config2_tensor, only_mib=zvc_only)
     # ---- ZFP at other rates and on configuration 1
     g = torch.Generator(device=dev); g.manual_seed(0)
     big = torch.softmax(torch.randn((32, 12, 512, 512), generator=g, device=dev), dim=-1).contiguous()
