@@ -434,19 +434,23 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand4_kernel(
 }
 
 // The same once more for tensors larger than the memory-side cache (the size from which
-// the compaction is staged, too): the packed values of eight rows (2048 elements) are first
+// the compaction is staged, too): the packed values of four rows (1024 elements) are first
 // brought into an LDS region of the wavefront with aligned 16-byte loads -- whole lines per
-// instruction -- and picked from there.  Fetching them one by one from global memory, four
-// partly filled load instructions per row, is 6 % slower where the values come from HBM
-// (512 MiB: 0.168 against 0.178 ms) and the same where they come from the cache; on small
-// tensors the 33 KB of LDS per workgroup cost more occupancy than the loads gain
-// (32 MiB: 15.7 against 10.9 us), so those keep the kernel above.
+// instruction -- and picked from there, and the mask words of the next eight rows are asked
+// for while the current eight are expanded.  Fetching the values one by one from global
+// memory, four partly filled load instructions per row, is 15 % slower where they come from
+// HBM (512 MiB: 0.151 against 0.178 ms; staging eight rows at a time 0.167, two 0.163: less
+// LDS per wavefront means more wavefronts per compute unit to hide the two loads each group
+// waits for, fewer rows per group means more groups) and the same where they come from the
+// cache; on small tensors the LDS costs more occupancy than the loads gain, so those keep
+// the kernel above.
+constexpr int kRowsStaged = 4;  // divides kRowsInFlight
 
 __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand4_staged_kernel(
     const float* __restrict__ values, const uint32_t* __restrict__ mask, const int* __restrict__ begin,
     Geometry g, float* __restrict__ out)
 {
-  __shared__ __attribute__((aligned(16))) float lds_all[kWavesPerGroup][256 * kRowsInFlight + 8];
+  __shared__ __attribute__((aligned(16))) float lds_all[kWavesPerGroup][256 * kRowsStaged + 8];
   const int c = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
   if (c >= g.active) return;
   float* lds = lds_all[threadIdx.x >> 6];
@@ -459,11 +463,12 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand4_staged_kernel
   const int rows = (len + 255) >> 8;
   const unsigned sub = lane & 7u;  // my nibble inside the word I read
   const uint32_t below = (1u << (4u * sub)) - 1u;
+  uint32_t held_next = (int)lane < g.W ? mrow[lane] : 0u;
   for (int r0 = 0; r0 < rows; r0 += kRowsInFlight) {
-    uint32_t held, pre;  // pre: low half = set bits before my word in its row, high half = through it
-    {  // refill: 64 words = 8 rows
+    uint32_t held = held_next, pre;  // pre: low half = set bits before my word in its row, high half = through it
+    {  // 64 words = 8 rows; the next 64 are asked for now
       const int w = (r0 >> 3) * 64 + (int)lane;
-      held = w < g.W ? mrow[w] : 0u;
+      held_next = w + 64 < g.W ? mrow[w + 64] : 0u;
       const int first = w * 32;  // bits past the end of the chunk carry no data
       if (first + 32 > len) held = first >= len ? 0u : (held & ((1u << (len - first)) - 1u));
       const uint32_t cnt = (uint32_t)__popc(held);
@@ -475,55 +480,58 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand4_staged_kernel
       }
       pre = (s - cnt) | (s << 16);
     }
-    // where each row's values start inside the group, and how many the group has
-    unsigned row_start[kRowsInFlight], total = 0;
 #pragma unroll
-    for (int j = 0; j < kRowsInFlight; j++) {
-      row_start[j] = total;
-      total += (uint32_t)__builtin_amdgcn_readlane((int)pre, (j << 3) + 7) >> 16;
-    }
-    // values[off, off + total) to lds[shift ...] with loads aligned in global memory (shift = off % 4);
-    // the last group of four is fetched element by element so that nothing past the values is read
-    const unsigned shift = off & 3u;
-    const float* src = values + (off - shift);
-    const unsigned end = shift + total;
-    lds_order();  // the picks of the previous group are done
-    for (unsigned k = 4u * lane; k < end; k += 256u) {
-      if (k + 4u <= end) {
-        *reinterpret_cast<float4*>(lds + k) = *reinterpret_cast<const float4*>(src + k);
-      } else {
-        for (unsigned e = k; e < end; e++) lds[e] = src[e];
+    for (int h = 0; h < kRowsInFlight; h += kRowsStaged) {
+      // where each row's values start inside the group of four, and how many the group has
+      unsigned row_start[kRowsStaged], total = 0;
+#pragma unroll
+      for (int j = 0; j < kRowsStaged; j++) {
+        row_start[j] = total;
+        total += (uint32_t)__builtin_amdgcn_readlane((int)pre, ((h + j) << 3) + 7) >> 16;
       }
-    }
-    lds_order();
-    float4 x[kRowsInFlight];
+      // values[off, off + total) to lds[shift ...] with loads aligned in global memory (shift = off % 4);
+      // the last group of four is fetched element by element so that nothing past the values is read
+      const unsigned shift = off & 3u;
+      const float* src = values + (off - shift);
+      const unsigned end = shift + total;
+      lds_order();  // the picks of the previous group are done
+      for (unsigned k = 4u * lane; k < end; k += 256u) {
+        if (k + 4u <= end) {
+          *reinterpret_cast<float4*>(lds + k) = *reinterpret_cast<const float4*>(src + k);
+        } else {
+          for (unsigned e = k; e < end; e++) lds[e] = src[e];
+        }
+      }
+      lds_order();
+      float4 x[kRowsStaged];
 #pragma unroll
-    for (int j = 0; j < kRowsInFlight; j++) {
-      const int from = (j << 3) + (int)(lane >> 3);
-      const uint32_t w = (uint32_t)__shfl((int)held, from, 64);
-      const uint32_t p = (uint32_t)__shfl((int)pre, from, 64);
-      const uint32_t nib = (w >> (4u * sub)) & 15u;
-      unsigned rk = shift + row_start[j] + (p & 0xffffu) + (unsigned)__popc(w & below);
-      float4 v;
-      v.x = (nib & 1u) ? lds[rk] : 0.0f;
-      rk += nib & 1u;
-      v.y = (nib & 2u) ? lds[rk] : 0.0f;
-      rk += (nib >> 1) & 1u;
-      v.z = (nib & 4u) ? lds[rk] : 0.0f;
-      rk += (nib >> 2) & 1u;
-      v.w = (nib & 8u) ? lds[rk] : 0.0f;
-      x[j] = v;
-    }
-    off += total;
+      for (int j = 0; j < kRowsStaged; j++) {
+        const int from = ((h + j) << 3) + (int)(lane >> 3);
+        const uint32_t w = (uint32_t)__shfl((int)held, from, 64);
+        const uint32_t p = (uint32_t)__shfl((int)pre, from, 64);
+        const uint32_t nib = (w >> (4u * sub)) & 15u;
+        unsigned rk = shift + row_start[j] + (p & 0xffffu) + (unsigned)__popc(w & below);
+        float4 v;
+        v.x = (nib & 1u) ? lds[rk] : 0.0f;
+        rk += nib & 1u;
+        v.y = (nib & 2u) ? lds[rk] : 0.0f;
+        rk += (nib >> 1) & 1u;
+        v.z = (nib & 4u) ? lds[rk] : 0.0f;
+        rk += (nib >> 2) & 1u;
+        v.w = (nib & 8u) ? lds[rk] : 0.0f;
+        x[j] = v;
+      }
+      off += total;
 #pragma unroll
-    for (int j = 0; j < kRowsInFlight; j++) {
-      const int k = (r0 + j) * 256 + 4 * (int)lane;
-      if (k + 4 <= len) {
-        st_stream4(reinterpret_cast<float4*>(q + k), x[j]);
-      } else {  // ragged end of the last chunk
-        if (k < len) q[k] = x[j].x;
-        if (k + 1 < len) q[k + 1] = x[j].y;
-        if (k + 2 < len) q[k + 2] = x[j].z;
+      for (int j = 0; j < kRowsStaged; j++) {
+        const int k = (r0 + h + j) * 256 + 4 * (int)lane;
+        if (k + 4 <= len) {
+          st_stream4(reinterpret_cast<float4*>(q + k), x[j]);
+        } else {  // ragged end of the last chunk
+          if (k < len) q[k] = x[j].x;
+          if (k + 1 < len) q[k + 1] = x[j].y;
+          if (k + 2 < len) q[k + 2] = x[j].z;
+        }
       }
     }
   }
