@@ -688,3 +688,37 @@ def test_large_zvc_request_takes_the_single_pass(torch_cuda, device_pool_mib):
             assert torch.equal(out, x)
     finally:
         eng.close()
+
+
+def test_engine_falls_back_when_the_single_pass_gives_up(torch_cuda):
+    """The single pass reports a wait that ran out through a negative count (forced here
+    from the host, as in test_gpu_zvc.py: every kernel still exits normally); the
+    engine then compresses the tensor with the probe path and the swap is as good."""
+    torch = torch_cuda
+    from cswap_amd import swap
+    from cswap_amd._lib import lib
+
+    L = lib()
+    n = 48 << 20                                       # 192 MiB
+    g = torch.Generator(device="cuda"); g.manual_seed(22)
+    x = torch.relu(torch.randn(n, generator=g, device="cuda")).reshape(48, 64, 128, 128)
+    nnz = int((x != 0).sum().item())
+    eng = swap.SwapEngine(pinned_bytes=256 << 20, device_bytes=320 << 20)
+    try:
+        assert L.cswap_zvc_takes_single_pass(n, eng.process_for(n)) == 1
+        L.cswap_zvc_debug_set_lookback(4, 1)
+        try:
+            print("forced give-up inside the engine", flush=True)
+            tk = eng.pre(x, swap.SPARSE)
+        finally:
+            L.cswap_zvc_debug_set_lookback(0, 0)
+        eng.post(tk)
+        info = eng.info(tk)
+        assert info.policy == swap.SPARSE and info.nnz == nnz
+        out = torch.full_like(x, -1.0)
+        eng.swap_in(tk, out)
+        torch.cuda.synchronize()
+        eng.release(tk)
+        assert torch.equal(out, x)
+    finally:
+        eng.close()
