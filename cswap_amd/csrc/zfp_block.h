@@ -76,6 +76,19 @@ CSWAP_HD int ctz64(uint64_t v)  // 64 for v == 0
 #endif
 }
 
+// count of trailing zeros of a 32-bit word; some value >= 32 for v == 0 (the
+// device instruction gives 0xffffffff, which callers only compare and clamp)
+CSWAP_HD unsigned ctz32_or_more(uint32_t v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  unsigned t;
+  asm("v_ffbl_b32 %0, %1" : "=v"(t) : "v"(v));
+  return t;
+#else
+  return v ? (unsigned)__builtin_ctz(v) : 0xffffffffu;
+#endif
+}
+
 CSWAP_HD uint64_t low_mask(unsigned n)  // n in 0..64
 {
   return n >= 64 ? ~(uint64_t)0 : (((uint64_t)1 << n) - 1);
@@ -378,7 +391,7 @@ CSWAP_HD void settle(uint64_t& v)
 #endif
 }
 
-CSWAP_HD void settle32(uint32_t& v)
+CSWAP_HD void settle32(unsigned& v)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
   asm volatile("" : "+v"(v));
@@ -688,7 +701,7 @@ CSWAP_HD void encode_block_w64(const uint64_t (&q)[64], unsigned pos0, unsigned 
 
 // ---------------------------------------------------------------- decoder
 // mem.ld32(dword_index) reads the bit region; positions are absolute within it
-// and the block owns [pos0, pos0 + maxbits).  Reads may run up to 96 bits past
+// and the block owns [pos0, pos0 + maxbits).  Reads may run up to 128 bits past
 // the end of the block (the values are never used).
 // FENCED: the caller guarantees that the bit right after the block reads as one.
 // A run of zeros that the bit budget cuts short then ends at that bit by itself,
@@ -697,9 +710,9 @@ template <class Mem, int SIZE = 64, bool FENCED = false>
 struct BlockDecoder {
   Mem& mem;
   unsigned pos, limit;
-  unsigned n;
+  int nrem;  // SIZE - 1 - (coefficients already known significant): -1 once all of them are
 
-  CSWAP_HD BlockDecoder(Mem& m, unsigned pos0, unsigned maxbits) : mem(m), pos(pos0), limit(pos0 + maxbits), n(0) {}
+  CSWAP_HD BlockDecoder(Mem& m, unsigned pos0, unsigned maxbits) : mem(m), pos(pos0), limit(pos0 + maxbits), nrem(SIZE - 1) {}
 
   CSWAP_HD bool active() const { return pos < limit; }
 
@@ -717,8 +730,14 @@ struct BlockDecoder {
   // already in registers: the first one sits right behind the verbatim bits, the
   // one after a run right behind the run's terminating one-bit, so the step loop
   // turns once per positive test and not at all for a plane that adds nothing.
+  //
+  // A turn of the step loop looks at 32 stream bits.  That is enough when the run
+  // ends, or the coefficients run out, within 30 bits (the next group test is then
+  // inside the window as well); when some block of the wavefront needs more, the
+  // turn is redone on 64 bits for all of them.
   CSWAP_HD uint64_t plane()
   {
+    const unsigned n = (unsigned)(SIZE - 1 - nrem);
     unsigned left = sub_sat(limit, pos);
     unsigned m = n < left ? n : left;
     uint64_t w = window(pos);
@@ -726,31 +745,47 @@ struct BlockDecoder {
     settle(above);                                // one shift serves the verbatim mask and the group test
     uint64_t x = w ^ (m < 64 ? above << m : 0);   // the low m bits of w
     pos += m;
-    bool go = n < SIZE && pos < limit;            // a group test follows (then m = n < 64)
+    bool go = nrem >= 0 && pos < limit;           // a group test follows (then m = n < 64)
     bool test = go && ((uint32_t)above & 1u);
     pos += go ? 1u : 0u;
-    while (test) {                                // positive group test: a run of zeros, then a one
-      w = window(pos);
-      settle(w);
-      unsigned maxrun = SIZE - 1 - n;
-      if (!FENCED) {
-        unsigned avail = limit - pos;
-        maxrun = maxrun < avail ? maxrun : avail;
-      }
-      unsigned t = (unsigned)ctz64(w);
-      bool found = t < maxrun;  // t zeros then a one; else ran into the last position or the budget
-      unsigned r = found ? t : maxrun;
-      pos += r + (found ? 1u : 0u);  // FENCED and out of budget: "finds" the fence, pos = limit + 1
-      n += r;
-      x |= (uint64_t)1 << n;
-      n++;
-      // not found: n == SIZE or the budget is spent, either way the plane is over;
-      // found: t <= 62, so the next group test (bit t + 1) is still inside this window.
-      // (found also implies n < SIZE here; leaving the comparison out makes the compiler
-      // emit 46 more instructions per wavefront, so it stays)
-      go = found && n < SIZE && pos < limit;
-      test = go && ((uint32_t)(w >> ((t + 1) & 63)) & 1u);
-      pos += go ? 1u : 0u;
+    if (test) {                                   // positive group test: a run of zeros, then a one
+      unsigned d = dword_of(pos);
+      uint32_t w0 = mem.ld32(d), w1 = mem.ld32(d + 1);
+      do {
+        uint32_t lo = funnel_shr(w1, w0, pos);
+        unsigned maxrun = (unsigned)nrem;         // the run cannot pass the last coefficient
+        if (!FENCED) {
+          unsigned avail = limit - pos;
+          maxrun = maxrun < avail ? maxrun : avail;
+        }
+        unsigned t = ctz32_or_more(lo);           // at least 32 when the window holds no one-bit
+        unsigned r = t < maxrun ? t : maxrun;
+        uint32_t after = lo >> (t & 31);          // bit 0: the one that ended the run, bit 1: the next group test
+        if (CSWAP_ANY(r > 30)) {
+          const uint32_t w2 = mem.ld32(d + 2);
+          const uint64_t w64 = ((uint64_t)funnel_shr(w2, w1, pos) << 32) | lo;
+          t = (unsigned)ctz64(w64);
+          r = t < maxrun ? t : maxrun;
+          after = (uint32_t)(w64 >> (t & 63));
+        }
+        // If there is another turn, it starts behind the one-bit and the group test
+        // that follow these t zeros: its window is asked for now, so that the read
+        // is under way while the rest of this turn is worked out.
+        d = dword_of(pos + t + 2);
+        w0 = mem.ld32(d);
+        w1 = mem.ld32(d + 1);
+        const bool found = t < maxrun;  // t zeros then a one; else ran into the last position or the budget
+        pos += r + (found ? 1u : 0u);   // FENCED and out of budget: "finds" the fence, pos = limit + 1
+        settle32(pos);                  // (this sum and the one below are one add-with-carry each; merged they are four)
+        nrem -= (int)r;
+        x |= ((uint64_t)1 << (SIZE - 1)) >> nrem;
+        nrem--;
+        // not found: every coefficient is significant now or the budget is spent, either way the
+        // plane is over; found: t <= 62, so the next group test is bit 1 of `after`
+        go = found && nrem >= 0 && pos < limit;
+        test = go && (after & 2u);
+        pos += go ? 1u : 0u;
+      } while (test);
     }
     return x;
   }
@@ -801,17 +836,39 @@ CSWAP_HD uint32_t decode_planes32(Dec& dec, uint32_t (&lo)[32], uint32_t (&hi)[3
 
 // Integer back end of a 4x4x4 block up to and including the inverse lifting
 // along z and y (decode.cuh:127-179 and the first two passes of :181-226).
+// inv_lift4 on inputs that still carry the negabinary constant (X = x + c and so
+// on, mod 2^32): only w has to be freed of it before its shift; y drops it in the
+// three-input add that follows, z + x drops both at once and x - z never had it.
+CSWAP_HD void inv_lift4_biased(int32_t& x, int32_t& y, int32_t& z, int32_t& w, uint32_t c)
+{
+  const uint32_t X = (uint32_t)x, Y = (uint32_t)y, Z = (uint32_t)z;
+  w = (int32_t)((uint32_t)w - c);
+  y = (int32_t)(Y + (uint32_t)(w >> 1) + (0u - c));
+  w = wsub(w, y >> 1);
+  z = (int32_t)(Z + X + (0u - 2u * c));
+  x = (int32_t)(X - Z);
+  { int32_t y0 = y; y = wadd(y, w); w = wsub(w, y0); }
+  { int32_t y0 = y; y = wadd(y, z); z = wsub(z, y0); }
+  { int32_t w0 = w; w = wadd(w, x); x = wsub(x, w0); }
+}
+
 template <class Dec>
 CSWAP_HD void decode_ints3_zy(Dec& dec, int32_t (&ib)[64])
 {
   uint32_t lo[32], hi[32];
   const uint32_t c = decode_planes32(dec, lo, hi);
 #pragma unroll
-  for (int i = 0; i < 32; i++) {
-    ib[kPerm3.v[i]] = (int32_t)(lo[i] - c);
-    ib[kPerm3.v[32 + i]] = (int32_t)(hi[i] - c);
+  for (int i = 0; i < 32; i++) {  // still with the negabinary constant added: the z pass takes it out
+    ib[kPerm3.v[i]] = (int32_t)lo[i];
+    ib[kPerm3.v[32 + i]] = (int32_t)hi[i];
   }
-  inv_xform3_zy(ib);
+#pragma unroll
+  for (int i = 0; i < 16; i++) inv_lift4_biased(ib[i], ib[i + 16], ib[i + 32], ib[i + 48], c);
+#pragma unroll
+  for (int z = 0; z < 4; z++)
+#pragma unroll
+    for (int x = 0; x < 4; x++)
+      inv_lift4(ib[16 * z + x], ib[16 * z + x + 4], ib[16 * z + x + 8], ib[16 * z + x + 12]);
 }
 
 // int64 coefficients: the high words from the first 32 planes, the low words from

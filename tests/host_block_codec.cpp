@@ -16,7 +16,7 @@ struct ArrayBits {            // the bit region is the whole stream, addressed i
 
 extern "C" {
 
-// stream must hold ceil(blocks*maxbits/64)+2 zeroed words (the codec may touch 96 bits past a block)
+// stream must hold ceil(blocks*maxbits/64)+2 zeroed words (the codec may touch 128 bits past a block)
 void host_zfp_encode3(const float* in, size_t nx, size_t ny, size_t nz, unsigned maxbits, uint64_t* stream)
 {
   size_t mx = (nx + 3) / 4, my = (ny + 3) / 4, mz = (nz + 3) / 4;
