@@ -432,7 +432,7 @@ CSWAP_HD uint32_t funnel_shr(uint32_t hi, uint32_t lo, unsigned s)  // ({hi,lo} 
 // mem.or32(dword_index, value); bit positions are absolute within that region.
 // The block owns [pos0, pos0 + maxbits).  GUARD = true cuts every write at the
 // end of the block (needed when the next block's bits follow immediately);
-// GUARD = false lets the last plane spill up to 96 bits past the end, which the
+// GUARD = false lets the last plane spill up to 128 bits past the end, which the
 // caller must provide as slack and ignore.
 template <class Mem, bool GUARD, int SIZE = 64>
 struct BlockEncoder {
@@ -475,8 +475,13 @@ struct BlockEncoder {
     put(n < 64 ? x ^ (rest << n) : x, n);
     if (n < SIZE) {
       bool more = true;
-      while (rest != 0 && more && pos < limit) {
-        unsigned t1 = (unsigned)ctz64(rest) + 1;  // zeros before the next one-bit, and that bit
+      // Without the guard a block that runs out of budget inside this loop simply goes
+      // on to the end of the plane: what it writes past its end (less than 128 bits) lands
+      // in the slack and is dropped.
+      while (rest != 0 && more && (!GUARD || pos < limit)) {
+        unsigned t1;  // zeros before the next one-bit, and that bit
+        if (CSWAP_ANY((uint32_t)rest == 0)) t1 = (unsigned)ctz64(rest) + 1;
+        else t1 = ctz32_or_more((uint32_t)rest) + 1;
         unsigned q = pos + t1;
         n += t1;
         more = n < SIZE;                     // a one-bit at the last position is implied, not written

@@ -65,7 +65,7 @@ __host__ __device__ inline unsigned slot_bits(unsigned maxbits)
 }
 __host__ __device__ inline unsigned region_dwords(unsigned maxbits)
 {
-  return ((2u * slot_bits(maxbits) + 4u) + 3u) & ~3u;  // + padding for the 96-bit over-read / over-write
+  return ((2u * slot_bits(maxbits) + 4u) + 3u) & ~3u;  // + padding for the 128-bit over-read / over-write
 }
 
 // ------------------------------------------------------------- block <-> field

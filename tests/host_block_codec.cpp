@@ -33,6 +33,35 @@ void host_zfp_encode3(const float* in, size_t nx, size_t ny, size_t nz, unsigned
   }
 }
 
+// Same encode through the unguarded variant: every block is coded into a private,
+// zeroed slot of maxbits + 128 bits, as the device does for whole-word rates, and
+// only its first maxbits bits are kept.  Returns the highest dword index (relative
+// to the slot) that any block wrote a non-zero value to.
+unsigned host_zfp_encode3_slots(const float* in, size_t nx, size_t ny, size_t nz, unsigned maxbits, uint64_t* stream)
+{
+  size_t mx = (nx + 3) / 4, my = (ny + 3) / 4, mz = (nz + 3) / 4;
+  const unsigned W = maxbits / 64;  // maxbits % 64 == 0
+  const unsigned slot_dwords = 2 * W + 4 + 8;  // 8 more so that a write past the 128 bits of slack is seen, not a crash
+  uint32_t* slot = new uint32_t[slot_dwords];
+  unsigned top = 0;
+  for (size_t b = 0; b < mx * my * mz; b++) {
+    size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
+    unsigned bx = nx - x0 < 4 ? nx - x0 : 4, by = ny - y0 < 4 ? ny - y0 : 4, bz = nz - z0 < 4 ? nz - z0 : 4;
+    float f[64];
+    for (int i = 0; i < 64; i++) f[i] = 0.0f;
+    for (unsigned z = 0; z < bz; z++) for (unsigned y = 0; y < by; y++) for (unsigned x = 0; x < bx; x++)
+      f[x + 4 * y + 16 * z] = in[(x0 + x) + nx * ((y0 + y) + ny * (z0 + z))];
+    if (bx < 4 || by < 4 || bz < 4) cswap::pad_block3(f, bx, by, bz);
+    memset(slot, 0, 4 * (size_t)slot_dwords);
+    ArrayBits mem{slot};
+    cswap::encode_block<false>(f, 0u, maxbits, mem);
+    memcpy(stream + b * W, slot, 8 * (size_t)W);
+    for (unsigned d = 0; d < slot_dwords; d++) if (slot[d] && d > top) top = d;
+  }
+  delete[] slot;
+  return top;
+}
+
 void host_zfp_decode3(const uint64_t* stream, size_t nx, size_t ny, size_t nz, unsigned maxbits, float* out)
 {
   size_t mx = (nx + 3) / 4, my = (ny + 3) / 4, mz = (nz + 3) / 4;

@@ -23,6 +23,8 @@ def host():
     L.host_zfp_encode3.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     L.host_zfp_decode3.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     L.host_zfp_decode3_fenced.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
+    L.host_zfp_encode3_slots.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
+    L.host_zfp_encode3_slots.restype = C.c_uint
     L.host_transpose32.argtypes = [C.c_void_p]
     L.host_zfp_encode_low.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     L.host_zfp_decode_low.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
@@ -81,6 +83,11 @@ def test_block_codec_matches_golden_vectors(host, golden):
         k = min(sb.size, stream.size)
         assert np.array_equal(sb[:k], stream[:k]), (name, rate)
         assert not sb[k:].any() and not stream[k:].any()
+        if maxbits % 64 == 0:  # the encoder variant the device uses for whole-word rates
+            s2 = np.zeros(words, dtype=np.uint64)
+            top = host.host_zfp_encode3_slots(f.ctypes.data, nx, ny, nz, maxbits, s2.ctypes.data)
+            assert np.array_equal(s2.view(np.uint8)[:k], stream[:k]), (name, rate, "slots")
+            assert top < maxbits // 32 + 4, (name, rate, "wrote past the 128 bits of slack")
         g = np.zeros((words + 2) * 8, dtype=np.uint8)
         g[:k] = stream[:k]
         o = np.zeros_like(f)
@@ -198,3 +205,24 @@ def test_64_bit_block_codec_agrees_with_checker_on_tiny_and_huge_doubles(host):
             host.host_zfp_decode_w64(s.ctypes.data, 0, 3, 4, 8, 4, maxbits, o.ctypes.data)
             d = oracle.zfp_decode_64(want, f.shape, maxbits, np.float64)
             assert np.array_equal(o.view(np.uint64), d.view(np.uint64)), (scale, maxbits)
+
+
+def test_unguarded_encoder_stays_inside_its_slack(host):
+    """The encoder variant without end-of-block guards lets a block that runs out
+    of budget finish its bit plane.  On noise, where a plane that starts with few
+    significant coefficients finds many at once, what it writes past the block's
+    end must stay within the 128 bits of slack, and the kept bits must equal the
+    guarded encoder's."""
+    rng = np.random.default_rng(11)
+    for maxbits in (64, 128, 192, 256, 512):
+        for scale in (1.0, 1e-3, 1e4):
+            f = (rng.standard_normal((8, 16, 64)) * scale).astype(np.float32)
+            f[rng.random(f.shape) < 0.1] *= 1e3          # a few outliers: leading planes with long runs
+            nz, ny, nx = f.shape
+            words = (nx // 4) * (ny // 4) * (nz // 4) * maxbits // 64
+            a = np.zeros(words + 2, dtype=np.uint64)
+            host.host_zfp_encode3(f.ctypes.data, nx, ny, nz, maxbits, a.ctypes.data)
+            b = np.zeros(words, dtype=np.uint64)
+            top = host.host_zfp_encode3_slots(f.ctypes.data, nx, ny, nz, maxbits, b.ctypes.data)
+            assert np.array_equal(a[:words], b), (maxbits, scale)
+            assert top < maxbits // 32 + 4, (maxbits, scale, top)
