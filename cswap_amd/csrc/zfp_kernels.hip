@@ -41,16 +41,26 @@ typedef float stream_f4 __attribute__((ext_vector_type(4)));
 typedef unsigned long long stream_u2 __attribute__((ext_vector_type(2)));
 
 // ------------------------------------------------------------- LDS adapter
-// The bit region the block codec ORs into / reads from is LDS, addressed in
-// dwords: it serves as the dynamically indexable extension of the register
-// file (a lane cannot index its registers with a run-time bit position).
+// The bit region the block codec ORs into / reads from is LDS: it serves as the
+// dynamically indexable extension of the register file (a lane cannot index
+// its registers with a run-time bit position).  The codec hands over the byte
+// offset of a dword as the LDS address itself, so bit positions count from LDS
+// address 0: a block's first bit is bit0 + its offset within the region.  (With
+// a pointer to the region plus an offset, every access would cost one more
+// instruction that adds the region's address.)
+typedef __attribute__((address_space(3))) uint32_t lds_u32;
 struct LdsBits {
-  uint32_t* lds;
+  unsigned bit0;  // bit position of the region's first bit
+  __device__ __forceinline__ explicit LdsBits(uint32_t* region)
+      : bit0(8u * (unsigned)(size_t)(__attribute__((address_space(3))) void*)region)
+  {
+  }
+  __device__ __forceinline__ static lds_u32* at(unsigned d) { return (lds_u32*)(size_t)d; }
   __device__ __forceinline__ void or32(unsigned d, uint32_t v) const
   {
-    __hip_atomic_fetch_or(&lds[d], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);  // ds_or_b32
+    __hip_atomic_fetch_or(at(d), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);  // ds_or_b32
   }
-  __device__ __forceinline__ uint32_t ld32(unsigned d) const { return lds[d]; }
+  __device__ __forceinline__ uint32_t ld32(unsigned d) const { return *at(d); }
 };
 
 // Layout of the wave's LDS bit region.
@@ -270,14 +280,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void
   __syncthreads();
 
   if (lane < valid) {
-    LdsBits mem{lds};
+    LdsBits mem(lds);
     if (INT) {
       int32_t v[64];
 #pragma unroll
       for (int i = 0; i < 64; i++) v[i] = __float_as_int(f[i]);
-      encode_block_i32<!WHOLE>(v, lane * slot, maxbits, mem);
+      encode_block_i32<!WHOLE>(v, mem.bit0 + lane * slot, maxbits, mem);
     } else {
-      encode_block<!WHOLE>(f, lane * slot, maxbits, mem);
+      encode_block<!WHOLE>(f, mem.bit0 + lane * slot, maxbits, mem);
     }
   }
   __syncthreads();
@@ -305,12 +315,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void
   if (lane < valid) {
     int32_t ib[64];
     float w;
-    LdsBits mem{lds};
+    LdsBits mem(lds);
     if (INT) {
       w = 0.0f;
-      decode_block_i32_zy<WHOLE>(mem, lane * slot, maxbits, ib);
+      decode_block_i32_zy<WHOLE>(mem, mem.bit0 + lane * slot, maxbits, ib);
     } else {
-      decode_block_zy<WHOLE>(mem, lane * slot, maxbits, ib, w);
+      decode_block_zy<WHOLE>(mem, mem.bit0 + lane * slot, maxbits, ib, w);
     }
     // block coordinates and addresses are worked out only now, from a lane id
     // that is recomputed here and tied to a decoded value: otherwise they (or
@@ -410,8 +420,8 @@ __global__ __launch_bounds__(64) void zfp_encode3_w64_kernel(const uint64_t* __r
   zero_region(lds_raw, lane, maxbits);
   __syncthreads();
   if (lane < valid) {
-    LdsBits mem{lds};
-    encode_block_w64<!WHOLE, INT>(q, lane * slot_bits(maxbits), maxbits, mem);
+    LdsBits mem(lds);
+    encode_block_w64<!WHOLE, INT>(q, mem.bit0 + lane * slot_bits(maxbits), maxbits, mem);
   }
   __syncthreads();
   store_region<WHOLE>(lds, lane, first, valid, maxbits, fd.stream16, stream);
@@ -431,8 +441,8 @@ __global__ __launch_bounds__(64) void zfp_decode3_w64_kernel(const uint64_t* __r
   __syncthreads();
   if (lane < valid) {
     uint64_t q[64];
-    LdsBits mem{lds};
-    decode_block_w64<INT, WHOLE>(mem, lane * slot_bits(maxbits), maxbits, q);
+    LdsBits mem(lds);
+    decode_block_w64<INT, WHOLE>(mem, mem.bit0 + lane * slot_bits(maxbits), maxbits, q);
     store_block_w64<ONCE>(out, fd, first + lane, q);
   }
 }
@@ -502,8 +512,8 @@ __global__ __launch_bounds__(64) void zfp_encode_low_f32_kernel(const float* __r
   if (lane < valid) {
     float f[16];
     load_block_low<DIMS>(in, fd, first + lane, f);
-    LdsBits mem{lds};
-    encode_block_low<DIMS, true, INT>(f, lane * maxbits, maxbits, mem);
+    LdsBits mem(lds);
+    encode_block_low<DIMS, true, INT>(f, mem.bit0 + lane * maxbits, maxbits, mem);
   }
   __syncthreads();
   const unsigned nwords = (valid * maxbits + 63u) >> 6;
@@ -528,8 +538,8 @@ __global__ __launch_bounds__(64) void zfp_decode_low_f32_kernel(const uint64_t* 
   __syncthreads();
   if (lane < valid) {
     float f[16];
-    LdsBits mem{lds};
-    decode_block_low<DIMS, INT>(mem, lane * maxbits, maxbits, f);
+    LdsBits mem(lds);
+    decode_block_low<DIMS, INT>(mem, mem.bit0 + lane * maxbits, maxbits, f);
     store_block_low<DIMS>(out, fd, first + lane, f);
   }
 }
@@ -567,8 +577,8 @@ __global__ __launch_bounds__(64) void zfp_encode_low_w64_kernel(const uint64_t* 
 #pragma unroll
       for (int x = 0; x < 4; x++) pad4(q[x], q[x + 4], q[x + 8], q[x + 12], by);
     }
-    LdsBits mem{lds};
-    encode_block_low_w64<DIMS, true, INT>(q, lane * maxbits, maxbits, mem);
+    LdsBits mem(lds);
+    encode_block_low_w64<DIMS, true, INT>(q, mem.bit0 + lane * maxbits, maxbits, mem);
   }
   __syncthreads();
   const unsigned nwords = (valid * maxbits + 63u) >> 6;
@@ -593,8 +603,8 @@ __global__ __launch_bounds__(64) void zfp_decode_low_w64_kernel(const uint64_t* 
   __syncthreads();
   if (lane < valid) {
     uint64_t q[16];
-    LdsBits mem{lds};
-    decode_block_low_w64<DIMS, INT>(mem, lane * maxbits, maxbits, q);
+    LdsBits mem(lds);
+    decode_block_low_w64<DIMS, INT>(mem, mem.bit0 + lane * maxbits, maxbits, q);
     const uint32_t b = first + lane;
     const uint32_t r = b / fd.mx;
     const uint32_t x0 = (b - r * fd.mx) * 4, y0 = DIMS == 2 ? r * 4 : 0;

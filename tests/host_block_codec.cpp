@@ -7,10 +7,10 @@
 #include "../cswap_amd/csrc/zfp_block.h"
 
 namespace {
-struct ArrayBits {            // the bit region is the whole stream, addressed in dwords
+struct ArrayBits {            // the bit region is the whole stream, addressed by the byte offset of a dword
   uint32_t* dw;
-  void or32(unsigned d, uint32_t v) const { dw[d] |= v; }
-  uint32_t ld32(unsigned d) const { return dw[d]; }
+  void or32(unsigned d, uint32_t v) const { dw[d / 4] |= v; }
+  uint32_t ld32(unsigned d) const { return dw[d / 4]; }
 };
 }
 
