@@ -796,20 +796,41 @@ struct BlockDecoder {
         d = dword_of(pos + t + 2);
         w0 = mem.ld32(d);
         w1 = mem.ld32(d + 4);
-        const bool found = t < maxrun;  // t zeros then a one; else ran into the last position or the budget
+        // found: t zeros, then a one; else the run reached the last position or the budget.
+        // With the fence the run is only ever cut by the coefficients that are left, so
+        // "found" is the same as "coefficients are left after this one": the carry of the
+        // decrement below says it, and no comparison of its own is needed.
+        unsigned left_after = (unsigned)nrem - r;
+        x |= ((uint64_t)1 << (SIZE - 1)) >> left_after;
+        unsigned dec;  // left_after - 1, written as an addition so that the carry is "some are left"
+        const bool some_left = __builtin_uadd_overflow(left_after, 0xffffffffu, &dec);
+        nrem = (int)dec;
+        const bool found = FENCED ? some_left : t < maxrun;
         pos += r + (found ? 1u : 0u);   // FENCED and out of budget: "finds" the fence, pos = limit + 1
         settle32(pos);                  // (this sum and the one below are one add-with-carry each; merged they are four)
-        nrem -= (int)r;
-        x |= ((uint64_t)1 << (SIZE - 1)) >> nrem;
-        nrem--;
-        // not found: every coefficient is significant now or the budget is spent, either way the
-        // plane is over; found: t <= 62, so the next group test is bit 1 of `after`
-        go = found && nrem >= 0 && pos < limit;
+        // not found: the plane is over; found: t <= 62, so the next group test is bit 1 of `after`
+        go = found && some_left && pos < limit;
         test = go && (after & 2u);
         pos += go ? 1u : 0u;
       } while (test);
     }
     return x;
+  }
+
+  // One of the leading planes.  While no block of the wavefront has a significant
+  // coefficient, a plane that is empty in all of them is one zero bit per block
+  // (mirror of BlockEncoder::leading_plane).
+  CSWAP_HD uint64_t leading_plane()
+  {
+    if (!CSWAP_ANY(nrem != SIZE - 1)) {
+      const bool act = pos < limit;
+      const uint32_t bit = (mem.ld32(dword_of(pos)) >> (pos & 31)) & 1u;
+      if (!CSWAP_ANY(act && bit)) {
+        pos += act ? 1u : 0u;
+        return 0;
+      }
+    }
+    return plane();
   }
 };
 
@@ -830,7 +851,8 @@ CSWAP_HD uint32_t decode_planes32(Dec& dec, uint32_t (&lo)[32], uint32_t (&hi)[3
 {
 #pragma unroll
   for (int k = 31; k >= 16; k--) {  // planes that no block of the wavefront can reach are zero without a read
-    uint64_t x = CSWAP_ANY(dec.active()) ? dec.plane() : 0;
+    uint64_t x = 0;
+    if (CSWAP_ANY(dec.active())) x = k >= 28 ? dec.leading_plane() : dec.plane();
     lo[k] = (uint32_t)x;
     hi[k] = (uint32_t)(x >> 32);
   }
