@@ -347,9 +347,9 @@ def zvc_extras(torch, api, dev, ex, config2_tensor, only_mib=0):
         st = torch.cuda.current_stream().cuda_stream
         three = ev_ms(torch, lambda: L.cswap_zvc_compress(t.data_ptr(), n, api.PROCESS, begin.data_ptr(),
                                                           nnz.data_ptr(), values.data_ptr(), mask.data_ptr(), st), reps)
-        ws = torch.empty(L.cswap_zvc_workspace_bytes(api.PROCESS), dtype=torch.uint8, device=dev)
+        ws = api.zvc_workspace(api.PROCESS, dev)
         # count + scan + compact as one operation, as the swap engine runs it for a ZVC request: the
-        # single pass from 128 MiB on, the three kernels below
+        # single pass from 64 MiB on, the three kernels below
         full = ev_ms(torch, lambda: L.cswap_zvc_compress_fused(t.data_ptr(), n, api.PROCESS, ws.data_ptr(),
                                                                begin.data_ptr(), nnz.data_ptr(),
                                                                values.data_ptr(), mask.data_ptr(), st), reps)

@@ -105,6 +105,7 @@ _SIGNATURES = {
     "cswap_zvc_compress": (i32, [vp, i32, i32, vp, vp, vp, vp, vp]),
     "cswap_zvc_workspace_bytes": (sz, [i32]),
     "cswap_zvc_compress_fused": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp]),
+    "cswap_zvc_workspace_clear": (i32, [vp, i32, vp]),
     "cswap_zvc_debug_set_lookback": (None, [u, u]),
     "cswap_zvc_compress_fused_static": (i32, [vp, i32, i32, vp, vp, vp, vp, vp]),
     "cswap_probe_nnz": (i32, [vp, sz, vp, vp]),

@@ -153,7 +153,7 @@ def zvc_compress(t: torch.Tensor, process: int = PROCESS, fused: bool = False):
     begin = torch.zeros(process, dtype=torch.int32, device=dev)
     nnz = torch.zeros(1, dtype=torch.int32, device=dev)
     if fused:
-        ws = torch.empty(lib().cswap_zvc_workspace_bytes(process), dtype=torch.uint8, device=dev)
+        ws = zvc_workspace(process, dev)
         check(lib().cswap_zvc_compress_fused(t.data_ptr(), n, process, ws.data_ptr(), begin.data_ptr(),
                                              nnz.data_ptr(), values.data_ptr(), mask.data_ptr(), _stream()),
               "cswap_zvc_compress_fused")
@@ -161,6 +161,15 @@ def zvc_compress(t: torch.Tensor, process: int = PROCESS, fused: bool = False):
         check(lib().cswap_zvc_compress(t.data_ptr(), n, process, begin.data_ptr(), nnz.data_ptr(),
                                        values.data_ptr(), mask.data_ptr(), _stream()), "cswap_zvc_compress")
     return values, mask, begin, nnz
+
+
+def zvc_workspace(process: int = PROCESS, device=None) -> torch.Tensor:
+    """A workspace for the single-pass compression, allocated and prepared
+    (cswap_zvc_workspace_clear) on the current stream."""
+    ws = torch.empty(lib().cswap_zvc_workspace_bytes(process), dtype=torch.uint8,
+                     device=device if device is not None else torch.device("cuda"))
+    check(lib().cswap_zvc_workspace_clear(ws.data_ptr(), process, _stream()), "cswap_zvc_workspace_clear")
+    return ws
 
 
 def probe_nnz(t: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:

@@ -197,6 +197,8 @@ extern "C" int cswap_engine_create(cswap_engine** out, const cswap_engine_config
     if ((err = hipHostMalloc((void**)&e->h_nnz, 256, hipHostMallocDefault)) != hipSuccess) { fail(err); break; }
     if ((err = hipMalloc((void**)&e->d_nnz, 256)) != hipSuccess) { fail(err); break; }
     if ((err = hipMalloc(&e->d_ws, cswap_zvc_workspace_bytes(kWsProcess))) != hipSuccess) { fail(err); break; }
+    if ((rc = cswap_zvc_workspace_clear(e->d_ws, kWsProcess, nullptr)) != CSWAP_OK) break;
+    if ((err = hipStreamSynchronize(nullptr)) != hipSuccess) { fail(err); break; }
     if ((err = hipEventCreateWithFlags(&e->ev_probe, hipEventDisableTiming)) != hipSuccess) { fail(err); break; }
     e->hpool.reset(cfg.pinned_pool_bytes);
     e->dpool.reset(cfg.device_pool_bytes);
@@ -309,6 +311,7 @@ static int single_pass_sparse(cswap_engine* e, Ticket& t, const float* d_in, hip
   }
   if (*e->h_nnz < 0) {  // kernels have finished (the event): the block can go back at once
     e->dpool.free(off, worst);
+    (void)cswap_zvc_workspace_clear(e->d_ws, kWsProcess, compute);  // a failed run leaves the workspace unusable
     return 1;
   }
   t.nnz = (size_t)*e->h_nnz;

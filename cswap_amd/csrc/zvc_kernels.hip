@@ -545,13 +545,29 @@ constexpr unsigned kSpinLimit = 1u << 20;
 // cswap_zvc_debug_set_lookback: the bound of the waits, and whether tile 0 is never published
 static unsigned g_spin_limit = kSpinLimit, g_skip_first = 0;
 
-// Clears the workspace and arms *nnz: the scanner lowers it to the total with atomicMin, a
-// wait that ran out lowers it to -1, so -1 wins whichever comes first.
-__global__ void zvc_ws_zero_kernel(uint32_t* ws, int words, int* nnz)
+// Head of a workspace.  ws[0]: kWsMagic once cswap_zvc_workspace_clear has prepared it;
+// ws[1]: not 0 after a run whose bounded waits ran out (stays until the next clear, and
+// every run that finds it reports failure); ws[3]: number of runs whose scanner has
+// finished.  The status words proper start at ws[16].  A run that succeeds leaves them
+// zero again: whoever consumes a status word clears it.
+//
+// Who reports what.  The scanner is ahead of everybody else by two stages, so the
+// checks and the result are its business and cost the data workgroups nothing: it looks
+// at ws[0] and ws[1] when it starts, and when it has published the last offset it writes
+// *nnz (the total, or -1 if the flag is up by then) and only then steps ws[3].  A wavefront
+// whose wait ran out raises the flag at once; before it ends it waits (bounded) for ws[3]
+// to move and then writes -1 itself, so its -1 lands after whatever the scanner wrote, and
+// a scanner that is late finds the flag.  A workspace that is refused (never prepared, or
+// left behind by a failed run) makes the scanner write -1 and hand out offsets of zero, so
+// that every workgroup runs through without waiting; the data workgroups keep every offset
+// they are given inside the tensor, whatever the word held.
+constexpr uint32_t kWsMagic = 0x5a564331u;
+constexpr int kWsFlag = 1, kWsRuns = 3;
+
+__global__ void zvc_ws_clear_kernel(uint32_t* ws, int words)
 {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < words) ws[i] = 0u;
-  if (i == 0) *nnz = 0x7fffffff;
+  if (i < words) ws[i] = i == 0 ? kWsMagic : 0u;
 }
 
 __device__ __forceinline__ uint32_t ld_status(const uint32_t* p)
@@ -583,12 +599,15 @@ __device__ __forceinline__ void st_status(uint32_t* p, uint32_t v)
 // Needs: chunk length a multiple of 32 (the mask is then the flat bit mask and a chunk
 // starts on a half row), two status words per tile in the workspace, a 16-byte aligned
 // values pointer, and all G+1 workgroups resident at once (the waits are bounded).
-// Workspace, zero before the launch: ws[16 + t] = kTileReady | count of tile t,
-// ws[16 + tiles + t] = kTileReady | number of non-zeros before tile t.
+// Workspace (prepared once by cswap_zvc_workspace_clear; a run leaves it as it found it):
+// ws[16 + t] = kTileReady | count of tile t, ws[16 + tiles + t] = kTileReady | number of
+// non-zeros before tile t; the scanner clears a count when it has read it, a workgroup the
+// offsets of its tiles when it is through, so no launch is spent on clearing.
 //
 // Measured on one MI355X, half of the elements zero (this kernel / count + scan + compact):
-// 512 MiB 0.191 / 0.240 ms, 256 MiB 0.097 / 0.115 ms, 32 MiB 0.024 / 0.020 ms (a tensor of
-// a few rounds of the grid does not fill the pipeline).
+// 512 MiB 0.161 / 0.240 ms, 256 MiB 0.082 / 0.115 ms, 128 MiB 0.046 / 0.056, 64 MiB 0.031 /
+// 0.033, 32 MiB 0.021 / 0.020 ms (a tensor of a few rounds of the grid does not fill the
+// pipeline).
 constexpr int kSWaves = 16, kSRows = 12;
 constexpr int kSTileRows = kSWaves * kSRows, kSTileElems = kSTileRows * 64;
 constexpr int kSSlots = 5;   // tiles of a workgroup in registers
@@ -623,15 +642,18 @@ __device__ void zvc_stream_scanner(uint32_t* ws, int tiles, int step, int* nnz, 
   const unsigned lane = lane_id();
   uint32_t* status = ws + 16;
   uint32_t* offset = ws + 16 + tiles;
+  const uint32_t magic = ld_status(&ws[0]), flag0 = ld_status(&ws[kWsFlag]);
+  const bool refused = magic != kWsMagic || flag0 != 0u;
+  if (refused && lane == 0) *nnz = -1;
   unsigned carry = 0;
   // `step` tiles at a time (at most 256): the tiles that the data workgroups count in the same
   // stage, so that a step never waits for a count that is published a stage later than the rest
   for (int t0 = 0; t0 < tiles; t0 += step) {
     // lane l owns tiles t0 + 4l .. t0 + 4l + 3
     const int stop = t0 + step < tiles ? t0 + step : tiles;
-    uint32_t v[4];
+    uint32_t v[4] = {kTileReady, kTileReady, kTileReady, kTileReady};
     unsigned spins = 0;
-    for (;;) {
+    while (!refused) {
       bool missing = false;
 #pragma unroll
       for (int r = 0; r < 4; r++) {
@@ -640,14 +662,19 @@ __device__ void zvc_stream_scanner(uint32_t* ws, int tiles, int step, int* nnz, 
         missing |= (v[r] & kTileReady) == 0u;
       }
       if (__ballot(missing) == 0ull) break;
-      if (++spins > spin_limit) {  // give up: report it through *nnz; the offsets that follow are garbage below n
-        if (lane == 0) {
-          atomicOr(&ws[1], 1u);
-          atomicMin(nnz, -1);
-        }
+      if (++spins > spin_limit) {  // give up: flag it; the offsets that follow are garbage below n
+        if (lane == 0) atomicOr(&ws[kWsFlag], 1u);
         break;
       }
       __builtin_amdgcn_s_sleep(4);
+    }
+    // these counts have been read: clear them for the next run
+    if (!refused) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int t = t0 + 4 * (int)lane + r;
+        if (t < stop) st_status(&status[t], 0u);
+      }
     }
     unsigned c[4], mine = 0;
 #pragma unroll
@@ -665,7 +692,11 @@ __device__ void zvc_stream_scanner(uint32_t* ws, int tiles, int step, int* nnz, 
     }
     carry += (unsigned)__builtin_amdgcn_readlane((int)incl, 63);
   }
-  if (lane == 0) atomicMin(nnz, (int)carry);
+  if (lane == 0) {
+    if (!refused) *nnz = ld_status(&ws[kWsFlag]) != 0u ? -1 : (int)carry;
+    __threadfence();
+    __hip_atomic_fetch_add(&ws[kWsRuns], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 }
 
 template <bool HINT>
@@ -684,7 +715,7 @@ __global__ __launch_bounds__(64 * kSWaves) void zvc_stream_kernel(
   const unsigned lane = lane_id();
   const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   uint32_t* status = ws + 16;
-  const uint32_t* offset = ws + 16 + g.tiles;
+  uint32_t* offset = ws + 16 + g.tiles;
   const int iters = (g.tiles - w + G - 1) / G;  // >= 1: the grid has no more data workgroups than there are tiles
   // chunk index = half row / W by multiply and shift (exact while half rows * W < 2^40)
   const unsigned long long w_magic = ((1ull << 40) + (unsigned)g.E / 32u - 1) / ((unsigned)g.E / 32u);
@@ -732,16 +763,17 @@ __global__ __launch_bounds__(64 * kSWaves) void zvc_stream_kernel(
     if (wv == 0 && exists && lane == 0 && !(skip_first && t == 0)) st_status(&status[t], kTileReady | total[slot]);
   };
   // waits (bounded) until the scanner has published the offset of tile t
+  bool gave_up = false;
+  uint32_t runs0 = 0;  // ws[kWsRuns] when this wavefront gave up
   auto await_offset = [&](int t) {
     unsigned spins = 0;
     while ((ov & kTileReady) == 0u) {
       if (++spins > spin_limit) {
-        // give up: report it through *nnz and go on with what is there, so that every
-        // workgroup still reaches its end (offsets stay below n, the output is garbage)
-        if (lane == 0) {
-          atomicOr(&ws[1], 1u);
-          atomicMin(nnz, -1);
-        }
+        // give up: flag it and go on with what is there, so that every workgroup
+        // still reaches its end (offsets are kept inside the tensor, the output is garbage)
+        if (lane == 0) atomicOr(&ws[kWsFlag], 1u);
+        if (!gave_up) runs0 = ld_status(&ws[kWsRuns]);  // the scanner has not finished: it still owes this offset
+        gave_up = true;
         break;
       }
       __builtin_amdgcn_s_sleep(2);
@@ -802,8 +834,16 @@ __global__ __launch_bounds__(64 * kSWaves) void zvc_stream_kernel(
       const int t = i * G + w;
       // ---- this tile's offset was asked for a stage ago; ask for the next one
       await_offset(t);
-      out_prefix = ov & ~kTileReady;
       out_total = total[s];
+      // whatever the word held (a workspace that was never prepared, a wait that ran out): what this
+      // tile writes stays inside the tensor
+      // (in a vector register on purpose: as a scalar the compiler fetches the word's value the
+      // moment it was asked for, which waits for every load in flight)
+      {
+        uint32_t given = ov & ~kTileReady;
+        asm volatile("" : "+v"(given));
+        out_prefix = min(given, (unsigned)g.n - out_total);
+      }
       // ---- the previous tile leaves
       if (i > 0) write_out(prev_prefix, prev_total);
       prev_prefix = out_prefix;
@@ -874,6 +914,15 @@ __global__ __launch_bounds__(64 * kSWaves) void zvc_stream_kernel(
     }
   }
   write_out(prev_prefix, prev_total);
+  // ---- the offsets of my tiles have all been read: clear them for the next run (here and not tile by
+  // tile: a store per stage from one wavefront, small as it is, costs the pipeline 4 % at 256 MiB)
+  for (int i = (int)threadIdx.x; i < iters; i += 64 * kSWaves) st_status(&offset[i * G + w], 0u);
+  // ---- a wavefront whose wait ran out says so after the scanner has written its result
+  if (gave_up) {
+    for (unsigned spins = 0; ld_status(&ws[kWsRuns]) == runs0 && spins < spin_limit; spins++)
+      __builtin_amdgcn_s_sleep(2);
+    if (lane == 0) *nnz = -1;
+  }
 }
 
 // ------------------------------------------------------------------ probe
@@ -1078,7 +1127,7 @@ static int device_compute_units()
 static int status_words(int process);
 // Tensors of at least this many bytes take the single pass in cswap_zvc_compress_fused; smaller ones
 // finish sooner with the three kernels (a few rounds of the grid do not fill the pipeline).
-static unsigned long long g_single_pass_bytes = 128ull << 20;  // cswap_zvc_set_single_pass_bytes
+static unsigned long long g_single_pass_bytes = 64ull << 20;  // cswap_zvc_set_single_pass_bytes
 
 extern "C" size_t cswap_zvc_set_single_pass_bytes(size_t bytes)
 {
@@ -1123,9 +1172,6 @@ extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, v
   if (!single_pass) return cswap_zvc_compress(d_in, n, process, d_begin, d_nnz, d_values, d_mask, stream);
   // one workgroup per compute unit, the last of them the scanner
   const int data_groups = sg.tiles < cus - 1 ? sg.tiles : cus - 1;
-  const int words = 2 * sg.tiles + 16;
-  hipLaunchKernelGGL(zvc_ws_zero_kernel, dim3((words + 255) / 256), dim3(256), 0, (hipStream_t)stream, ws, words,
-                     d_nnz);
   if (4ull * (unsigned long long)n >= g_staged_compact_bytes)
     hipLaunchKernelGGL(zvc_stream_kernel<true>, dim3(data_groups + 1), dim3(64 * kSWaves), 0, (hipStream_t)stream,
                        d_in, sg, ws, d_begin, d_nnz, d_values, d_mask, g_spin_limit, g_skip_first);
@@ -1140,7 +1186,7 @@ extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, v
 // because they cannot allocate one: the status words live in this array, one copy
 // per GPU, held until the process ends.
 constexpr int kStaticProcessMax = 65536;
-static __device__ __align__(256) uint32_t scratch[kStaticProcessMax + 16];
+static __device__ __align__(256) uint32_t scratch[kStaticProcessMax + 16] = {kWsMagic};  // prepared from the start
 
 namespace {
 constexpr int kMaxDevices = 64;
@@ -1148,24 +1194,44 @@ std::mutex g_scratch_mutex;
 uint32_t* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, once looked up
 }  // namespace
 
+// device address of this GPU's copy of `scratch` (looked up on first use), or an error code
+static int static_workspace(uint32_t** ws)
+{
+  int dev = -1;
+  CSWAP_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return CSWAP_E_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {  // first call on this GPU: where its copy of the array lives
+    void* p = nullptr;
+    CSWAP_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    g_scratch_ptr[dev] = static_cast<uint32_t*>(p);
+  }
+  *ws = g_scratch_ptr[dev];
+  return CSWAP_OK;
+}
+
 extern "C" int cswap_zvc_compress_fused_static(const float* d_in, int n, int process, int* d_begin, int* d_nnz,
                                                float* d_values, uint32_t* d_mask, cswap_stream_t stream)
 {
   if (process > kStaticProcessMax) return CSWAP_E_NOMEM;
-  int dev = -1;
-  CSWAP_HIP_TRY(hipGetDevice(&dev));
-  if (dev < 0 || dev >= kMaxDevices) return CSWAP_E_UNSUPPORTED;
-  uint32_t* ws;
-  {
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    if (!g_scratch_ptr[dev]) {  // first call on this GPU: where its copy of the array lives
-      void* p = nullptr;
-      CSWAP_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
-      g_scratch_ptr[dev] = static_cast<uint32_t*>(p);
-    }
-    ws = g_scratch_ptr[dev];
-  }
+  uint32_t* ws = nullptr;
+  int rc = static_workspace(&ws);
+  if (rc) return rc;
   return cswap_zvc_compress_fused(d_in, n, process, ws, d_begin, d_nnz, d_values, d_mask, stream);
+}
+
+extern "C" int cswap_zvc_workspace_clear(void* d_ws, int process, cswap_stream_t stream)
+{
+  uint32_t* ws = static_cast<uint32_t*>(d_ws);
+  if (!ws) {  // the static array of the current GPU
+    int rc = static_workspace(&ws);
+    if (rc) return rc;
+    process = kStaticProcessMax;
+  }
+  if (process <= 0) return CSWAP_E_ARG;
+  const int words = status_words(process) + 16;
+  hipLaunchKernelGGL(zvc_ws_clear_kernel, dim3((words + 255) / 256), dim3(256), 0, (hipStream_t)stream, ws, words);
+  return check_launch();
 }
 
 extern "C" int cswap_probe_nnz(const float* d_in, size_t n, unsigned long long* d_nnz, cswap_stream_t stream)

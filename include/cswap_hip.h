@@ -164,23 +164,36 @@ int cswap_zvc_compress(const float* d_in, int n, int process, int* d_begin, int*
  * scanner workgroup has turned the published tile counts into offsets, and then
  * write mask, offsets and packed values, so HBM traffic is the algorithmic
  * 4 + 1/8 + 4*density bytes per element.  Smaller tensors than
- * cswap_zvc_set_single_pass_bytes says run the three kernels, which finish sooner there.  d_ws is scratch of cswap_zvc_workspace_bytes(process) bytes (at
- * least 256 KiB), cleared by the call itself; calls that share a workspace must
- * not overlap.  Shapes the single pass does not take -- a chunk length that is not
- * a multiple of 32, d_values not 16-byte aligned, more than 32768 tiles of 12288
- * elements -- run the three kernels instead.  The workgroups wait for each other's
- * counts; that wait is bounded, and if it ever runs out (for example because the
- * kernel does not get the whole GPU) the kernel still finishes but *d_nnz is -1
- * and the other outputs are undefined: a caller must treat a negative count as
- * failure (the return value cannot tell, the call does not synchronise). */
+ * cswap_zvc_set_single_pass_bytes says run the three kernels, which finish sooner there.  d_ws is a
+ * workspace of cswap_zvc_workspace_bytes(process) bytes (at least 256 KiB) that
+ * cswap_zvc_workspace_clear has prepared once, after it was allocated; every call
+ * that succeeds leaves it ready for the next one (the kernel clears each status
+ * word as it consumes it, so no launch is spent on clearing); calls that share a
+ * workspace must not overlap.  Shapes the single pass does not take -- a chunk
+ * length that is not a multiple of 32, d_values not 16-byte aligned, more than
+ * 32768 tiles of 12288 elements -- run the three kernels instead.  The workgroups
+ * wait for each other's counts; that wait is bounded, and if it ever runs out (for
+ * example because the kernel does not get the whole GPU) the kernel still finishes
+ * but *d_nnz is -1 and the other outputs are undefined: a caller must treat a
+ * negative count as failure (the return value cannot tell, the call does not
+ * synchronise).  A workspace that was never prepared is reported the same way, and
+ * so is every later call on a workspace after a failure, until
+ * cswap_zvc_workspace_clear has been called on it again. */
 size_t cswap_zvc_workspace_bytes(int process);
 int cswap_zvc_compress_fused(const float* d_in, int n, int process, void* d_ws, int* d_begin,
                              int* d_nnz, float* d_values, uint32_t* d_mask, cswap_stream_t stream);
+/* No counterpart in the reference.  Prepares a workspace of
+ * cswap_zvc_workspace_bytes(process) bytes for cswap_zvc_compress_fused (one small
+ * kernel on `stream`): once after allocating it, and again after a call that
+ * reported failure.  d_ws == NULL: the static workspace of
+ * cswap_zvc_compress_fused_static on the current GPU (which starts out prepared;
+ * `process` is ignored). */
+int cswap_zvc_workspace_clear(void* d_ws, int process, cswap_stream_t stream);
 /* 1 if cswap_zvc_compress_fused would run the single pass for this shape (given a
  * 16-byte aligned d_values), 0 if it would run the three kernels.  Host only. */
 int cswap_zvc_takes_single_pass(int n, int process);
 /* No counterpart in the reference: the tensor size in bytes from which
- * cswap_zvc_compress_fused runs the single pass (default 128 MiB: below that the
+ * cswap_zvc_compress_fused runs the single pass (default 64 MiB: below that the
  * three kernels finish sooner; 0 = whenever the shape allows, SIZE_MAX = never).
  * Returns the previous value.  Process-wide. */
 size_t cswap_zvc_set_single_pass_bytes(size_t bytes);
@@ -196,7 +209,9 @@ void cswap_zvc_debug_set_lookback(unsigned spin_limit, unsigned skip_first);
  * array of the library (256 KiB per GPU, held until the process ends), so the
  * call takes no workspace and allocates nothing.  process <= 65536, otherwise
  * CSWAP_E_NOMEM.  Every call on a GPU uses that GPU's one array: calls that
- * overlap on one GPU (different streams, different threads) race. */
+ * overlap on one GPU (different streams, different threads) race.  After a call
+ * that reported failure (*d_nnz == -1), cswap_zvc_workspace_clear(NULL, 0, stream)
+ * makes the array usable again. */
 int cswap_zvc_compress_fused_static(const float* d_in, int n, int process, int* d_begin, int* d_nnz,
                                     float* d_values, uint32_t* d_mask, cswap_stream_t stream);
 

@@ -17,7 +17,7 @@ def torch_cuda():
 
 @pytest.fixture(scope="module", autouse=True)
 def single_pass_at_any_size():
-    """cswap_zvc_compress_fused runs its single pass only from 128 MiB on (the three
+    """cswap_zvc_compress_fused runs its single pass only from 64 MiB on (the three
     kernels finish sooner below); the tests here want it on small shapes too."""
     from cswap_amd._lib import lib
 
@@ -31,10 +31,12 @@ def test_size_rule_of_the_single_pass():
 
     L = lib()
     assert L.cswap_zvc_takes_single_pass(P * 64, P) == 1          # forced on for this module
-    mine = L.cswap_zvc_set_single_pass_bytes(128 << 20)
+    forced = L.cswap_zvc_set_single_pass_bytes(64 << 20)
+    assert forced == 0
+    mine = forced
     try:
         assert L.cswap_zvc_takes_single_pass(P * 512, P) == 0      # 32 MiB: three kernels
-        assert L.cswap_zvc_takes_single_pass(P * 2048, P) == 1     # 128 MiB
+        assert L.cswap_zvc_takes_single_pass(P * 1024, P) == 1     # 64 MiB
         assert L.cswap_zvc_takes_single_pass(P * 4096 + 5, P) == 0  # chunk length 4097: not whole half rows
         assert L.cswap_zvc_takes_single_pass(1 << 30, 1024) == 0   # more tiles than the workspace has words for
     finally:
@@ -186,13 +188,16 @@ def test_single_pass_pipeline_kernel(torch_cuda, n, process):
 
 
 def test_fused_repeated_calls_share_a_workspace(torch_cuda):
-    """The workspace is cleared by every call: back-to-back calls on one stream
-    with the same scratch buffer give the same result."""
+    """A workspace is prepared once; every call that succeeds leaves it ready for the
+    next: back-to-back calls on one stream with the same workspace, for tensors of
+    different sizes, give the right result, and afterwards every word of it but the
+    first is zero again."""
     torch = torch_cuda
+    from cswap_amd import api
     from cswap_amd._lib import check, lib
 
     L = lib()
-    ws = torch.empty(L.cswap_zvc_workspace_bytes(P), dtype=torch.uint8, device="cuda")
+    ws = api.zvc_workspace(P)
     g = torch.Generator(device="cuda"); g.manual_seed(3)
     outs = []
     for rep, n in enumerate((P * 512, P * 64, P * 512)):
@@ -206,6 +211,30 @@ def test_fused_repeated_calls_share_a_workspace(torch_cuda):
         assert k == int((t != 0).sum().item())
         assert torch.equal(values[:k], t[t != 0])
         assert int(ws.view(torch.int32)[1].item()) == 0      # no bounded wait ran out
+        words = ws.view(torch.int32)
+        assert int(words[3].item()) == rep + 1               # runs that the scanner has finished
+        assert int(words[4:].count_nonzero().item()) == 0 and int(words[2].item()) == 0   # every status word consumed and cleared
+
+
+def test_fused_refuses_a_workspace_that_was_not_prepared(torch_cuda):
+    """A workspace that never went through cswap_zvc_workspace_clear is reported as a
+    failure (nnz == -1), whatever it holds: zeros, or words that look like results
+    (which the kernel then keeps from sending any write outside the outputs)."""
+    torch = torch_cuda
+    from cswap_amd._lib import check, lib
+
+    L = lib()
+    n = P * 256
+    t = torch.relu(torch.randn(n, device="cuda"))
+    values = torch.empty(n, device="cuda"); mask = torch.empty(n // 32, dtype=torch.int32, device="cuda")
+    begin = torch.zeros(P, dtype=torch.int32, device="cuda")
+    for fill in (0, -1):
+        ws = torch.full((L.cswap_zvc_workspace_bytes(P) // 4,), fill, dtype=torch.int32, device="cuda")
+        nnz = torch.zeros(1, dtype=torch.int32, device="cuda")
+        check(L.cswap_zvc_compress_fused(t.data_ptr(), n, P, ws.data_ptr(), begin.data_ptr(), nnz.data_ptr(),
+                                         values.data_ptr(), mask.data_ptr(), None), "fused")
+        torch.cuda.synchronize()
+        assert int(nnz.item()) == -1, fill
 
 
 def test_fused_reports_a_wait_that_ran_out(torch_cuda):
@@ -213,7 +242,8 @@ def test_fused_reports_a_wait_that_ran_out(torch_cuda):
     Forced from the host: the count of the first tile is never published and the bound
     is a few re-reads, so whoever waits for it gives up at once, every kernel still
     exits normally, and the caller sees nnz == -1 instead of made-up offsets.  The
-    next call, with the defaults back, is correct again."""
+    workspace stays refused until it is cleared; after that, with the defaults back,
+    a call is correct again."""
     torch = torch_cuda
     from cswap_amd import api
     from cswap_amd._lib import check, lib
@@ -222,7 +252,7 @@ def test_fused_reports_a_wait_that_ran_out(torch_cuda):
     n = P * 256
     x = np.maximum(np.random.default_rng(5).standard_normal(n), 0).astype(np.float32)
     t = torch.from_numpy(x).cuda()
-    ws = torch.empty(L.cswap_zvc_workspace_bytes(P), dtype=torch.uint8, device="cuda")
+    ws = api.zvc_workspace(P)
     values = torch.empty(n, device="cuda"); mask = torch.empty(n // 32, dtype=torch.int32, device="cuda")
     begin = torch.zeros(P, dtype=torch.int32, device="cuda"); nnz = torch.zeros(1, dtype=torch.int32, device="cuda")
     L.cswap_zvc_debug_set_lookback(4, 1)
@@ -235,6 +265,12 @@ def test_fused_reports_a_wait_that_ran_out(torch_cuda):
         L.cswap_zvc_debug_set_lookback(0, 0)
     assert int(nnz.item()) == -1
     assert int(ws.view(torch.int32)[1].item()) == 1
+    nnz.zero_()
+    check(L.cswap_zvc_compress_fused(t.data_ptr(), n, P, ws.data_ptr(), begin.data_ptr(), nnz.data_ptr(),
+                                     values.data_ptr(), mask.data_ptr(), None), "fused")
+    torch.cuda.synchronize()
+    assert int(nnz.item()) == -1                              # still refused: the failure sticks
+    check(L.cswap_zvc_workspace_clear(ws.data_ptr(), P, None), "clear")
     check(L.cswap_zvc_compress_fused(t.data_ptr(), n, P, ws.data_ptr(), begin.data_ptr(), nnz.data_ptr(),
                                      values.data_ptr(), mask.data_ptr(), None), "fused")
     torch.cuda.synchronize()

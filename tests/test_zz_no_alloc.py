@@ -10,6 +10,7 @@ P = 512 * 32
 
 
 def _run(torch, L, x, process, static):
+    from cswap_amd import api
     from cswap_amd._lib import check
 
     n = x.numel()
@@ -22,7 +23,7 @@ def _run(torch, L, x, process, static):
         check(L.cswap_zvc_compress_fused_static(x.data_ptr(), n, process, begin.data_ptr(), nnz.data_ptr(),
                                                 values.data_ptr(), mask.data_ptr(), None), "fused_static")
     else:
-        ws = torch.empty(L.cswap_zvc_workspace_bytes(process), dtype=torch.uint8, device="cuda")
+        ws = api.zvc_workspace(process)
         check(L.cswap_zvc_compress_fused(x.data_ptr(), n, process, ws.data_ptr(), begin.data_ptr(), nnz.data_ptr(),
                                          values.data_ptr(), mask.data_ptr(), None), "fused")
     torch.cuda.synchronize()
@@ -50,6 +51,22 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
         for a, b in zip(got[1:], want[1:]):
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
         assert np.array_equal(got[1], x[x != 0].cpu().numpy())
+    # A run whose bounded waits run out (forced from the host: the first tile's count is never
+    # published, the bound is a few re-reads) reports -1 and leaves the static array refused
+    # until cswap_zvc_workspace_clear(NULL, ...) has prepared it again.
+    n = P * 64
+    x = torch.relu(torch.randn(n, generator=g, device="cuda"))
+    L.cswap_zvc_debug_set_lookback(4, 1)
+    try:
+        print("static entry point: forced give-up", flush=True)
+        assert _run(torch, L, x, P, static=True)[0] == -1
+    finally:
+        L.cswap_zvc_debug_set_lookback(0, 0)
+    assert _run(torch, L, x, P, static=True)[0] == -1
+    assert L.cswap_zvc_workspace_clear(None, 0, None) == 0
+    got = _run(torch, L, x, P, static=True)
+    assert got[0] == int((x != 0).sum().item())
+    assert np.array_equal(got[1], x[x != 0].cpu().numpy())
     L.cswap_zvc_set_single_pass_bytes(size_rule)
     # beyond the static array: refused, nothing launched
     x = torch.zeros(1 << 20, device="cuda")
