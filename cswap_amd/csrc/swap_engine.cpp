@@ -283,8 +283,8 @@ static int probe_tensor(cswap_engine* e, Ticket& t, const float* d_in, hipStream
   return CSWAP_OK;
 }
 
-// An explicit ZVC request for a large tensor: count, scan and compaction in one pass over the
-// tensor, straight into a staging block of the worst-case size that is cut back to what was
+// An explicit ZVC request for a tensor that one of the single-kernel forms takes: count, scan and
+// compaction in one pass over the tensor, straight into a staging block of the worst-case size that is cut back to what was
 // needed once the non-zero count is on the host (the same small round trip a probe makes).
 // Returns 1 if it did not run (no room for the worst case, a chunk count beyond the
 // workspace) or did not finish its job (the bounded wait inside the kernel ran out): the caller

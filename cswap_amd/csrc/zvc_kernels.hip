@@ -925,6 +925,167 @@ __global__ __launch_bounds__(64 * kSWaves) void zvc_stream_kernel(
   }
 }
 
+// ------------------------------------------------------------------ one kernel for small tensors
+// Up to 32 MiB the whole tensor fits in the registers of one grid: every workgroup (one per
+// compute unit, sixteen wavefronts) loads its share once -- wavefront v of workgroup w owns R
+// consecutive rows of 64 elements --, counts it, writes its mask words, and publishes its count.
+// There is no scanner: every workgroup reads all the counts itself, one trip through memory
+// instead of two, takes the sum of those before it as its offset, and stores its non-zeros
+// straight from the registers (at these sizes the values array stays in the memory-side cache,
+// where whole-line stores through an LDS stage gain nothing).  Workgroup 0 writes the total.
+//
+// The counts live in two arrays of 256 words at the end of the workspace, used in turns: run
+// k publishes into array k & 1 and every workgroup clears its word of the other one, which
+// nobody reads any more; ws[kWsSmallRuns] counts the runs.  The grid is the same for every
+// size, so every word is cleared every time.  Failure works as in the pipeline kernel: a wait
+// that runs out raises the sticky flag, the offsets are kept inside the tensor, and the
+// wavefront that gave up writes -1 after workgroup 0 has stepped the run counter.
+constexpr int kQWaves = 16;
+constexpr int kQGroupsMax = 256;
+constexpr int kWsSmallRuns = 4;
+constexpr int kSmallWords = 2 * kQGroupsMax;  // taken from the end of the workspace's status words
+
+template <int R>
+__global__ __launch_bounds__(64 * kQWaves) void zvc_small_kernel(
+    const float* __restrict__ in, StreamGeometry g, uint32_t* __restrict__ ws, uint32_t* __restrict__ counts,
+    int* __restrict__ begin, int* __restrict__ nnz, float* __restrict__ values, uint32_t* __restrict__ mask,
+    unsigned spin_limit, unsigned skip_first)
+{
+  constexpr int kHeld = (R + 31) / 32;  // registers of mask words: lane l of register h holds half row 64h + l
+  __shared__ unsigned s_cnt[kQWaves];
+  __shared__ unsigned s_head[4];        // refused, parity, my offset, total
+  const int G = (int)gridDim.x, w = (int)blockIdx.x;
+  const unsigned lane = lane_id();
+  const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int r0 = (w * kQWaves + wv) * R;  // my first row
+
+  // ---- my rows; rows that do not exist are read from the start of the tensor and ignored
+  const long long first = (long long)r0 * 64;
+  long long left_ll = (long long)g.n - first;
+  left_ll = left_ll < 0 ? 0 : (left_ll > R * 64 ? R * 64 : left_ll);
+  const int left = (int)left_ll;
+  const float* base = in + (left > 0 ? first : 0);
+  const unsigned last = (unsigned)max(left - 1, 0);
+  float x[R];
+#pragma unroll
+  for (int j = 0; j < R; j++) x[j] = base[min(lane + 64u * j, last)];
+  if (threadIdx.x == 0) {  // together with the data: is the workspace usable, and which count array is this run's
+    const uint32_t magic = ld_status(&ws[0]), flag = ld_status(&ws[kWsFlag]), runs = ld_status(&ws[kWsSmallRuns]);
+    s_head[0] = (magic != kWsMagic || flag != 0u) ? 1u : 0u;
+    s_head[1] = runs;
+  }
+
+  // ---- count, and the mask words (two per row, straight from the ballots)
+  unsigned cnt = 0;
+  uint32_t held[kHeld];
+#pragma unroll
+  for (int h = 0; h < kHeld; h++) held[h] = 0;
+#pragma unroll
+  for (int j = 0; j < R; j++) {
+    const unsigned long long m = __ballot(x[j] != 0.0f && (int)lane < left - 64 * j);
+    cnt += popc64(m);
+    if (lane == 2u * (j % 32)) held[j / 32] = (uint32_t)m;
+    if (lane == 2u * (j % 32) + 1u) held[j / 32] = (uint32_t)(m >> 32);
+  }
+#pragma unroll
+  for (int h = 0; h < kHeld; h++) {
+    const long long word = ((long long)r0 + 32 * h) * 2 + lane;
+    if ((int)lane < 2 * (R - 32 * h) && word < (long long)g.mask_words) mask[word] = held[h];
+  }
+  if (lane == 0) s_cnt[wv] = cnt;
+  __syncthreads();
+  if (s_head[0] != 0u) {  // refused: nothing is published, nothing written but the verdict
+    if (w == 0 && threadIdx.x == 0) *nnz = -1;
+    return;
+  }
+  const uint32_t runs0 = s_head[1];
+  uint32_t* mine_arr = counts + (runs0 & 1u) * kQGroupsMax;
+  const unsigned wave_cnt = lane < (unsigned)kQWaves ? s_cnt[lane] : 0u;
+  const unsigned wave_incl = wave_inclusive_scan(wave_cnt);
+  const unsigned group_total = (unsigned)__builtin_amdgcn_readlane((int)wave_incl, kQWaves - 1);
+  const unsigned woff = (unsigned)__builtin_amdgcn_readlane((int)(wave_incl - wave_cnt), wv);
+  if (threadIdx.x == 0) {
+    st_status(&counts[((runs0 & 1u) ^ 1u) * kQGroupsMax + w], 0u);
+    if (!(skip_first && w == 0)) st_status(&mine_arr[w], kTileReady | group_total);
+  }
+
+  // ---- wavefront 0 collects everybody's count: lane l looks at workgroups 4l .. 4l+3
+  bool gave_up = false;
+  if (wv == 0) {
+    uint32_t v[4];
+    unsigned spins = 0;
+    for (;;) {
+      bool missing = false;
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int k = 4 * (int)lane + r;
+        v[r] = k < G ? ld_status(&mine_arr[k]) : kTileReady;
+        missing |= (v[r] & kTileReady) == 0u;
+      }
+      if (__ballot(missing) == 0ull) break;
+      if (++spins > spin_limit) {
+        if (lane == 0) atomicOr(&ws[kWsFlag], 1u);
+        gave_up = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
+    }
+    unsigned c[4], lane_sum = 0;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      c[r] = v[r] & ~kTileReady;
+      lane_sum += c[r];
+    }
+    const unsigned incl = wave_inclusive_scan(lane_sum);
+    // counts of the workgroups before mine: whole lanes below lane w/4, and the first w%4 of that lane
+    unsigned part = incl - lane_sum;
+#pragma unroll
+    for (int r = 0; r < 3; r++) part += r < (w & 3) ? c[r] : 0u;
+    const unsigned before_me = (unsigned)__builtin_amdgcn_readlane((int)part, w >> 2);
+    const unsigned total = (unsigned)__builtin_amdgcn_readlane((int)incl, 63);
+    if (lane == 0) {
+      // whatever the words held: what this workgroup writes stays inside the tensor
+      s_head[2] = min(before_me, (unsigned)g.n - group_total);
+      s_head[3] = total;
+    }
+  }
+  __syncthreads();
+  uint32_t flag_late = 0;
+  if (w == 0 && threadIdx.x == 0) flag_late = ld_status(&ws[kWsFlag]);  // asked for now, looked at when the rows are out
+
+  // ---- my non-zeros, row by row, straight from the lanes that hold them; chunk starts on the way
+  unsigned at = s_head[2] + woff;
+  const unsigned long long w_magic = ((1ull << 40) + (unsigned)g.E / 32u - 1) / ((unsigned)g.E / 32u);
+#pragma unroll
+  for (int h = 0; h < kHeld; h++) {
+    const unsigned in_word = (unsigned)__popc(held[h]);
+    const unsigned before = wave_inclusive_scan(in_word) - in_word;
+    const unsigned half = 2u * ((unsigned)r0 + 32u * h) + lane;
+    const unsigned c = (unsigned)(((unsigned long long)half * w_magic) >> 40);
+    if ((int)lane < 2 * (R - 32 * h) && c * ((unsigned)g.E / 32u) == half && (int)c < g.active)
+      begin[c] = (int)(at + before);
+#pragma unroll
+    for (int j = 32 * h; j < R && j < 32 * h + 32; j++) {
+      const float v = x[j];
+      const bool nz = v != 0.0f && (int)lane < left - 64 * j;
+      const unsigned long long m = __ballot(nz);
+      if (nz) values[at + rank_below(m)] = v;
+      at += popc64(m);
+    }
+  }
+
+  // ---- the verdict
+  if (w == 0 && threadIdx.x == 0) {
+    *nnz = (gave_up || flag_late != 0u) ? -1 : (int)s_head[3];
+    __threadfence();
+    __hip_atomic_fetch_add(&ws[kWsSmallRuns], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else if (gave_up && w != 0) {  // (wavefront 0 of another workgroup) after workgroup 0 has spoken
+    for (unsigned spins = 0; ld_status(&ws[kWsSmallRuns]) == runs0 && spins < spin_limit; spins++)
+      __builtin_amdgcn_s_sleep(2);
+    if (lane == 0) *nnz = -1;
+  }
+}
+
 // ------------------------------------------------------------------ probe
 __global__ void zero_u64_kernel(unsigned long long* p) { *p = 0ull; }
 
@@ -1146,15 +1307,40 @@ static bool single_pass_shape(const Geometry& g, int n, int process, StreamGeome
   sg.tiles = (sg.rows + kSTileRows - 1) / kSTileRows;
   // whole half rows per chunk, two status words per tile in the workspace, a compute unit for
   // every workgroup, and a tensor large enough to fill the pipeline
-  return g.E % 32 == 0 && mask_words < (1ll << 31) - 64 && 2 * sg.tiles <= status_words(process) &&
+  return g.E % 32 == 0 && mask_words < (1ll << 31) - 64 && 2 * sg.tiles <= status_words(process) - kSmallWords &&
          device_compute_units() > 1 && 4ull * (unsigned long long)n >= g_single_pass_bytes;
+}
+
+// Whether the one-kernel form for small tensors takes this shape (a tensor below the size from
+// which the pipeline kernel runs, whole half rows per chunk, the whole tensor in the registers
+// of one grid); fills the geometry, the grid and the rows per wavefront.
+static bool small_pass_shape(const Geometry& g, int n, int process, StreamGeometry& sg, int* groups, int* rows_per_wave)
+{
+  sg.n = n; sg.E = g.E; sg.process = process; sg.active = g.active;
+  const long long mask_words = (long long)g.W * process;
+  sg.mask_words = (int)mask_words;
+  sg.rows = (int)((mask_words + 1) / 2);
+  sg.tiles = 0;
+  const int cus = device_compute_units();
+  const int G = cus < kQGroupsMax ? cus : kQGroupsMax;
+  if (G < 1 || g.E % 32 != 0 || g_single_pass_bytes == ~0ull || 4ull * (unsigned long long)n >= g_single_pass_bytes) return false;
+  // every row of the mask layout has an owner, also the rows of chunks that hold no data (their words are zero)
+  int R = 8;  // 8, 16 or 32 rows per wavefront (64 would need more registers than a wavefront of sixteen has)
+  while (R <= 32 && (long long)G * kQWaves * R < (long long)sg.rows) R *= 2;
+  if (R > 32) return false;
+  *groups = G;
+  *rows_per_wave = R;
+  return true;
 }
 
 extern "C" int cswap_zvc_takes_single_pass(int n, int process)
 {
   Geometry g;
   StreamGeometry sg;
-  return make_geometry(g, n, process) == CSWAP_OK && single_pass_shape(g, n, process, sg);
+  int groups, rows;
+  if (make_geometry(g, n, process) != CSWAP_OK) return 0;
+  if (single_pass_shape(g, n, process, sg)) return 1;
+  return small_pass_shape(g, n, process, sg, &groups, &rows) ? 2 : 0;
 }
 
 extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, void* d_ws, int* d_begin,
@@ -1169,6 +1355,18 @@ extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, v
   StreamGeometry sg;
   // anything the single pass does not take, or an output that is not 16-byte aligned, runs the three kernels
   const bool single_pass = single_pass_shape(g, n, process, sg) && (reinterpret_cast<uintptr_t>(d_values) & 15u) == 0;
+  int groups = 0, rows = 0;
+  if (!single_pass && small_pass_shape(g, n, process, sg, &groups, &rows)) {
+    uint32_t* counts = ws + 16 + status_words(process) - kSmallWords;
+#define CSWAP_SMALL(R)                                                                                              \
+  hipLaunchKernelGGL(zvc_small_kernel<R>, dim3(groups), dim3(64 * kQWaves), 0, (hipStream_t)stream, d_in, sg, ws, \
+                     counts, d_begin, d_nnz, d_values, d_mask, g_spin_limit, g_skip_first)
+    if (rows == 8) CSWAP_SMALL(8);
+    else if (rows == 16) CSWAP_SMALL(16);
+    else CSWAP_SMALL(32);
+#undef CSWAP_SMALL
+    return check_launch();
+  }
   if (!single_pass) return cswap_zvc_compress(d_in, n, process, d_begin, d_nnz, d_values, d_mask, stream);
   // one workgroup per compute unit, the last of them the scanner
   const int data_groups = sg.tiles < cus - 1 ? sg.tiles : cus - 1;

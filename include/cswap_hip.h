@@ -164,14 +164,17 @@ int cswap_zvc_compress(const float* d_in, int n, int process, int* d_begin, int*
  * scanner workgroup has turned the published tile counts into offsets, and then
  * write mask, offsets and packed values, so HBM traffic is the algorithmic
  * 4 + 1/8 + 4*density bytes per element.  Smaller tensors than
- * cswap_zvc_set_single_pass_bytes says run the three kernels, which finish sooner there.  d_ws is a
+ * cswap_zvc_set_single_pass_bytes says (64 MiB) do not fill that pipeline; of those,
+ * tensors whose mask layout has at most 131072 rows of 64 elements (32 MiB) run
+ * another one-kernel form -- the whole tensor in the registers of one grid, every
+ * workgroup reads everybody's count -- and the rest the three kernels.  d_ws is a
  * workspace of cswap_zvc_workspace_bytes(process) bytes (at least 256 KiB) that
  * cswap_zvc_workspace_clear has prepared once, after it was allocated; every call
  * that succeeds leaves it ready for the next one (the kernel clears each status
  * word as it consumes it, so no launch is spent on clearing); calls that share a
- * workspace must not overlap.  Shapes the single pass does not take -- a chunk
- * length that is not a multiple of 32, d_values not 16-byte aligned, more than
- * 32768 tiles of 12288 elements -- run the three kernels instead.  The workgroups
+ * workspace must not overlap.  Shapes the one-kernel forms do not take -- a chunk
+ * length that is not a multiple of 32, for the pipeline d_values not 16-byte
+ * aligned or more than 32512 tiles of 12288 elements -- run the three kernels instead.  The workgroups
  * wait for each other's counts; that wait is bounded, and if it ever runs out (for
  * example because the kernel does not get the whole GPU) the kernel still finishes
  * but *d_nnz is -1 and the other outputs are undefined: a caller must treat a
@@ -189,12 +192,14 @@ int cswap_zvc_compress_fused(const float* d_in, int n, int process, void* d_ws, 
  * cswap_zvc_compress_fused_static on the current GPU (which starts out prepared;
  * `process` is ignored). */
 int cswap_zvc_workspace_clear(void* d_ws, int process, cswap_stream_t stream);
-/* 1 if cswap_zvc_compress_fused would run the single pass for this shape (given a
- * 16-byte aligned d_values), 0 if it would run the three kernels.  Host only. */
+/* What cswap_zvc_compress_fused would run for this shape (given a 16-byte aligned
+ * d_values): 1 the pipeline kernel, 2 the one-kernel form for small tensors, 0 the
+ * three kernels.  Host only. */
 int cswap_zvc_takes_single_pass(int n, int process);
 /* No counterpart in the reference: the tensor size in bytes from which
- * cswap_zvc_compress_fused runs the single pass (default 64 MiB: below that the
- * three kernels finish sooner; 0 = whenever the shape allows, SIZE_MAX = never).
+ * cswap_zvc_compress_fused runs the pipeline kernel (default 64 MiB; 0 = whenever
+ * the shape allows, and then the form for small tensors never runs; SIZE_MAX =
+ * the three kernels for every tensor).
  * Returns the previous value.  Process-wide. */
 size_t cswap_zvc_set_single_pass_bytes(size_t bytes);
 /* For tests of that failure path only.  spin_limit: how many times a wavefront

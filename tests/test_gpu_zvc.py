@@ -26,6 +26,18 @@ def single_pass_at_any_size():
     lib().cswap_zvc_set_single_pass_bytes(before)
 
 
+@pytest.fixture(params=["pipeline", "small"])
+def fused_form(request):
+    """The two single-kernel forms behind cswap_zvc_compress_fused: the pipeline kernel, forced
+    on at any size (what the module-wide fixture sets), and the one-kernel form that the size
+    rule picks for tensors of up to 32 MiB (the pipeline kernel takes over at 64 MiB)."""
+    from cswap_amd._lib import lib
+
+    before = lib().cswap_zvc_set_single_pass_bytes(0 if request.param == "pipeline" else 64 << 20)
+    yield request.param
+    lib().cswap_zvc_set_single_pass_bytes(before)
+
+
 def test_size_rule_of_the_single_pass():
     from cswap_amd._lib import lib
 
@@ -35,8 +47,10 @@ def test_size_rule_of_the_single_pass():
     assert forced == 0
     mine = forced
     try:
-        assert L.cswap_zvc_takes_single_pass(P * 512, P) == 0      # 32 MiB: three kernels
-        assert L.cswap_zvc_takes_single_pass(P * 1024, P) == 1     # 64 MiB
+        assert L.cswap_zvc_takes_single_pass(P * 512, P) == 2      # 32 MiB: the one-kernel form for small tensors
+        assert L.cswap_zvc_takes_single_pass(P * 512 + 32 * P, P) == 0   # 34 MiB: too large for it, three kernels
+        assert L.cswap_zvc_takes_single_pass(P * 64 + 5, P) == 0   # chunk length 65: three kernels
+        assert L.cswap_zvc_takes_single_pass(P * 1024, P) == 1     # 64 MiB: the pipeline kernel
         assert L.cswap_zvc_takes_single_pass(P * 4096 + 5, P) == 0  # chunk length 4097: not whole half rows
         assert L.cswap_zvc_takes_single_pass(1 << 30, 1024) == 0   # more tiles than the workspace has words for
     finally:
@@ -143,17 +157,19 @@ def test_expand_four_per_lane(torch_cuda, compact_form, n, process):
 
 
 @pytest.mark.parametrize("pct", [30, 50, 70, 90])
-def test_fused_single_pass_config2(torch_cuda, pct):
+def test_fused_single_pass_config2(torch_cuda, fused_form, pct):
+    from cswap_amd._lib import lib
     from cswap_amd.workloads import config2_tensor
 
     x = config2_tensor(pct).reshape(-1)
+    assert lib().cswap_zvc_takes_single_pass(x.size, P) == (1 if fused_form == "pipeline" else 2)
     check_against_oracle(x, run_gpu(torch_cuda, x, fused=True))
 
 
 @pytest.mark.parametrize("n,process", [(1, P), (33, P), (1000, P), (P - 1, P), (P + 1, P), (1_000_003, P),
                                         (P * 62 + 17, P), (P * 96 + 5, P), (P * 2048, P), (P * 4100 + 3, P),
                                         (300_001, 7), (64 * 9000 + 1, 64), (5000, 1)])
-def test_fused_single_pass_ragged(torch_cuda, n, process):
+def test_fused_single_pass_ragged(torch_cuda, fused_form, n, process):
     """Every register-tile size of the fused kernel (8..128 values per lane), the
     fallback for chunks above 8192 elements, partial last chunks, idle chunks."""
     rng = np.random.default_rng(n % 1000 + process)
@@ -172,14 +188,18 @@ def test_fused_single_pass_ragged(torch_cuda, n, process):
     (1024 * 16384, 1024),        # one chunk = one tile
     (999 * 160 - 37, 999),       # an odd number of mask words in all
     (64 * 2048 - 13, 64), (992, 1), (32, 1), (4096, 8)])
-def test_single_pass_pipeline_kernel(torch_cuda, n, process):
-    """Shapes the pipeline form of the single-pass compression accepts (chunk length a
+def test_single_pass_pipeline_kernel(torch_cuda, fused_form, n, process):
+    """Shapes the single-kernel forms of the compression accept (chunk length a
     multiple of 32, at most 16384): grids smaller and larger than the number of tiles,
     partial rows, chunks that start in the middle of a row, idle chunks."""
     import oracle
+    from cswap_amd._lib import lib
 
     E, W, K = oracle.zvc_geometry(n, process)
     assert E % 32 == 0 and E <= 16384
+    takes = lib().cswap_zvc_takes_single_pass(n, process)
+    rows = (W * process + 1) // 2                 # 64-element rows of the mask layout; the small form holds 256 x 16 x 32
+    assert takes == (1 if fused_form == "pipeline" or 4 * n >= 64 << 20 else (2 if rows <= 131072 else 0))
     rng = np.random.default_rng(n % 977 + process)
     zeros = rng.uniform(0.2, 0.9)
     x = (rng.standard_normal(n, dtype=np.float32) * (rng.random(n, dtype=np.float32) > zeros)).astype(np.float32)
@@ -187,7 +207,7 @@ def test_single_pass_pipeline_kernel(torch_cuda, n, process):
     check_against_oracle(x, run_gpu(torch_cuda, x, process, fused=True), process)
 
 
-def test_fused_repeated_calls_share_a_workspace(torch_cuda):
+def test_fused_repeated_calls_share_a_workspace(torch_cuda, fused_form):
     """A workspace is prepared once; every call that succeeds leaves it ready for the
     next: back-to-back calls on one stream with the same workspace, for tensors of
     different sizes, give the right result, and afterwards every word of it but the
@@ -212,11 +232,18 @@ def test_fused_repeated_calls_share_a_workspace(torch_cuda):
         assert torch.equal(values[:k], t[t != 0])
         assert int(ws.view(torch.int32)[1].item()) == 0      # no bounded wait ran out
         words = ws.view(torch.int32)
-        assert int(words[3].item()) == rep + 1               # runs that the scanner has finished
-        assert int(words[4:].count_nonzero().item()) == 0 and int(words[2].item()) == 0   # every status word consumed and cleared
+        assert int(words[3 if fused_form == "pipeline" else 4].item()) == rep + 1     # runs that have finished
+        if fused_form == "pipeline":                         # every status word consumed and cleared
+            assert int(words[5:].count_nonzero().item()) == 0 and int(words[2].item()) == 0
+        else:                                                # all but this run's counts, which the next run clears
+            tail = words[16:].clone()
+            mine = tail.numel() - 512 + 256 * (rep & 1)
+            assert int(tail[mine:mine + 256].count_nonzero().item()) == 256
+            tail[mine:mine + 256] = 0
+            assert int(tail.count_nonzero().item()) == 0
 
 
-def test_fused_refuses_a_workspace_that_was_not_prepared(torch_cuda):
+def test_fused_refuses_a_workspace_that_was_not_prepared(torch_cuda, fused_form):
     """A workspace that never went through cswap_zvc_workspace_clear is reported as a
     failure (nnz == -1), whatever it holds: zeros, or words that look like results
     (which the kernel then keeps from sending any write outside the outputs)."""
@@ -237,7 +264,7 @@ def test_fused_refuses_a_workspace_that_was_not_prepared(torch_cuda):
         assert int(nnz.item()) == -1, fill
 
 
-def test_fused_reports_a_wait_that_ran_out(torch_cuda):
+def test_fused_reports_a_wait_that_ran_out(torch_cuda, fused_form):
     """The single-pass kernel's waits for the counts of other workgroups are bounded.
     Forced from the host: the count of the first tile is never published and the bound
     is a few re-reads, so whoever waits for it gives up at once, every kernel still
