@@ -321,6 +321,31 @@ def test_special_values_and_extremes(torch_cuda, compact_form):
                          run_gpu(torch_cuda, np.arange(1, n + 1, dtype=np.float32)))
 
 
+def test_special_values_and_extremes_single_kernel(torch_cuda, fused_form):
+    """The same through both single-kernel forms: -0.0 is a zero, NaN, the infinities and the
+    smallest subnormal are not; an all-zero tensor, a tensor without zeros, and tensors of one
+    half row and of one workgroup's share."""
+    from cswap_amd._lib import lib
+
+    n = P * 64
+    x = np.zeros(n, dtype=np.float32)
+    x[[3, 10, 11, 12, 13, 70, n - 1]] = [-0.0, np.nan, np.inf, -np.inf, 1e-45, -2.5, 7.0]
+    assert lib().cswap_zvc_takes_single_pass(n, P) == (1 if fused_form == "pipeline" else 2)
+    got = run_gpu(torch_cuda, x, fused=True)
+    assert got[3] == 6
+    assert np.array_equal(got[0].view(np.uint32), x[[10, 11, 12, 13, 70, n - 1]].view(np.uint32))
+    want = x.copy(); want[3] = 0.0
+    assert np.array_equal(got[4].view(np.uint32), want.view(np.uint32))
+    for y in (np.zeros(n, np.float32), np.arange(1, n + 1, dtype=np.float32),
+              np.ones(32, np.float32), np.zeros(32, np.float32)):
+        process = P if y.size == n else 1
+        assert lib().cswap_zvc_takes_single_pass(y.size, process) != 0
+        check_against_oracle(y, run_gpu(torch_cuda, y, process, fused=True), process)
+    rng = np.random.default_rng(17)
+    y = (rng.standard_normal(16 * 32 * 64 + 96, dtype=np.float32) * (rng.random(16 * 32 * 64 + 96) < 0.5)).astype(np.float32)
+    check_against_oracle(y, run_gpu(torch_cuda, y, y.size // 32, fused=True), y.size // 32)   # chunks of one half row
+
+
 def test_reference_call_sequence(torch_cuda):
     """The four launchers in the order CSWAP+/Execution.h:88-95 calls them, with a
     host read of nnz in between, produce what the one-call path produces."""
