@@ -994,7 +994,7 @@ __global__ __launch_bounds__(64 * kQWaves) void zvc_small_kernel(
   }
   if (lane == 0) s_cnt[wv] = cnt;
   __syncthreads();
-  if (s_head[0] != 0u) {  // refused: nothing is published, nothing written but the verdict
+  if (s_head[0] != 0u) {  // refused: nothing is published, nothing written but the result
     if (w == 0 && threadIdx.x == 0) *nnz = -1;
     return;
   }
@@ -1074,7 +1074,7 @@ __global__ __launch_bounds__(64 * kQWaves) void zvc_small_kernel(
     }
   }
 
-  // ---- the verdict
+  // ---- the result
   if (w == 0 && threadIdx.x == 0) {
     *nnz = (gave_up || flag_late != 0u) ? -1 : (int)s_head[3];
     __threadfence();
