@@ -227,6 +227,8 @@ def headline_fractions(ex):
         "zvc_512MiB": pick("zvc_relu_512MiB", "compress_total_hbm_frac", "expand_hbm_frac"),
         "zvc_config2_50pct": pick("zvc_config2_s50", "compress_total_hbm_frac", "expand_hbm_frac"),
     }
+    if ex.get("box_memory_GBs"):
+        also["box_copy_GBs"] = ex["box_memory_GBs"]["copy_read_plus_write"]
     sw = ex.get("swap")
     if sw and "total_none_ms" in sw:
         also["swap_config4_ms"] = {"raw": sw["total_none_ms"], "selector": sw["total_auto_ms"]}
@@ -445,7 +447,16 @@ def extras(torch, api, dev, zvc_only=0):
                 "compress_GBs_fp32": round(4 * n / e / 1e6, 1), "decompress_GBs_fp32": round(4 * n / d / 1e6, 1),
                 "compress_hbm_frac": round(bpv * n / e / 1e6 / HBM_PEAK_GBS, 4),
                 "decompress_hbm_frac": round(bpv * n / d / 1e6 / HBM_PEAK_GBS, 4)}
-    del big
+    # ---- what this box's memory gives plain kernels on the same 402.7 MB buffer (bytes moved per second):
+    # torch's device copy (reads and writes it), fill (writes it), and this library's read-only counting pass
+    other = torch.empty_like(big)
+    cnt = torch.zeros(1, dtype=torch.int64, device=dev)
+    nb = 4 * big.numel()
+    ex["box_memory_GBs"] = {
+        "copy_read_plus_write": round(2 * nb / ev_ms(torch, lambda: other.copy_(big), 40) / 1e6, 1),
+        "fill_write": round(nb / ev_ms(torch, lambda: other.fill_(1.0), 40) / 1e6, 1),
+        "count_nonzero_read": round(nb / ev_ms(torch, lambda: api.probe_nnz(big, out=cnt), 40) / 1e6, 1)}
+    del big, other
 
     # ---- configuration 5's other tensors (rates 8 and 16) and configuration 3's stack (rates 4/8/16)
     from cswap_amd.workloads import config3_fields, config5_tensor_torch
