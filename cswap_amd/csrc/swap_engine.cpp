@@ -5,8 +5,16 @@
 //   swap_out  = pre  : (probe, select,) compress on the compute stream, then an
 //                      async device-to-host copy on a dedicated copy stream
 //   swap_wait = post : wait for that copy; the device tensor may then be freed
-//   swap_in          : async host-to-device copy on the copy stream, then
-//                      decompress on the compute stream
+//   swap_in          : async host-to-device copy on a second copy stream (the link
+//                      carries both directions at once), then decompress on the
+//                      compute stream; a compressed tensor whose outbound copy has
+//                      not finished yet is decompressed straight from its staging
+//                      block, without touching the link
+// Nothing here makes the host wait unless it has to: a staging block whose copy
+// has finished is taken back the next time somebody needs room (an event query),
+// a released ticket whose work is still in flight gives its memory back when that
+// work is done, and only a request that finds the pools full waits, for the oldest
+// work in flight.
 // Differences by design: copies are ordered against kernels with events instead
 // of device-wide synchronisation (the reference's ZFP path runs on the default
 // stream between two cudaDeviceSynchronize calls, CSWAP+/zfp/cuZFP.cu:393-399);
@@ -86,7 +94,9 @@ class Pool {
   size_t size_ = 0;
 };
 
-enum TicketState { kFree = 0, kOutInFlight = 1, kOnHost = 2, kInInFlight = 3, kPrefetched = 4 };
+// kReleasing: released by the caller while some of its work was still in flight; invisible to
+// the caller (the ticket number is not handed out again until that work is done)
+enum TicketState { kFree = 0, kOutInFlight = 1, kOnHost = 2, kInInFlight = 3, kPrefetched = 4, kReleasing = 5 };
 
 struct Ticket {
   int state = kFree;
@@ -99,6 +109,10 @@ struct Ticket {
   bool dev_held = false;
   size_t probe_off = 0, probe_bytes = 0;  // the probe's chunk counts (ZVC offsets), kept until the payload has them
   bool probe_held = false;
+  bool out_pending = false;       // the outbound copy (ev_copy) is not known to have finished
+  bool done_pending = false;      // a decompression that reads the staging block (ev_done) is not known to have finished
+  bool keep_staged = false;       // a prefetch found the payload still in its staging block: it stays there
+  unsigned long long seq = 0;     // order of the swap-outs: the oldest work in flight is waited for first
   hipEvent_t ev_ready = nullptr;  // compute stream: compressed data / destination ready
   hipEvent_t ev_copy = nullptr;   // copy stream: transfer finished
   hipEvent_t ev_done = nullptr;   // compute stream: decompression finished
@@ -108,7 +122,9 @@ struct Ticket {
 
 struct cswap_engine {
   std::mutex mu;
-  hipStream_t copy = nullptr;
+  hipStream_t copy = nullptr;     // device to host
+  hipStream_t copy_in = nullptr;  // host to device
+  unsigned long long next_seq = 1;
   char* h_base = nullptr;
   char* d_base = nullptr;
   Pool hpool, dpool;
@@ -152,6 +168,7 @@ extern "C" void cswap_engine_destroy(cswap_engine* e)
 {
   if (!e) return;
   if (e->copy) (void)hipStreamSynchronize(e->copy);
+  if (e->copy_in) (void)hipStreamSynchronize(e->copy_in);
   for (auto& t : e->tickets) {
     if (t.ev_ready) (void)hipEventDestroy(t.ev_ready);
     if (t.ev_copy) (void)hipEventDestroy(t.ev_copy);
@@ -164,6 +181,7 @@ extern "C" void cswap_engine_destroy(cswap_engine* e)
   if (e->h_base) (void)hipHostFree(e->h_base);
   if (e->d_base) (void)hipFree(e->d_base);
   if (e->copy) (void)hipStreamDestroy(e->copy);
+  if (e->copy_in) (void)hipStreamDestroy(e->copy_in);
   delete e;
 }
 
@@ -192,6 +210,7 @@ extern "C" int cswap_engine_create(cswap_engine** out, const cswap_engine_config
     if ((err = hipGetDevice(&e->device)) != hipSuccess) { fail(err); break; }
     // default priority on purpose; non-blocking so it never serialises with the null stream
     if ((err = hipStreamCreateWithFlags(&e->copy, hipStreamNonBlocking)) != hipSuccess) { fail(err); break; }
+    if ((err = hipStreamCreateWithFlags(&e->copy_in, hipStreamNonBlocking)) != hipSuccess) { fail(err); break; }
     if ((err = hipHostMalloc((void**)&e->h_base, cfg.pinned_pool_bytes, hipHostMallocDefault)) != hipSuccess) { fail(err); break; }
     if ((err = hipMalloc((void**)&e->d_base, cfg.device_pool_bytes)) != hipSuccess) { fail(err); break; }
     if ((err = hipHostMalloc((void**)&e->h_nnz, 256, hipHostMallocDefault)) != hipSuccess) { fail(err); break; }
@@ -245,6 +264,82 @@ static void drop_device(cswap_engine* e, Ticket& t)
   }
 }
 
+// Has the event fired?  Does not wait; "not yet" is an answer, not an error to leave behind.
+static bool event_done(hipEvent_t ev)
+{
+  const hipError_t r = hipEventQuery(ev);
+  if (r != hipSuccess) (void)hipGetLastError();
+  return r == hipSuccess;
+}
+
+// The outbound copy of t has finished: its staging goes back, unless a prefetch asked for the
+// payload to stay on the device, in which case the ticket is now simply prefetched.
+static void land_outbound(cswap_engine* e, Ticket& t)
+{
+  t.out_pending = false;
+  if (t.keep_staged && t.dev_held) {
+    if (t.probe_held) {
+      e->dpool.free(t.probe_off, t.probe_bytes);
+      t.probe_held = false;
+    }
+    t.state = kPrefetched;
+  } else {
+    drop_device(e, t);
+    t.state = kOnHost;
+  }
+  t.keep_staged = false;
+}
+
+static void free_ticket(cswap_engine* e, Ticket& t)
+{
+  drop_device(e, t);
+  e->hpool.free(t.host_off, t.host_bytes);
+  t.out_pending = t.done_pending = t.keep_staged = false;
+  t.state = kFree;
+}
+
+// Looks at what is in flight without waiting: an outbound copy that has finished lets its
+// staging block go, a released ticket whose work is done gives everything back.
+static void reclaim_finished(cswap_engine* e)
+{
+  for (auto& t : e->tickets) {
+    if (t.state != kOutInFlight && t.state != kReleasing && !(t.state == kInInFlight && t.out_pending)) continue;
+    if (t.out_pending && event_done(t.ev_copy)) t.out_pending = false;
+    if (t.done_pending && event_done(t.ev_done)) t.done_pending = false;
+    if (t.state == kOutInFlight && !t.out_pending) {
+      land_outbound(e, t);
+    } else if (t.state == kReleasing && !t.out_pending && !t.done_pending) {
+      free_ticket(e, t);
+    }
+  }
+}
+
+// Waits for the oldest work in flight whose end gives memory back (an outbound copy, a
+// released ticket) and takes that memory back.  false: nothing of the kind is in flight.
+static bool reclaim_oldest(cswap_engine* e, bool released_only = false)
+{
+  Ticket* oldest = nullptr;
+  for (auto& t : e->tickets)
+    if (((t.state == kOutInFlight && !released_only) || t.state == kReleasing) && (!oldest || t.seq < oldest->seq))
+      oldest = &t;
+  if (!oldest) return false;
+  if (oldest->out_pending) (void)hipEventSynchronize(oldest->ev_copy);
+  if (oldest->state == kReleasing && oldest->done_pending) (void)hipEventSynchronize(oldest->ev_done);
+  reclaim_finished(e);
+  return true;
+}
+
+// An allocation from one of the pools that takes back finished work first and, if there is
+// still no room, waits for work in flight, oldest first, until there is or nothing is left.
+static bool alloc_reclaiming(cswap_engine* e, Pool& pool, size_t bytes, size_t* off)
+{
+  if (pool.alloc(bytes, off)) return true;
+  reclaim_finished(e);
+  while (!pool.alloc(bytes, off))
+    if (!reclaim_oldest(e)) return false;
+  return true;
+}
+
 // Error path of swap_out: kernels already queued on the compute stream may
 // still write the staging block, so it is given back only once they are done.
 static void abandon_device(cswap_engine* e, Ticket& t, hipStream_t compute)
@@ -264,7 +359,7 @@ static int probe_tensor(cswap_engine* e, Ticket& t, const float* d_in, hipStream
 {
   const size_t cnt_bytes = 4 * (size_t)t.process;
   size_t off;
-  if (!e->dpool.alloc(cnt_bytes, &off)) {
+  if (!alloc_reclaiming(e, e->dpool, cnt_bytes, &off)) {
     if (required) return CSWAP_E_NOMEM;
     t.nnz = t.n;
     return CSWAP_OK;
@@ -296,7 +391,10 @@ static int single_pass_sparse(cswap_engine* e, Ticket& t, const float* d_in, hip
   const size_t hdr = zvc_header_bytes((int)t.n, t.process);
   const size_t worst = hdr + 4 * t.n;
   size_t off;
-  if (!e->dpool.alloc(worst, &off)) return 1;
+  if (!e->dpool.alloc(worst, &off)) {  // the worst case is optional: take back what has finished, wait for nothing
+    reclaim_finished(e);
+    if (!e->dpool.alloc(worst, &off)) return 1;
+  }
   char* base = e->d_base + off;
   int rc = cswap_zvc_compress_fused(d_in, (int)t.n, t.process, e->d_ws, (int*)base, e->d_nnz, (float*)(base + hdr),
                                     (uint32_t*)(base + 4 * (size_t)t.process), compute);
@@ -336,7 +434,7 @@ static int reserve_blocks(cswap_engine* e, Ticket& t, int requested)
     t.bytes_out = t.policy == CSWAP_POLICY_SPARSE ? zvc_header_bytes((int)t.n, t.process) + 4 * t.nnz
                                                   : cswap_zfp_stream_capacity(t.nx, t.ny, t.nz, e->maxbits);
     size_t off;
-    if (e->dpool.alloc(t.bytes_out, &off)) {
+    if (alloc_reclaiming(e, e->dpool, t.bytes_out, &off)) {
       t.dev_off = off; t.dev_bytes = t.bytes_out; t.dev_held = true;
     } else if (requested == CSWAP_POLICY_AUTO) {
       t.policy = CSWAP_POLICY_NONE;
@@ -350,7 +448,7 @@ static int reserve_blocks(cswap_engine* e, Ticket& t, int requested)
     t.bytes_out = 4 * t.n;
   }
   size_t hoff;
-  if (!e->hpool.alloc(t.bytes_out, &hoff)) {
+  if (!alloc_reclaiming(e, e->hpool, t.bytes_out, &hoff)) {
     drop_device(e, t);
     return CSWAP_E_NOMEM;
   }
@@ -410,15 +508,24 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   const bool zvc_ok = n <= 0x7fffffffull;
   if (policy == CSWAP_POLICY_SPARSE && !zvc_ok) return CSWAP_E_ARG;
 
+  reclaim_finished(e);
   int id = -1;
-  for (size_t i = 0; i < e->tickets.size(); i++)
-    if (e->tickets[i].state == kFree) { id = (int)i; break; }
-  if (id < 0) return CSWAP_E_NOMEM;
+  for (;;) {
+    for (size_t i = 0; i < e->tickets.size(); i++)
+      if (e->tickets[i].state == kFree) { id = (int)i; break; }
+    if (id >= 0) break;
+    // every ticket taken: a released one whose work is still in flight comes back when that work is done
+    bool releasing = false;
+    for (auto& o : e->tickets) releasing |= o.state == kReleasing;
+    if (!releasing || !reclaim_oldest(e)) return CSWAP_E_NOMEM;
+  }
   Ticket& t = e->tickets[(size_t)id];
   const int requested = policy;
   t.policy = policy; t.n = n; t.nnz = n; t.nx = nx; t.ny = ny; t.nz = nz;
   t.dev_held = false;
   t.probe_held = false;
+  t.out_pending = t.done_pending = t.keep_staged = false;
+  t.seq = e->next_seq++;
   t.process = zvc_ok ? process_for(e, n) : 0;
   cswap_costs costs = e->costs;  // the selector prices the ZVC header with this tensor's chunk count
   if (t.process) costs.process = t.process;
@@ -442,7 +549,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     if (rc < 0) return rc;
     if (rc == 0) {
       size_t hoff;
-      if (!e->hpool.alloc(t.bytes_out, &hoff)) {
+      if (!alloc_reclaiming(e, e->hpool, t.bytes_out, &hoff)) {
         (void)hipStreamSynchronize(compute);
         drop_device(e, t);
         return CSWAP_E_NOMEM;
@@ -457,6 +564,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
         return rc;
       }
       t.state = kOutInFlight;
+      t.out_pending = true;
       *ticket = id;
       return CSWAP_OK;
     }
@@ -482,6 +590,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     return rc;
   }
   t.state = kOutInFlight;
+  t.out_pending = true;
   *ticket = id;
   return CSWAP_OK;
 }
@@ -499,10 +608,10 @@ extern "C" int cswap_swap_wait(cswap_engine* e, int ticket)
   Ticket* t = get_ticket(e, ticket);
   if (!t) return CSWAP_E_ARG;
   if (t->state == kOnHost) return CSWAP_OK;
+  if (t->state == kPrefetched && t->dev_held) return CSWAP_OK;  // landed while a prefetch held its payload
   if (t->state != kOutInFlight) return CSWAP_E_STATE;
   CSWAP_HIP_TRY(hipEventSynchronize(t->ev_copy));
-  drop_device(e, *t);
-  t->state = kOnHost;
+  land_outbound(e, *t);
   return CSWAP_OK;
 }
 
@@ -511,9 +620,15 @@ static int settle_outbound(cswap_engine* e, Ticket& t)
 {
   if (t.state != kOutInFlight) return CSWAP_OK;
   CSWAP_HIP_TRY(hipEventSynchronize(t.ev_copy));
-  drop_device(e, t);
-  t.state = kOnHost;
+  land_outbound(e, t);
   return CSWAP_OK;
+}
+
+// A compressed tensor whose outbound copy may still be on its way has its payload in the
+// staging pool: whoever wants it back needs neither the end of that copy nor the link.
+static bool payload_still_staged(const Ticket& t)
+{
+  return t.state == kOutInFlight && t.dev_held && t.policy != CSWAP_POLICY_NONE;
 }
 
 extern "C" int cswap_swap_prefetch(cswap_engine* e, int ticket)
@@ -522,19 +637,27 @@ extern "C" int cswap_swap_prefetch(cswap_engine* e, int ticket)
   std::lock_guard<std::mutex> lock(e->mu);
   Ticket* t = get_ticket(e, ticket);
   if (!t) return CSWAP_E_ARG;
+  reclaim_finished(e);
   if (t->state == kPrefetched) return CSWAP_OK;
+  if (payload_still_staged(*t)) {  // it is on the device already, and now it stays: swap_in will read it there
+    t->keep_staged = true;
+    return CSWAP_OK;
+  }
   int rc = settle_outbound(e, *t);
   if (rc) return rc;
   if (t->state != kOnHost) return CSWAP_E_STATE;
   size_t off;
-  if (!e->dpool.alloc(t->bytes_out, &off)) return CSWAP_E_NOMEM;
+  // a prefetch is optional: it waits for what released tickets still owe the pool (their release used to
+  // wait for that), not for copies on the link
+  while (!e->dpool.alloc(t->bytes_out, &off))
+    if (!reclaim_oldest(e, true)) return CSWAP_E_NOMEM;
   t->dev_off = off; t->dev_bytes = t->bytes_out; t->dev_held = true;
-  // the staging region was released only after the events of its last user were waited for,
-  // so the copy stream has nothing to order against
-  hipError_t err = hipMemcpyAsync(e->d_base + off, e->h_base + t->host_off, t->bytes_out, hipMemcpyHostToDevice, e->copy);
-  if (err == hipSuccess) err = hipEventRecord(t->ev_copy, e->copy);
+  // the staging region was released only after the events of its last user were seen to have
+  // fired, so the copy stream has nothing to order against
+  hipError_t err = hipMemcpyAsync(e->d_base + off, e->h_base + t->host_off, t->bytes_out, hipMemcpyHostToDevice, e->copy_in);
+  if (err == hipSuccess) err = hipEventRecord(t->ev_copy, e->copy_in);
   if (err != hipSuccess) {
-    (void)hipStreamSynchronize(e->copy);
+    (void)hipStreamSynchronize(e->copy_in);
     drop_device(e, *t);
     return hip_fail(err);
   }
@@ -549,13 +672,20 @@ extern "C" int cswap_swap_in(cswap_engine* e, int ticket, float* d_out, cswap_st
   std::lock_guard<std::mutex> lock(e->mu);
   Ticket* t = get_ticket(e, ticket);
   if (!t) return CSWAP_E_ARG;
-  int rc = settle_outbound(e, *t);
+  reclaim_finished(e);
+  const bool staged = payload_still_staged(*t);
+  int rc = staged ? CSWAP_OK : settle_outbound(e, *t);
   if (rc) return rc;
-  if (t->state != kOnHost && t->state != kPrefetched) return CSWAP_E_STATE;
+  if (!staged && t->state != kOnHost && t->state != kPrefetched) return CSWAP_E_STATE;
 
   hipError_t err = hipSuccess;
-  void* src = nullptr;  // device address of the payload once ev_copy has fired
-  if (t->state == kPrefetched) {
+  void* src = nullptr;  // device address of the payload once it is there
+  if (staged) {
+    // the payload is complete when the compression has run (ev_ready); the outbound copy goes on
+    // reading the same block, which stays with the ticket until both are done
+    src = e->d_base + t->dev_off;
+    err = hipStreamWaitEvent(compute, t->ev_ready, 0);
+  } else if (t->state == kPrefetched) {
     src = e->d_base + t->dev_off;
     err = hipStreamWaitEvent(compute, t->ev_copy, 0);
     if (err == hipSuccess && t->policy == CSWAP_POLICY_NONE)
@@ -564,22 +694,24 @@ extern "C" int cswap_swap_in(cswap_engine* e, int ticket, float* d_out, cswap_st
     src = d_out;
     if (t->policy != CSWAP_POLICY_NONE) {
       size_t off;
-      if (!e->dpool.alloc(t->bytes_out, &off)) return CSWAP_E_NOMEM;
+      if (!alloc_reclaiming(e, e->dpool, t->bytes_out, &off)) return CSWAP_E_NOMEM;
       t->dev_off = off; t->dev_bytes = t->bytes_out; t->dev_held = true;
       src = e->d_base + off;
     }
     // the copy may not overtake earlier work of the compute stream on d_out
     err = hipEventRecord(t->ev_ready, compute);
-    if (err == hipSuccess) err = hipStreamWaitEvent(e->copy, t->ev_ready, 0);
-    if (err == hipSuccess) err = hipMemcpyAsync(src, e->h_base + t->host_off, t->bytes_out, hipMemcpyHostToDevice, e->copy);
-    if (err == hipSuccess) err = hipEventRecord(t->ev_copy, e->copy);
+    if (err == hipSuccess) err = hipStreamWaitEvent(e->copy_in, t->ev_ready, 0);
+    if (err == hipSuccess) err = hipMemcpyAsync(src, e->h_base + t->host_off, t->bytes_out, hipMemcpyHostToDevice, e->copy_in);
+    if (err == hipSuccess) err = hipEventRecord(t->ev_copy, e->copy_in);
     if (err == hipSuccess) err = hipStreamWaitEvent(compute, t->ev_copy, 0);
   }
   if (err != hipSuccess) {
-    (void)hipStreamSynchronize(e->copy);
+    (void)hipStreamSynchronize(e->copy_in);
     (void)hipStreamSynchronize(compute);
-    drop_device(e, *t);
-    t->state = kOnHost;
+    if (!staged) {
+      drop_device(e, *t);
+      t->state = kOnHost;
+    }
     return hip_fail(err);
   }
   if (t->policy == CSWAP_POLICY_SPARSE) {
@@ -591,7 +723,8 @@ extern "C" int cswap_swap_in(cswap_engine* e, int ticket, float* d_out, cswap_st
     rc = cswap_zfp_decompress_f32((const uint64_t*)src, t->nx, t->ny, t->nz, 0, 0, 0, e->maxbits, d_out, compute);
   }
   err = hipEventRecord(t->ev_done, compute);
-  t->state = kInInFlight;
+  t->state = kInInFlight;  // (from the staging block: out_pending stays up, the outbound copy may still run)
+  t->done_pending = true;
   if (rc) return rc;
   if (err != hipSuccess) return hip_fail(err);
   return CSWAP_OK;
@@ -603,14 +736,14 @@ extern "C" int cswap_swap_release(cswap_engine* e, int ticket)
   std::lock_guard<std::mutex> lock(e->mu);
   Ticket* t = get_ticket(e, ticket);
   if (!t) return CSWAP_E_ARG;
-  if (t->state == kFree) return CSWAP_E_STATE;
-  hipError_t err = hipSuccess;
-  if (t->state == kOutInFlight || t->state == kPrefetched) err = hipEventSynchronize(t->ev_copy);
-  if (t->state == kInInFlight) err = hipEventSynchronize(t->ev_done);
-  drop_device(e, *t);
-  e->hpool.free(t->host_off, t->host_bytes);
-  t->state = kFree;
-  return err == hipSuccess ? CSWAP_OK : hip_fail(err);
+  if (t->state == kFree || t->state == kReleasing) return CSWAP_E_STATE;
+  // what of its work is still in flight?  (a prefetch's inbound copy fires the same event as an outbound one)
+  if (t->state == kPrefetched) t->out_pending = true;
+  if (t->out_pending && event_done(t->ev_copy)) t->out_pending = false;
+  if (t->done_pending && event_done(t->ev_done)) t->done_pending = false;
+  if (!t->out_pending && !t->done_pending) free_ticket(e, *t);
+  else t->state = kReleasing;  // its memory comes back when that work is done (reclaim_finished)
+  return CSWAP_OK;
 }
 
 extern "C" int cswap_swap_info(cswap_engine* e, int ticket, cswap_ticket_info* info)
@@ -624,7 +757,8 @@ extern "C" int cswap_swap_info(cswap_engine* e, int ticket, cswap_ticket_info* i
   info->nnz = t->nnz;
   info->bytes_in = 4 * t->n;
   info->bytes_out = t->bytes_out;
-  info->state = t->state;
+  // to the caller a released ticket is free, and a payload that a prefetch found still staged is prefetched
+  info->state = t->state == kReleasing ? (int)kFree : (t->state == kOutInFlight && t->keep_staged ? (int)kPrefetched : t->state);
   return CSWAP_OK;
 }
 

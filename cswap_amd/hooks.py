@@ -23,10 +23,11 @@ E_NOMEM = -4   # CSWAP_E_NOMEM
 
 
 class _Handle:
-    __slots__ = ("ticket", "shape", "keep", "key", "refs", "out")
+    __slots__ = ("ticket", "shape", "keep", "key", "refs", "out", "raw")
 
-    def __init__(self, ticket, shape, keep, key):
+    def __init__(self, ticket, shape, keep, key, raw):
         self.ticket, self.shape, self.keep, self.key = ticket, shape, keep, key
+        self.raw = raw       # swapped out as it is: the outbound copy reads the tensor itself
         self.refs = 1        # how many autograd nodes saved this tensor
         self.out = None      # the swapped-in tensor while further nodes still have to ask for it
 
@@ -45,11 +46,15 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
     least ``min_bytes``) through ``engine``; everything else is saved as usual.
 
     The outbound copy of a tensor overlaps with whatever the compute stream does
-    next.  Up to ``depth`` copies are left in flight: packing one more first waits
-    for the oldest and lets its device copy go (the reference waits one layer
-    later, CSWAP+/vgg16-cifar10.cpp:221-228, i.e. depth 1).  With depth 2 the
-    probe and the compression of tensor i run while tensor i-1 is still on the
-    link, so the link does not idle between tensors.
+    next.  The last ``depth`` tensors packed keep their device copy; packing one
+    more lets the oldest go.  A tensor that went out raw is read by its copy, so
+    that first waits for the copy (the reference waits one layer later,
+    CSWAP+/vgg16-cifar10.cpp:221-228, i.e. depth 1); a compressed tensor's copy
+    reads the engine's staging block, so its device tensor simply goes, stream
+    ordered behind the compression, and the host waits for nothing: the forward
+    pass runs ahead of the link as far as the staging pool has room (the engine
+    takes blocks back as their copies finish and makes a request wait only when
+    the pool is full).
 
     A tensor that several nodes save (the output of a ReLU is saved by the ReLU
     and by the convolution or pooling that consumes it; attention probabilities by
@@ -59,8 +64,10 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
     swapped-in tensor, viewed in each node's shape, to every node that asks for it.
 
     The last ``depth`` tensors of the forward pass are still on the device when it
-    ends (their copies are the ones in flight) and are the first that backward
-    asks for: they are handed back as they are, without a transfer.
+    ends and are the first that backward asks for: they are handed back as they
+    are, without a transfer.  The compressed tensors before them whose outbound
+    copies are still queued have their payloads in the staging pool, and the
+    engine decompresses those from there, again without the link.
 
     Backward asks for the tensors in roughly the reverse of the order they were
     packed in, so each unpack also starts the inbound copy of the ``prefetch``
@@ -104,7 +111,8 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         """Wait for the oldest outbound copies until at most ``keep_in_flight`` are left."""
         while len(self._pending) > keep_in_flight:
             h = self._pending.pop(0)
-            self.engine.post(h.ticket)   # Execution::post: copy done, device memory may go
+            if h.raw:
+                self.engine.post(h.ticket)   # Execution::post: copy done, device memory may go
             h.keep = None
             self._live.pop(h.key, None)
 
@@ -153,7 +161,7 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         by = self.stats.setdefault("by_policy", {})
         name = {swap.NONE: "raw", swap.SPARSE: "zvc", swap.ZFP: "zfp"}.get(info.policy, str(info.policy))
         by[name] = by.get(name, 0) + 1
-        h = _Handle(ticket, tuple(t.shape), t, key)   # keeps the device copy alive until the copy finished
+        h = _Handle(ticket, tuple(t.shape), t, key, info.policy == swap.NONE)   # keeps the device copy alive for now
         self._pending.append(h)
         self._live[key] = h
         self._order.append(h)

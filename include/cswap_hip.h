@@ -299,9 +299,13 @@ typedef struct cswap_engine cswap_engine;
 typedef struct {
   size_t pinned_pool_bytes;   /* host side: compressed tensors live here while swapped out */
   size_t device_pool_bytes;   /* device staging for compressed data in flight: every tensor between swap_out and
-                                 swap_wait, and between prefetch / swap_in and release, holds a block of its
-                                 compressed size (raw swaps hold none going out).  When the pool is full an
-                                 AUTO request goes out raw, an explicit one and a prefetch return CSWAP_E_NOMEM. */
+                                 the end of its outbound copy, and between prefetch / swap_in and the end of its
+                                 decompression, holds a block of its compressed size (raw swaps hold none going
+                                 out).  Blocks come back as that work finishes, without anybody waiting; a
+                                 request that finds the pool full waits for the oldest work in flight, and only
+                                 when nothing in flight can make room does an AUTO request go out raw and an
+                                 explicit one return CSWAP_E_NOMEM (a prefetch, being optional, waits only for
+                                 what released tickets still hold). */
   int    process;             /* ZVC chunk count; 0 = per tensor size (cswap_engine_tune result, else cswap_zvc_pick_process) */
   unsigned zfp_maxbits;       /* bits per 4x4x4 block for policy ZFP; 0 = 512 (8 bits/value) */
   int    max_tickets;         /* tensors that may be swapped out at once; 0 = 256 */
@@ -328,20 +332,26 @@ int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, size_t ny, siz
 /* Execution::post: block the host until the copy of `ticket` has finished;
  * afterwards the caller may free or overwrite the device tensor. */
 int cswap_swap_wait(cswap_engine* e, int ticket);
-/* Backward side: copy back on the copy stream, then decompress into d_out on
+/* Backward side: copy back on the engine's inbound copy stream (its own: both
+ * directions of the link can be busy at once), then decompress into d_out on
  * `compute` (ordered by an event).  Returns at once; the data is ready when
- * `compute` reaches this point. */
+ * `compute` reaches this point.  A compressed tensor whose outbound copy has not
+ * finished yet is still in its staging block and is decompressed from there: no
+ * wait for the copy, nothing on the link. */
 int cswap_swap_in(cswap_engine* e, int ticket, float* d_out, cswap_stream_t compute);
 /* Backward side, ahead of time: start the host-to-device copy of the payload
  * into the engine's device staging pool on the copy stream, before a
  * destination exists, so that it overlaps the backward compute of the layers
  * that run first.  A later cswap_swap_in then only waits for that copy and
- * decompresses (policy NONE: one device-to-device copy).  Idempotent; the
+ * decompresses (policy NONE: one device-to-device copy).  For a compressed tensor
+ * whose outbound copy is still in flight the payload is on the device already: it
+ * is kept there and nothing is copied.  Idempotent; the
  * reference's counterpart lives in its patched autograd engine, which it does
  * not ship (fields read at Execution.h:260-262,278-282). */
 int cswap_swap_prefetch(cswap_engine* e, int ticket);
-/* Return the ticket's host (and any device) memory to the pools.  Waits for the
- * work of the ticket that is still in flight. */
+/* Give the ticket up.  Returns at once: its host (and any device) memory goes back
+ * to the pools when the work of the ticket that is still in flight has finished,
+ * and the ticket number is not handed out again before that. */
 int cswap_swap_release(cswap_engine* e, int ticket);
 int cswap_swap_info(cswap_engine* e, int ticket, cswap_ticket_info* info);
 /* Number of probes so far: counting passes followed by the host round trip for

@@ -722,3 +722,70 @@ def test_engine_falls_back_when_the_single_pass_gives_up(torch_cuda):
         assert torch.equal(out, x)
     finally:
         eng.close()
+
+
+@pytest.mark.parametrize("policy_name", ["sparse", "zfp"])
+def test_swap_in_while_the_outbound_copy_is_in_flight_reads_the_staging_block(torch_cuda, policy_name):
+    """A compressed tensor that is asked back before its outbound copy has finished is
+    decompressed straight from its staging block (no wait for the copy, nothing on the
+    link); the result is what a swap through the host gives, the ticket can be released
+    at once, and the pools are whole again afterwards."""
+    torch = torch_cuda
+    from cswap_amd import swap
+
+    pol = {"sparse": swap.SPARSE, "zfp": swap.ZFP}[policy_name]
+    eng = swap.SwapEngine(pinned_bytes=64 << 20, device_bytes=24 << 20)
+    try:
+        x = relu_tensor(torch, (16, 64, 32, 32), 0.6, 21)               # 4 MiB
+        plain = torch.full_like(x, -5.0)
+        tk = eng.pre(x, pol); eng.post(tk); eng.swap_in(tk, plain)
+        torch.cuda.synchronize(); eng.release(tk)
+        for rep in range(6):
+            outs = []
+            for k in range(3):                                           # several in flight at once
+                tk = eng.pre(x, pol)
+                out = torch.full_like(x, -7.0)
+                if k == 1:
+                    eng.prefetch(tk)                                     # found on the device: stays there
+                    assert eng.info(tk).state == 4
+                eng.swap_in(tk, out)
+                assert eng.info(tk).state == 3
+                eng.release(tk)                                          # at once; memory comes back when the work is done
+                assert eng.info(tk).state == 0
+                outs.append(out)
+            torch.cuda.synchronize()
+            for out in outs:
+                assert torch.equal(out.view(torch.int32), plain.view(torch.int32)), (policy_name, rep)
+        big = torch.zeros(64, 64, (24 << 20) // 4 // 4096 - 8, device="cuda")
+        tk = eng.pre(big, swap.ZFP)                                      # a quarter of the staging pool; and the host pool
+        eng.post(tk); eng.release(tk)
+        tk = eng.pre(torch.zeros(64, 64, (60 << 20) // 4 // 4096, device="cuda"), swap.NONE)   # 60 of 64 MiB pinned
+        eng.post(tk); eng.release(tk)
+    finally:
+        eng.close()
+
+
+def test_a_full_staging_pool_makes_requests_wait_not_fail(torch_cuda):
+    """Swap-outs issued back to back, without waiting for any copy, into a staging pool
+    that holds two payloads: each request that finds the pool full waits for the oldest
+    copy in flight instead of failing or going out raw, and everything comes back intact."""
+    torch = torch_cuda
+    from cswap_amd import api, swap
+
+    x = relu_tensor(torch, (32, 64, 32, 32), 0.5, 22)                    # 8 MiB, 2 MiB at 8 bits per value
+    eng = swap.SwapEngine(pinned_bytes=64 << 20, device_bytes=(4 << 20) + (256 << 10))
+    try:
+        want = api.cuda_decompress(api.cuda_compress(x, 512), x.shape, 512)
+        tks = [eng.pre(x, swap.ZFP if k % 2 else swap.AUTO) for k in range(8)]
+        for tk in tks:
+            info = eng.info(tk)
+            assert info.policy in (swap.ZFP, swap.SPARSE), info.policy   # none degraded to a raw swap
+        for tk in tks:
+            out = torch.full_like(x, -1.0)
+            eng.swap_in(tk, out)
+            torch.cuda.synchronize()
+            exact = eng.info(tk).policy == swap.SPARSE
+            assert torch.equal(out.view(torch.int32), (x if exact else want).view(torch.int32))
+            eng.release(tk)
+    finally:
+        eng.close()
