@@ -237,9 +237,10 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
 
 
 def _measure_step(step, params, make_ctx, reps=5):
-    """Best wall time of ``step(ctx)`` over ``reps`` runs after two warm-up runs, the
-    step's peak in torch's allocator above what is allocated before it, and the
-    hook statistics of the last run."""
+    """Median and best wall time of ``step(ctx)`` over ``reps`` runs after two warm-up
+    runs (a step whose copies overlap compute differently from run to run has a
+    spread worth showing), the step's peak in torch's allocator above what is
+    allocated before it, and the hook statistics of the last run."""
     import time
 
     for _ in range(2):
@@ -249,7 +250,7 @@ def _measure_step(step, params, make_ctx, reps=5):
     torch.cuda.synchronize()
     base = torch.cuda.memory_allocated()     # weights, input and whatever else the process holds
     torch.cuda.reset_peak_memory_stats()
-    best = None
+    times = []
     stats = None
     for _ in range(reps):
         ctx = make_ctx()
@@ -257,10 +258,10 @@ def _measure_step(step, params, make_ctx, reps=5):
         t0 = time.perf_counter()
         step(ctx)
         torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        best = dt if best is None else min(best, dt)
+        times.append((time.perf_counter() - t0) * 1e3)
         stats = ctx.stats if ctx is not None else None
-    return best * 1e3, (torch.cuda.max_memory_allocated() - base) / 1e6, stats
+    times.sort()
+    return (times[len(times) // 2], times[0]), (torch.cuda.max_memory_allocated() - base) / 1e6, stats
 
 
 def _swap_rows(res, eng, step, params, min_bytes, reps):
@@ -269,7 +270,8 @@ def _swap_rows(res, eng, step, params, min_bytes, reps):
                            ("selector_remembered", swap.AUTO, {"memo": memo})):
         ms, mb, st = _measure_step(step, params,
                                    lambda: swap_saved_tensors(eng, policy=pol, min_bytes=min_bytes, **kw), reps)
-        res[label] = {"step_ms": round(ms, 2), "step_peak_MB": round(mb, 1), "swapped_tensors": st["swapped"],
+        res[label] = {"step_ms": round(ms[0], 2), "step_ms_best": round(ms[1], 2), "step_peak_MB": round(mb, 1),
+                      "swapped_tensors": st["swapped"],
                       "swapped_MB": round(st["bytes_in"] / 1e6, 1), "link_MB": round(st["bytes_out"] / 1e6, 1),
                       "shared": st["shared"], "by_policy": dict(st.get("by_policy", {})),
                       "prefetched": st.get("prefetched", 0), "resident": st.get("resident", 0),
@@ -305,12 +307,12 @@ def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int =
 
     res = {"model": f"VGG-16 BN, batch {batch}, 3x{image}x{image}", "min_bytes": min_bytes}
     base_ms, base_mb, _ = _measure_step(step, params, lambda: None)
-    res["no_swap"] = {"step_ms": round(base_ms, 2), "step_peak_MB": round(base_mb, 1)}
+    res["no_swap"] = {"step_ms": round(base_ms[0], 2), "step_peak_MB": round(base_mb, 1)}
     staging = 192 << 20
     eng = swap.SwapEngine(pinned_bytes=4 << 30, device_bytes=staging)
     eng.calibrate()
     res["staging_pool_MB"] = round(staging / 1e6, 1)    # device memory the engine holds besides torch's allocator
-    _swap_rows(res, eng, step, params, min_bytes, 5)
+    _swap_rows(res, eng, step, params, min_bytes, 9)
     eng.close()
     return res
 
@@ -361,12 +363,12 @@ def bench_transformer_step(dev, layers: int = 4, batch: int = 32, seq: int = 512
 
     res = {"model": f"{layers} encoder blocks, batch {batch}, seq {seq}, hidden {hidden}, {heads} heads",
            "min_bytes": min_bytes}
-    ms, mb, _ = _measure_step(step, params, lambda: None, 4)
-    res["no_swap"] = {"step_ms": round(ms, 2), "step_peak_MB": round(mb, 1)}
+    ms, mb, _ = _measure_step(step, params, lambda: None, 5)
+    res["no_swap"] = {"step_ms": round(ms[0], 2), "step_peak_MB": round(mb, 1)}
     staging = 768 << 20
     eng = swap.SwapEngine(pinned_bytes=12 << 30, device_bytes=staging)
     eng.calibrate()
     res["staging_pool_MB"] = round(staging / 1e6, 1)
-    _swap_rows(res, eng, step, params, min_bytes, 4)
+    _swap_rows(res, eng, step, params, min_bytes, 9)
     eng.close()
     return res
