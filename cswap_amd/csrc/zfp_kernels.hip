@@ -77,6 +77,20 @@ __host__ __device__ inline unsigned region_dwords(unsigned maxbits)
 {
   return ((2u * slot_bits(maxbits) + 4u) + 3u) & ~3u;  // + padding for the 128-bit over-read / over-write
 }
+// The 32-bit decoder's slot is the block and its fence of 64 ones, nothing more: the
+// window it reads through reaches up to 64 bits further, into the next lane's block
+// (or the region's padding), and those bits are never looked at.  What this saves in
+// LDS is two more wavefronts per compute unit at 16 bits per value (8720 bytes a
+// wavefront instead of 9232), and the stride of 2 (mod 4) dwords halves the bank
+// conflicts between lanes.  Slots are 8-byte aligned only.
+__host__ __device__ inline unsigned dec_slot_bits(unsigned maxbits)
+{
+  return (maxbits & 63u) ? maxbits : maxbits + 64u;
+}
+__host__ __device__ inline unsigned dec_region_dwords(unsigned maxbits)
+{
+  return ((2u * dec_slot_bits(maxbits) + 4u) + 3u) & ~3u;
+}
 
 // ------------------------------------------------------------- block <-> field
 __device__ __forceinline__ void block_origin(const Field3& fd, uint32_t b, uint32_t& x0, uint32_t& y0,
@@ -232,18 +246,26 @@ __device__ __forceinline__ void store_region(const uint32_t* lds, unsigned lane,
 
 // the wave's coded blocks from the stream into LDS; whole-word rates get the
 // fence of ones behind every block that the fenced decoder relies on
-template <bool WHOLE>
+template <bool WHOLE, bool SLOT16 = true>
 __device__ __forceinline__ void load_region(uint32_t* lds, unsigned lane, uint32_t first, uint32_t valid,
-                                            unsigned maxbits, int stream16, const uint64_t* __restrict__ stream)
+                                            unsigned maxbits, unsigned slot, int stream16,
+                                            const uint64_t* __restrict__ stream)
 {
   if (WHOLE) {
     if (lane < valid) {
       const unsigned W = maxbits >> 6;
-      uint64_t* dst = reinterpret_cast<uint64_t*>(lds + lane * (slot_bits(maxbits) / 32));
+      uint64_t* dst = reinterpret_cast<uint64_t*>(lds + lane * (slot / 32));
       const uint64_t* src = stream + (size_t)(first + lane) * W;
       if ((W & 1u) == 0 && stream16) {
-        for (unsigned j = 0; j < W; j += 2)
-          *reinterpret_cast<ulonglong2*>(dst + j) = *reinterpret_cast<const ulonglong2*>(src + j);
+        for (unsigned j = 0; j < W; j += 2) {
+          const ulonglong2 v = *reinterpret_cast<const ulonglong2*>(src + j);
+          if (SLOT16) {
+            *reinterpret_cast<ulonglong2*>(dst + j) = v;
+          } else {
+            dst[j] = v.x;
+            dst[j + 1] = v.y;
+          }
+        }
       } else {
         for (unsigned j = 0; j < W; j++) dst[j] = src[j];
       }
@@ -262,8 +284,13 @@ __device__ __forceinline__ void load_region(uint32_t* lds, unsigned lane, uint32
 // region_dwords(maxbits) dwords.
 // INT: the field holds int32 values (moved as 32-bit patterns through the same loads and stores)
 // ONCE: the field is loaded with the nontemporal hint (Field3::read_once)
-template <bool WHOLE, bool INT = false, bool ONCE = false>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void zfp_encode3_f32_kernel(const float* __restrict__ in, Field3 fd,
+// WPE: wavefronts per SIMD the kernel is built for and held to.  Five, except from 16 bits
+// per value on: there a wavefront's LDS region (9 KB and more) lets 16 or 17 wavefronts
+// into a compute unit, unevenly over its SIMDs, and the encoder measured fastest with
+// three per SIMD (402.7 MB at 16 bits per value: 130-133 us against 139-140 us with four
+// or five), the decoder with four (137-140 us against 143-156 us).
+template <bool WHOLE, bool INT = false, bool ONCE = false, int WPE = 5>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void zfp_encode3_f32_kernel(const float* __restrict__ in, Field3 fd,
                                                              unsigned maxbits,
                                                              uint64_t* __restrict__ stream)
 {
@@ -298,8 +325,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void
 // and the late block coordinates below reach without spilling): measured
 // 2.5 % faster than the four that the unconstrained 105 registers allow; six
 // (80 registers) spills and is slower again.
-template <bool WHOLE, bool INT = false>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void zfp_decode3_f32_kernel(const uint64_t* __restrict__ stream, Field3 fd,
+template <bool WHOLE, bool INT = false, int WPE = 5>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void zfp_decode3_f32_kernel(const uint64_t* __restrict__ stream, Field3 fd,
                                                              unsigned maxbits, float* __restrict__ out)
 {
   extern __shared__ uint4 lds_raw[];
@@ -307,9 +334,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void
   const unsigned lane = threadIdx.x;
   const uint32_t first = blockIdx.x * 64u;
   const uint32_t valid = min(64u, fd.nblocks - first);
-  const unsigned slot = slot_bits(maxbits);
+  const unsigned slot = dec_slot_bits(maxbits);
 
-  load_region<WHOLE>(lds, lane, first, valid, maxbits, fd.stream16, stream);
+  load_region<WHOLE, false>(lds, lane, first, valid, maxbits, slot, fd.stream16, stream);
   __syncthreads();
 
   if (lane < valid) {
@@ -437,7 +464,7 @@ __global__ __launch_bounds__(64) void zfp_decode3_w64_kernel(const uint64_t* __r
   const unsigned lane = threadIdx.x;
   const uint32_t first = blockIdx.x * 64u;
   const uint32_t valid = min(64u, fd.nblocks - first);
-  load_region<WHOLE>(lds, lane, first, valid, maxbits, fd.stream16, stream);
+  load_region<WHOLE>(lds, lane, first, valid, maxbits, slot_bits(maxbits), fd.stream16, stream);
   __syncthreads();
   if (lane < valid) {
     uint64_t q[64];
@@ -700,6 +727,8 @@ extern "C" size_t cswap_zfp_stream_capacity(size_t nx, size_t ny, size_t nz, uns
 
 // element kinds of a field
 enum Elem { kF32 = 0, kI32 = 1, kF64 = 2, kI64 = 3 };
+// whole-word rates from this many bits per block of 64 values on run the 32-bit kernels built for fewer wavefronts per SIMD
+constexpr unsigned kFewerWavesFrom = 1024;
 static unsigned elem_bytes(Elem e) { return e == kF32 || e == kI32 ? 4u : 8u; }
 
 #define CSWAP_LAUNCH3(KERNEL_, T_, ARG0_, ARG3_)                                                                   \
@@ -728,7 +757,21 @@ static int compress3(const void* d_in, Elem elem, size_t nx, size_t ny, size_t n
   const bool is_int = elem == kI32 || elem == kI64;
   if (elem_bytes(elem) == 4) {
     const float* in = static_cast<const float*>(d_in);
-    if (fd.read_once && fd.rows16 && whole && !is_int)
+    const bool once = fd.read_once && fd.rows16;
+    if (whole && maxbits >= kFewerWavesFrom) {
+      if (once && !is_int)
+        hipLaunchKernelGGL((zfp_encode3_f32_kernel<true, false, true, 3>), dim3(grid), dim3(64), lds_bytes, st, in,
+                           fd, maxbits, d_stream);
+      else if (once)
+        hipLaunchKernelGGL((zfp_encode3_f32_kernel<true, true, true, 3>), dim3(grid), dim3(64), lds_bytes, st, in,
+                           fd, maxbits, d_stream);
+      else if (!is_int)
+        hipLaunchKernelGGL((zfp_encode3_f32_kernel<true, false, false, 3>), dim3(grid), dim3(64), lds_bytes, st, in,
+                           fd, maxbits, d_stream);
+      else
+        hipLaunchKernelGGL((zfp_encode3_f32_kernel<true, true, false, 3>), dim3(grid), dim3(64), lds_bytes, st, in,
+                           fd, maxbits, d_stream);
+    } else if (fd.read_once && fd.rows16 && whole && !is_int)
       hipLaunchKernelGGL((zfp_encode3_f32_kernel<true, false, true>), dim3(grid), dim3(64), lds_bytes, st, in, fd,
                          maxbits, d_stream);
     else if (fd.read_once && fd.rows16 && whole)
@@ -757,7 +800,15 @@ static int decompress3(const uint64_t* d_stream, Elem elem, size_t nx, size_t ny
   const bool is_int = elem == kI32 || elem == kI64;
   if (elem_bytes(elem) == 4) {
     float* out = static_cast<float*>(d_out);
-    CSWAP_LAUNCH3(zfp_decode3_f32_kernel, float, d_stream, out);
+    lds_bytes = (size_t)dec_region_dwords(maxbits) * 4;
+    if (whole && maxbits >= kFewerWavesFrom && !is_int)
+      hipLaunchKernelGGL((zfp_decode3_f32_kernel<true, false, 4>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd,
+                         maxbits, out);
+    else if (whole && maxbits >= kFewerWavesFrom)
+      hipLaunchKernelGGL((zfp_decode3_f32_kernel<true, true, 4>), dim3(grid), dim3(64), lds_bytes, st, d_stream, fd,
+                         maxbits, out);
+    else
+      CSWAP_LAUNCH3(zfp_decode3_f32_kernel, float, d_stream, out);
   } else {
     uint64_t* out = static_cast<uint64_t*>(d_out);
     if (fd.once64 && fd.rows16 && whole && !is_int)

@@ -12,6 +12,15 @@ struct ArrayBits {            // the bit region is the whole stream, addressed b
   void or32(unsigned d, uint32_t v) const { dw[d / 4] |= v; }
   uint32_t ld32(unsigned d) const { return dw[d / 4]; }
 };
+struct WatchedBits {          // the same for reading, remembering the highest dword that was asked for
+  const uint32_t* dw;
+  unsigned* top;
+  uint32_t ld32(unsigned d) const
+  {
+    if (d / 4 > *top) *top = d / 4;
+    return dw[d / 4];
+  }
+};
 }
 
 extern "C" {
@@ -77,24 +86,31 @@ void host_zfp_decode3(const uint64_t* stream, size_t nx, size_t ny, size_t nz, u
 }
 
 // Same decode through the fenced variant: every block is copied into a private
-// slot that is followed by one bits, as the device does for whole-word rates.
-void host_zfp_decode3_fenced(const uint64_t* stream, size_t nx, size_t ny, size_t nz, unsigned maxbits, float* out)
+// slot that is followed by 64 one bits, as the device does for whole-word rates,
+// and then by whatever the next lane's slot happens to hold (here: `junk`,
+// different for every block).  Returns the highest dword index, relative to the
+// slot, that any block read.
+unsigned host_zfp_decode3_fenced(const uint64_t* stream, size_t nx, size_t ny, size_t nz, unsigned maxbits, float* out,
+                                 uint32_t junk)
 {
   size_t mx = (nx + 3) / 4, my = (ny + 3) / 4, mz = (nz + 3) / 4;
   const unsigned W = maxbits / 64;  // maxbits % 64 == 0
-  uint32_t* slot = new uint32_t[2 * W + 8];
+  uint32_t* slot = new uint32_t[2 * W + 16];
+  unsigned top = 0;
   for (size_t b = 0; b < mx * my * mz; b++) {
     size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
     unsigned bx = nx - x0 < 4 ? nx - x0 : 4, by = ny - y0 < 4 ? ny - y0 : 4, bz = nz - z0 < 4 ? nz - z0 : 4;
     memcpy(slot, stream + b * W, 8 * (size_t)W);
-    memset(slot + 2 * W, 0xff, 32);
+    slot[2 * W] = slot[2 * W + 1] = 0xffffffffu;
+    for (unsigned d = 2 * W + 2; d < 2 * W + 16; d++) slot[d] = junk = junk * 1664525u + 1013904223u + (uint32_t)b;
     float f[64];
-    ArrayBits mem{slot};
+    WatchedBits mem{slot, &top};
     cswap::decode_block<true>(mem, 0u, maxbits, f);
     for (unsigned z = 0; z < bz; z++) for (unsigned y = 0; y < by; y++) for (unsigned x = 0; x < bx; x++)
       out[(x0 + x) + nx * ((y0 + y) + ny * (z0 + z))] = f[x + 4 * y + 16 * z];
   }
   delete[] slot;
+  return top;
 }
 
 // 2-D field a[ny][nx] (ny = 0: 1-D field a[nx])

@@ -22,7 +22,9 @@ def host():
     L = C.CDLL(SO)
     L.host_zfp_encode3.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     L.host_zfp_decode3.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
-    L.host_zfp_decode3_fenced.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
+    L.host_zfp_decode3_fenced.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p,
+                                          C.c_uint32]
+    L.host_zfp_decode3_fenced.restype = C.c_uint
     L.host_zfp_encode3_slots.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     L.host_zfp_encode3_slots.restype = C.c_uint
     L.host_transpose32.argtypes = [C.c_void_p]
@@ -95,8 +97,9 @@ def test_block_codec_matches_golden_vectors(host, golden):
         assert np.array_equal(o.view(np.uint32), dec.view(np.uint32)), (name, rate)
         if maxbits % 64 == 0:  # the variant the device uses for whole-word rates
             o2 = np.zeros_like(f)
-            host.host_zfp_decode3_fenced(g.ctypes.data, nx, ny, nz, maxbits, o2.ctypes.data)
+            top = host.host_zfp_decode3_fenced(g.ctypes.data, nx, ny, nz, maxbits, o2.ctypes.data, n)
             assert np.array_equal(o2.view(np.uint32), dec.view(np.uint32)), (name, rate, "fenced")
+            assert top < maxbits // 32 + 4, (name, rate, top)
         n += 1
     assert n >= 100
 
@@ -226,3 +229,28 @@ def test_unguarded_encoder_stays_inside_its_slack(host):
             top = host.host_zfp_encode3_slots(f.ctypes.data, nx, ny, nz, maxbits, b.ctypes.data)
             assert np.array_equal(a[:words], b), (maxbits, scale)
             assert top < maxbits // 32 + 4, (maxbits, scale, top)
+
+
+def test_fenced_decoder_ignores_what_lies_behind_its_fence(host):
+    """The device gives every lane a slot of the block's bits and 64 one bits; what
+    the decoder reads beyond those (the window it looks through is wider than what
+    it uses) belongs to the next lane.  On noise and on fields with outliers, at
+    every whole-word rate: the result does not depend on those bits, and no read
+    goes further than 128 bits past the block."""
+    rng = np.random.default_rng(12)
+    for maxbits in (64, 128, 192, 256, 512, 1024, 2048):
+        for scale in (1.0, 1e-3, 1e4):
+            f = (rng.standard_normal((8, 16, 64)) * scale).astype(np.float32)
+            f[rng.random(f.shape) < 0.1] *= 1e3
+            f[:, :4, :8] = 0.0                             # empty blocks: nothing but the fence is looked at
+            nz, ny, nx = f.shape
+            words = (nx // 4) * (ny // 4) * (nz // 4) * maxbits // 64
+            a = np.zeros(words + 2, dtype=np.uint64)
+            host.host_zfp_encode3(f.ctypes.data, nx, ny, nz, maxbits, a.ctypes.data)
+            plain = np.zeros_like(f)
+            host.host_zfp_decode3(a.ctypes.data, nx, ny, nz, maxbits, plain.ctypes.data)
+            for junk in (0, 1, 0xffffffff, 12345):
+                o = np.zeros_like(f)
+                top = host.host_zfp_decode3_fenced(a.ctypes.data, nx, ny, nz, maxbits, o.ctypes.data, junk)
+                assert np.array_equal(o.view(np.uint32), plain.view(np.uint32)), (maxbits, scale, junk)
+                assert top < maxbits // 32 + 4, (maxbits, scale, top)

@@ -311,7 +311,8 @@ def test_int32_golden_vectors(torch_cuda, golden_i32):
 
 
 @pytest.mark.parametrize("shape,maxbits", [((40, 36, 132), 512), ((33, 7, 9), 288), ((300, 260), 128), ((5000,), 40),
-                                           ((64, 64, 64), 1024)])
+                                           ((64, 64, 64), 1024),
+                                           ((32, 1024, 1024), 1024)])   # 128 MiB: loaded with the nontemporal hint
 def test_int32_fields_vs_checker(torch_cuda, shape, maxbits):
     import oracle
 
