@@ -301,10 +301,16 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) 
   const uint32_t valid = min(64u, fd.nblocks - first);
   const unsigned slot = slot_bits(maxbits);
 
+  // A wavefront in one of its memory phases (the loads here, the stores at the end) goes before
+  // the ones that are coding when both have an instruction to issue: its requests are what the
+  // compute unit's other wavefronts will be computing behind (measured on 402.7 MB: encode 100 ->
+  // 97 us at 8 bits per value, 129 -> 126 us at 16; the other way round 100 and 131 us).
   float f[64];
+  __builtin_amdgcn_s_setprio(3);
   if (lane < valid) load_block<ONCE>(in, fd, first, first + lane, f);  // in flight while the region is cleared
   zero_region(lds_raw, lane, maxbits);
   __syncthreads();
+  __builtin_amdgcn_s_setprio(0);
 
   if (lane < valid) {
     LdsBits mem(lds);
@@ -318,6 +324,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) 
     }
   }
   __syncthreads();
+  __builtin_amdgcn_s_setprio(3);
   store_region<WHOLE>(lds, lane, first, valid, maxbits, fd.stream16, stream);
 }
 
@@ -336,8 +343,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) 
   const uint32_t valid = min(64u, fd.nblocks - first);
   const unsigned slot = dec_slot_bits(maxbits);
 
+  __builtin_amdgcn_s_setprio(3);  // memory phases first, as in the encoder (here worth half a percent)
   load_region<WHOLE, false>(lds, lane, first, valid, maxbits, slot, fd.stream16, stream);
   __syncthreads();
+  __builtin_amdgcn_s_setprio(0);
 
   if (lane < valid) {
     int32_t ib[64];
@@ -356,6 +365,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) 
     uint32_t zero = 0;
     asm volatile("" : "+v"(zero) : "v"(ib[0]));
     const uint32_t b = first + __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));  // lane id again
+    __builtin_amdgcn_s_setprio(3);
     finish_and_store_block<INT>(out, fd, first, b, ib, w);
   }
 }
