@@ -609,6 +609,11 @@ extern "C" int cswap_swap_wait(cswap_engine* e, int ticket)
   if (!t) return CSWAP_E_ARG;
   if (t->state == kOnHost) return CSWAP_OK;
   if (t->state == kPrefetched && t->dev_held) return CSWAP_OK;  // landed while a prefetch held its payload
+  if (t->state == kInInFlight && t->out_pending) {  // swapped back in from its staging block before the copy had finished
+    CSWAP_HIP_TRY(hipEventSynchronize(t->ev_copy));
+    t->out_pending = false;
+    return CSWAP_OK;
+  }
   if (t->state != kOutInFlight) return CSWAP_E_STATE;
   CSWAP_HIP_TRY(hipEventSynchronize(t->ev_copy));
   land_outbound(e, *t);

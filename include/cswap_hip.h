@@ -330,7 +330,11 @@ void cswap_engine_destroy(cswap_engine* e);
 int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, size_t ny, size_t nz, int policy,
                    cswap_stream_t compute, int* ticket);
 /* Execution::post: block the host until the copy of `ticket` has finished;
- * afterwards the caller may free or overwrite the device tensor. */
+ * afterwards the caller may free or overwrite the device tensor.  Required for a
+ * raw swap only (policy NONE in cswap_swap_info), whose copy reads the tensor
+ * itself: a compressed swap has read it on `compute` by the time cswap_swap_out
+ * returns, so it may go back to a stream-ordered allocator at once and nobody
+ * has to wait.  Also answered after a cswap_swap_in that came first. */
 int cswap_swap_wait(cswap_engine* e, int ticket);
 /* Backward side: copy back on the engine's inbound copy stream (its own: both
  * directions of the link can be busy at once), then decompress into d_out on

@@ -750,6 +750,8 @@ def test_swap_in_while_the_outbound_copy_is_in_flight_reads_the_staging_block(to
                     assert eng.info(tk).state == 4
                 eng.swap_in(tk, out)
                 assert eng.info(tk).state == 3
+                if k == 2:
+                    eng.post(tk)                                         # a late wait for the outbound copy is still answered
                 eng.release(tk)                                          # at once; memory comes back when the work is done
                 assert eng.info(tk).state == 0
                 outs.append(out)
