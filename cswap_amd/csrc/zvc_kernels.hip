@@ -929,17 +929,20 @@ __global__ __launch_bounds__(64 * kSWaves) void zvc_stream_kernel(
 // Up to 32 MiB the whole tensor fits in the registers of one grid: every workgroup (one per
 // compute unit, sixteen wavefronts) loads its share once -- wavefront v of workgroup w owns R
 // consecutive rows of 64 elements --, counts it, writes its mask words, and publishes its count.
-// There is no scanner: every workgroup reads all the counts itself, one trip through memory
-// instead of two, takes the sum of those before it as its offset, and stores its non-zeros
+// There is no scanner: every workgroup reads the counts of the workgroups before it itself, one
+// trip through memory instead of two, takes their sum as its offset, and stores its non-zeros
 // straight from the registers (at these sizes the values array stays in the memory-side cache,
-// where whole-line stores through an LDS stage gain nothing).  Workgroup 0 writes the total.
+// where whole-line stores through an LDS stage gain nothing).  The last workgroup, which has
+// read every count but its own, writes the total.  Nobody waits for a workgroup with a higher
+// number than its own, so the grid makes progress however few of its workgroups the hardware
+// runs at a time (they are started in order).
 //
 // The counts live in two arrays of 256 words at the end of the workspace, used in turns: run
 // k publishes into array k & 1 and every workgroup clears its word of the other one, which
 // nobody reads any more; ws[kWsSmallRuns] counts the runs.  The grid is the same for every
 // size, so every word is cleared every time.  Failure works as in the pipeline kernel: a wait
 // that runs out raises the sticky flag, the offsets are kept inside the tensor, and the
-// wavefront that gave up writes -1 after workgroup 0 has stepped the run counter.
+// wavefront that gave up writes -1 after the last workgroup has stepped the run counter.
 constexpr int kQWaves = 16;
 constexpr int kQGroupsMax = 256;
 constexpr int kWsSmallRuns = 4;
@@ -1009,7 +1012,7 @@ __global__ __launch_bounds__(64 * kQWaves) void zvc_small_kernel(
     if (!(skip_first && w == 0)) st_status(&mine_arr[w], kTileReady | group_total);
   }
 
-  // ---- wavefront 0 collects everybody's count: lane l looks at workgroups 4l .. 4l+3
+  // ---- wavefront 0 collects the counts of the workgroups before this one: lane l looks at workgroups 4l .. 4l+3
   bool gave_up = false;
   if (wv == 0) {
     uint32_t v[4];
@@ -1019,7 +1022,7 @@ __global__ __launch_bounds__(64 * kQWaves) void zvc_small_kernel(
 #pragma unroll
       for (int r = 0; r < 4; r++) {
         const int k = 4 * (int)lane + r;
-        v[r] = k < G ? ld_status(&mine_arr[k]) : kTileReady;
+        v[r] = k < w ? ld_status(&mine_arr[k]) : kTileReady;
         missing |= (v[r] & kTileReady) == 0u;
       }
       if (__ballot(missing) == 0ull) break;
@@ -1042,7 +1045,7 @@ __global__ __launch_bounds__(64 * kQWaves) void zvc_small_kernel(
 #pragma unroll
     for (int r = 0; r < 3; r++) part += r < (w & 3) ? c[r] : 0u;
     const unsigned before_me = (unsigned)__builtin_amdgcn_readlane((int)part, w >> 2);
-    const unsigned total = (unsigned)__builtin_amdgcn_readlane((int)incl, 63);
+    const unsigned total = (unsigned)__builtin_amdgcn_readlane((int)incl, 63) + group_total;  // the last workgroup's is the tensor's
     if (lane == 0) {
       // whatever the words held: what this workgroup writes stays inside the tensor
       s_head[2] = min(before_me, (unsigned)g.n - group_total);
@@ -1051,7 +1054,7 @@ __global__ __launch_bounds__(64 * kQWaves) void zvc_small_kernel(
   }
   __syncthreads();
   uint32_t flag_late = 0;
-  if (w == 0 && threadIdx.x == 0) flag_late = ld_status(&ws[kWsFlag]);  // asked for now, looked at when the rows are out
+  if (w == G - 1 && threadIdx.x == 0) flag_late = ld_status(&ws[kWsFlag]);  // asked for now, looked at when the rows are out
 
   // ---- my non-zeros, row by row, straight from the lanes that hold them; chunk starts on the way
   unsigned at = s_head[2] + woff;
@@ -1075,11 +1078,11 @@ __global__ __launch_bounds__(64 * kQWaves) void zvc_small_kernel(
   }
 
   // ---- the result
-  if (w == 0 && threadIdx.x == 0) {
+  if (w == G - 1 && threadIdx.x == 0) {
     *nnz = (gave_up || flag_late != 0u) ? -1 : (int)s_head[3];
     __threadfence();
     __hip_atomic_fetch_add(&ws[kWsSmallRuns], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  } else if (gave_up && w != 0) {  // (wavefront 0 of another workgroup) after workgroup 0 has spoken
+  } else if (gave_up && w != G - 1) {  // (wavefront 0 of another workgroup) after the last workgroup has spoken
     for (unsigned spins = 0; ld_status(&ws[kWsSmallRuns]) == runs0 && spins < spin_limit; spins++)
       __builtin_amdgcn_s_sleep(2);
     if (lane == 0) *nnz = -1;
