@@ -167,7 +167,7 @@ int cswap_zvc_compress(const float* d_in, int n, int process, int* d_begin, int*
  * cswap_zvc_set_single_pass_bytes says (64 MiB) do not fill that pipeline; of those,
  * tensors whose mask layout has at most 131072 rows of 64 elements (32 MiB) run
  * another one-kernel form -- the whole tensor in the registers of one grid, every
- * workgroup reads everybody's count -- and the rest the three kernels.  d_ws is a
+ * workgroup reads the counts of the workgroups before it -- and the rest the three kernels.  d_ws is a
  * workspace of cswap_zvc_workspace_bytes(process) bytes (at least 256 KiB) that
  * cswap_zvc_workspace_clear has prepared once, after it was allocated; every call
  * that succeeds leaves it ready for the next one (the kernel clears each status
@@ -176,7 +176,8 @@ int cswap_zvc_compress(const float* d_in, int n, int process, int* d_begin, int*
  * length that is not a multiple of 32, for the pipeline d_values not 16-byte
  * aligned or more than 32512 tiles of 12288 elements -- run the three kernels instead.  The workgroups
  * wait for each other's counts; that wait is bounded, and if it ever runs out (for
- * example because the kernel does not get the whole GPU) the kernel still finishes
+ * example because the pipeline kernel, whose 256 workgroups all have to run at the
+ * same time, does not get the whole GPU) the kernel still finishes
  * but *d_nnz is -1 and the other outputs are undefined: a caller must treat a
  * negative count as failure (the return value cannot tell, the call does not
  * synchronise).  A workspace that was never prepared is reported the same way, and
