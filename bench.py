@@ -39,7 +39,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the two ZFP kernels on this workload, from two rocprofv3 --pmc runs
 # (FETCH_SIZE, WRITE_SIZE), each scaled by what the counter reads for a plain copy of the same tensor
 # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the summary of those runs is kept under profiles/
-HBM_TRAFFIC_BYTES_PER_LAUNCH = {"zfp_encode3_f32_kernel": 503603085, "zfp_decode3_f32_kernel": 503628556}
+HBM_TRAFFIC_BYTES_PER_LAUNCH = {"zfp_encode3_f32_kernel": 503500800, "zfp_decode3_f32_kernel": 503787520}
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
