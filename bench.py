@@ -195,7 +195,7 @@ def main():
         detail["cpu_baseline"] = cb
         result["cpu_baseline"] = {k: cb[k] for k in ("value", "unit", "cores", "kind", "sample")}
     if not args.no_extra:
-        ex = extras(torch, api, dev)
+        ex = extras(torch, api, dev, cpu=not args.no_cpu)
         detail["extra"] = ex
         result["also"] = headline_fractions(ex)
     if not args.no_extra or not args.no_cpu:
@@ -227,6 +227,9 @@ def headline_fractions(ex):
         "zvc_512MiB": pick("zvc_relu_512MiB", "compress_total_hbm_frac", "expand_hbm_frac"),
         "zvc_config2_50pct": pick("zvc_config2_s50", "compress_total_hbm_frac", "expand_hbm_frac"),
     }
+    zc = (ex.get("zvc_relu_256MiB") or {}).get("cpu_baseline")
+    if zc:     # the CPU sparse path on the 256 MiB tensor, one core: [compress, expand] GB/s of fp32
+        also["zvc_256MiB_cpu_GBs"] = [zc["one_core"]["compress_GBs_fp32"], zc["one_core"]["expand_GBs_fp32"]]
     if ex.get("box_memory_GBs"):
         also["box_copy_GBs"] = ex["box_memory_GBs"]["copy_read_plus_write"]
     sw = ex.get("swap")
@@ -332,7 +335,30 @@ def zfp_library_pair(sample, maxbits):
     return best
 
 
-def zvc_extras(torch, api, dev, ex, config2_tensor, only_mib=0):
+def zvc_cpu_baseline(t, process):
+    """The CPU checker's sparse path (count, prefix sum, compaction; expansion) on the
+    same tensor: one warm-up and the median of three runs, on one core and on all."""
+    import oracle
+
+    x = t.cpu().numpy().reshape(-1)
+    res = {"kind": "port", "sample": "the whole tensor, 1 warm-up + median of 3"}
+    for key, omp in (("one_core", False), ("all_cores", True)):
+        times = []
+        for i in range(4):
+            t0 = time.perf_counter()
+            values, mask, begin, nnz = oracle.zvc_compress(x, process, omp=omp)
+            t1 = time.perf_counter()
+            oracle.zvc_decompress(values, mask, begin, x.size, process, omp=omp)
+            t2 = time.perf_counter()
+            if i:
+                times.append((t1 - t0, t2 - t1))
+        c, e = median([a for a, _ in times]), median([b for _, b in times])
+        res[key] = {"compress_GBs_fp32": round(x.nbytes / c / 1e9, 3), "expand_GBs_fp32": round(x.nbytes / e / 1e9, 3),
+                    "cores": oracle.lib(True).orc_threads() if omp else 1}
+    return res
+
+
+def zvc_extras(torch, api, dev, ex, config2_tensor, only_mib=0, cpu=False):
     only_256 = bool(only_mib)
     # ---- ZVC compact / expand / probe
     def zvc_case(label, t):
@@ -410,7 +436,11 @@ def zvc_extras(torch, api, dev, ex, config2_tensor, only_mib=0):
     if only_mib and only_mib != 256:
         zvc_case(f"relu_{only_mib}MiB", torch.relu(torch.randn(only_mib << 18, generator=g, device=dev)))
         return ex
-    zvc_case("relu_256MiB", torch.relu(torch.randn(64 * 1024 * 1024, generator=g, device=dev)))
+    t256 = torch.relu(torch.randn(64 * 1024 * 1024, generator=g, device=dev))
+    zvc_case("relu_256MiB", t256)
+    if cpu:
+        ex["zvc_relu_256MiB"]["cpu_baseline"] = zvc_cpu_baseline(t256, api.PROCESS)
+    del t256
     # twice the size: mask and values (286 MB) no longer stay in the 256 MB memory-side cache
     # between the launches of a timing loop, as the 143 MB of the case above do
     if not only_256:
@@ -418,7 +448,7 @@ def zvc_extras(torch, api, dev, ex, config2_tensor, only_mib=0):
     return ex
 
 
-def extras(torch, api, dev, zvc_only=0):
+def extras(torch, api, dev, zvc_only=0, cpu=False):
     import numpy as np
 
     from cswap_amd.workloads import config1_field, config2_tensor, field_dims
@@ -509,7 +539,7 @@ def extras(torch, api, dev, zvc_only=0):
             "decompress_hbm_frac": round(bpv * n / d / 1e6 / HBM_PEAK_GBS, 4)}
     del base
 
-    zvc_extras(torch, api, dev, ex, config2_tensor)
+    zvc_extras(torch, api, dev, ex, config2_tensor, cpu=cpu)
 
     try:
         from cswap_amd import swap

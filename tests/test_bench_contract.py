@@ -72,8 +72,10 @@ def test_the_drivers_command_prints_a_short_last_line(tmp_path):
     _check_line(r, 20, 5)
     assert "extra" not in r and r["also"]
     assert r["also"]["box_copy_GBs"] > 1000                  # what a plain device copy reaches on this box
+    assert len(r["also"]["zvc_256MiB_cpu_GBs"]) == 2         # the CPU sparse path beside the ZVC figures
     for pair in r["also"].values():
         vals = pair.values() if isinstance(pair, dict) else (pair if isinstance(pair, list) else [pair])
         assert all(v > 0 for v in vals)
     full = json.loads(extra.read_text())
     assert full["value"] == r["value"] and "zvc_relu_512MiB" in full["extra"] and "swap" in full["extra"]
+    assert full["extra"]["zvc_relu_256MiB"]["cpu_baseline"]["all_cores"]["cores"] >= 1
