@@ -896,11 +896,25 @@ CSWAP_HD void inv_lift4_biased(int32_t& x, int32_t& y, int32_t& z, int32_t& w, u
   { int32_t w0 = w; w = wadd(w, x); x = wsub(x, w0); }
 }
 
+// Issue priority of the wavefront from here on, against the other wavefronts of its SIMD
+// (s_setprio; nothing on the host).
+template <int P>
+CSWAP_HD void issue_priority()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_s_setprio(P);
+#endif
+}
+
+// The caller runs the bit planes at the highest issue priority: that part is one dependent
+// chain through LDS reads per block, and every slot it waits for is added to its length.  The
+// lifting that follows is independent work that fills whatever slots are left, at the lowest.
 template <class Dec>
 CSWAP_HD void decode_ints3_zy(Dec& dec, int32_t (&ib)[64])
 {
   uint32_t lo[32], hi[32];
   const uint32_t c = decode_planes32(dec, lo, hi);
+  issue_priority<0>();
 #pragma unroll
   for (int i = 0; i < 32; i++) {  // still with the negabinary constant added: the z pass takes it out
     ib[kPerm3.v[i]] = (int32_t)lo[i];
