@@ -952,6 +952,7 @@ CSWAP_HD void decode_ints3(Dec& dec, int64_t (&ib)[64])
   }
 #pragma unroll
   for (int i = 0; i < 64; i++) ib[i] = (int64_t)((uint64_t)ib[i] - c);
+  issue_priority<0>();  // as in decode_ints3_zy: the planes above went first, the lifting fills in
   inv_xform3(ib);
 }
 

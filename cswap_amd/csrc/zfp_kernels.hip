@@ -479,12 +479,14 @@ __global__ __launch_bounds__(64) void zfp_decode3_w64_kernel(const uint64_t* __r
   const unsigned lane = threadIdx.x;
   const uint32_t first = blockIdx.x * 64u;
   const uint32_t valid = min(64u, fd.nblocks - first);
+  __builtin_amdgcn_s_setprio(3);  // the 32-bit decoder's priorities (here, at two wavefronts per SIMD, worth 2.6 %)
   load_region<WHOLE>(lds, lane, first, valid, maxbits, slot_bits(maxbits), fd.stream16, stream);
   __syncthreads();
   if (lane < valid) {
     uint64_t q[64];
     LdsBits mem(lds);
     decode_block_w64<INT, WHOLE>(mem, mem.bit0 + lane * slot_bits(maxbits), maxbits, q);
+    __builtin_amdgcn_s_setprio(1);
     store_block_w64<ONCE>(out, fd, first + lane, q);
   }
 }
