@@ -90,6 +90,7 @@ _SIGNATURES = {
     "cswap_zfp_decompress_f64_nd": (i32, [vp, i32, sz, sz, sz, pd, pd, pd, u, vp, vp]),
     "cswap_zfp_compress_i64_nd": (i32, [vp, i32, sz, sz, sz, pd, pd, pd, u, vp, vp]),
     "cswap_zfp_decompress_i64_nd": (i32, [vp, i32, sz, sz, sz, pd, pd, pd, u, vp, vp]),
+    "cswap_zfp_set_pair_bytes": (None, [sz, sz, C.POINTER(sz)]),
     "cswap_zvc_chunk_elems": (i32, [i32, i32]),
     "cswap_zvc_chunk_words": (i32, [i32, i32]),
     "cswap_zvc_active_chunks": (i32, [i32, i32]),

@@ -524,6 +524,24 @@ struct BlockEncoder {
     }
     plane(x);
   }
+
+  // Advances the state over a plane that somebody else codes (a block shared by two
+  // wavefronts): the same n and pos that plane(x) leaves behind, in closed form.  acc is
+  // the OR of every plane so far (n is one more than the index of its highest one-bit).
+  // A plane costs its n verbatim bits; for every one-bit at or above n a positive group
+  // test, the zeros before it and the bit itself, which is n_new - n value bits and
+  // popcount tests; and a negative test at the end -- unless the last coefficient was
+  // reached, which also saves that coefficient's one-bit (encode.cuh:331-344).
+  CSWAP_HD void skip_plane(uint64_t x, uint64_t& acc)
+  {
+    static_assert(SIZE == 64, "the closed form is written for blocks of 64 coefficients");
+    const uint64_t rest = n < 64 ? x >> n : 0;
+    acc |= x;
+    const unsigned n_new = acc ? 64u - (unsigned)__builtin_clzll(acc) : 0u;
+    const unsigned tests = (unsigned)__builtin_popcountll(rest);
+    pos += n_new + tests + (n_new < 64 ? 1u : (n < 64 ? ~0u : 0u));
+    n = n_new;
+  }
 };
 
 // 32 bit planes of 64 coefficients.  lo / hi hold the 32-bit words of the
@@ -719,6 +737,217 @@ CSWAP_HD void encode_block_w64(const uint64_t (&q)[64], unsigned pos0, unsigned 
     for (int i = 0; i < 64; i++) ib[i] = sat_i64(s * f64_from_bits(q[i]));
   }
   encode_ints3(ib, enc, kmin);
+}
+
+// ---------------------------------------------------------------- one block, two wavefronts
+// The "pair" form of the encoder, for fields that are too small to fill the chip with one
+// lane per block: a block is shared by lane l of two wavefronts (halves 0 and 1 of a
+// workgroup), each of which does half of every phase, so that twice as many wavefronts
+// with half the serial work each are in flight.  The halves exchange data through an
+// Exchange object (LDS and workgroup barriers on the device, shared arrays and a thread
+// barrier in the host build that the CPU tests run).  Results are those of encode_block.
+//
+//  load      half 0 holds the z-slices 0 and 3 of the block (p, q), half 1 the slices 2 and 1
+//  maximum   each half over its 32 values, exchanged                          (exchange 1)
+//  cast, lifting along x and y of both slices: no exchange
+//  lifting along z (fwd_lift4 on (x, y, z, w) = slices 0, 1, 2, 3): its first two lines pair
+//            slice 0 with 3 and slice 2 with 1, which is what each half holds; the rest pairs
+//            x with z and w with y, so half 0 sends w and gets z, half 1 the reverse
+//                                                                              (exchange 2)
+//            half 0 ends with the coefficients of z-index 0 and 2, half 1 with 1 and 3
+//  reorder   half 0 needs the coefficients 0..31 in coding order, half 1 the others: 19 of
+//            the 32 that a half holds stay (a register renaming), 13 change sides  (exchange 3)
+//  planes    each half transposes its 32 coefficients: its 32 bits of every plane  (exchange 4)
+//  coder     both halves walk all planes; half 0 codes the odd ones, half 1 the even ones, and
+//            each steps over the other's planes in closed form (BlockEncoder::skip_plane).
+//            Both OR into the same bit region, which therefore has to take ORs from two
+//            wavefronts (LDS atomics do).
+struct SeqOf {
+  int v[64];
+};
+constexpr SeqOf make_seq_of()
+{
+  SeqOf s = {};
+  for (int i = 0; i < 64; i++) s.v[kPerm3.v[i]] = i;
+  return s;
+}
+constexpr SeqOf kSeqOf = make_seq_of();  // position in coding order of the coefficient x + 4y + 16z
+
+// Slot r (0..31) of what a half holds after the z pass: r < 16 is its own slice register
+// (z-index 0 for half 0, 1 for half 1), r >= 16 the one that came from the partner and
+// was finished here (z-index 2 for half 0, 3 for half 1); r & 15 = x + 4y.
+template <int H>
+struct PairMap {
+  static constexpr int natural(int r) { return (r & 15) + 16 * (H == 0 ? (r < 16 ? 0 : 2) : (r < 16 ? 1 : 3)); }
+  static constexpr bool stays(int r) { return (kSeqOf.v[natural(r)] >> 5) == H; }
+  static constexpr int row(int r) { return kSeqOf.v[natural(r)] & 31; }  // row of the 32-row array of whoever gets it
+  static constexpr int sent_before(int r)
+  {
+    int j = 0;
+    for (int q = 0; q < r; q++) j += stays(q) ? 0 : 1;
+    return j;
+  }
+};
+constexpr int kPairSent = PairMap<0>::sent_before(32);
+static_assert(kPairSent == 13 && PairMap<1>::sent_before(32) == 13, "13 coefficients change sides in each direction");
+
+CSWAP_HD float pair_max(const float (&p)[16], const float (&q)[16])
+{
+  float m = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 16; i++) m = fmaxf(m, fmaxf(fabsf(p[i]), fabsf(q[i])));
+  return m;
+}
+
+// cast, lifting along x and y of both slices, and the first two lines of the lifting along z
+CSWAP_HD void pair_cast_xy_z1(float s, const float (&p)[16], const float (&q)[16], int32_t (&ip)[16], int32_t (&iq)[16])
+{
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    ip[i] = (int32_t)(s * p[i]);
+    iq[i] = (int32_t)(s * q[i]);
+  }
+#pragma unroll
+  for (int y = 0; y < 4; y++) {
+    fwd_lift4(ip[4 * y], ip[4 * y + 1], ip[4 * y + 2], ip[4 * y + 3]);
+    fwd_lift4(iq[4 * y], iq[4 * y + 1], iq[4 * y + 2], iq[4 * y + 3]);
+  }
+#pragma unroll
+  for (int x = 0; x < 4; x++) {
+    fwd_lift4(ip[x], ip[x + 4], ip[x + 8], ip[x + 12]);
+    fwd_lift4(iq[x], iq[x + 4], iq[x + 8], iq[x + 12]);
+  }
+#pragma unroll
+  for (int i = 0; i < 16; i++) {  // half 0: x += w; x >>= 1; w -= x.  half 1: z += y; z >>= 1; y -= z.
+    ip[i] = wadd(ip[i], iq[i]);
+    ip[i] >>= 1;
+    iq[i] = wsub(iq[i], ip[i]);
+  }
+}
+
+// the rest of the lifting along z; c receives the half's 32 coefficients in PairMap order
+template <int H>
+CSWAP_HD void pair_z2(const int32_t (&ip)[16], const int32_t (&iq)[16], const int32_t (&got)[16], int32_t (&c)[32])
+{
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    if (H == 0) {  // x = ip, z = got:  x += z; x >>= 1; z -= x
+      int32_t x = wadd(ip[i], got[i]);
+      x >>= 1;
+      c[i] = x;
+      c[16 + i] = wsub(got[i], x);
+    } else {       // w = got, y = iq:  w += y; w >>= 1; y -= w; w += y >> 1; y -= w >> 1
+      int32_t w = wadd(got[i], iq[i]);
+      w >>= 1;
+      int32_t y = wsub(iq[i], w);
+      w = wadd(w, y >> 1);
+      y = wsub(y, w >> 1);
+      c[i] = y;
+      c[16 + i] = w;
+    }
+  }
+}
+
+// the half's 32 bits of the planes 31..16: rows 16..31 of a afterwards (rows 0..15 keep what
+// pair_low_planes needs)
+CSWAP_HD void pair_top_planes(uint32_t (&a)[32])
+{
+  tr_stage<16, 0, 32>(a);
+  settle16<0>(a);
+  tr_stage<8, 16, 32>(a);
+  settle16<16>(a);
+  tr_stage<4, 16, 32, kPlain, true>(a);
+  settle16<16>(a);
+  tr_stage<2, 16, 32, kPlain, true>(a);
+  settle16<16>(a);
+  tr_stage<1, 16, 32, kNotOut, true>(a);
+}
+CSWAP_HD void pair_low_planes(uint32_t (&a)[32]) { tr_half<0, kNotOut>(a); }
+
+// 16 planes, highest first (x[15] .. x[0]); half 0 codes the odd ones.  top: these are the
+// planes 31..16, of which the first four get the treatment of leading planes.
+template <int H, class Enc>
+CSWAP_HD void pair_code16(const uint64_t (&x)[16], Enc& enc, uint64_t& acc, bool top)
+{
+#pragma unroll
+  for (int k = 15; k >= 0; k--) {
+    if ((k & 1) == (H == 0 ? 1 : 0)) {
+      if (top && k >= 12) enc.leading_plane(x[k]);
+      else enc.plane(x[k]);
+      acc |= x[k];
+    } else {
+      enc.skip_plane(x[k], acc);
+    }
+  }
+}
+
+// One half's share of a block.  p, q: the half's two z-slices ([x + 4y]; half 0: z = 0 and 3,
+// half 1: z = 2 and 1); live: false for the lanes past the end of the field (they go through
+// every exchange and write nothing).  The block owns [pos0, pos0 + maxbits) of the zeroed bit
+// region behind mem plus 128 bits of slack (unguarded coder).
+//
+// Exchange (every call is made by both halves, in this order):
+//   float    other_max(float)                      my maximum out, the partner's back
+//   void     swap16(const int32_t(&)[16], int32_t(&)[16])
+//   void     seq_put(int slot, uint32_t), seq_sync(), uint32_t seq_get(int slot)
+//   void     plane_put(int k, uint32_t), plane_sync(), uint64_t plane_get(int k)   (both halves' words)
+//   bool     more(bool)                            half 0's answer for both; also orders the
+//                                                  coder's writes before what follows
+//   void     done()                                after the low planes, if more() said yes
+template <int H, class Ex, class Mem>
+CSWAP_HD void pair_encode_half(const float (&p)[16], const float (&q)[16], bool live, unsigned pos0, unsigned maxbits,
+                               Mem& mem, Ex& ex)
+{
+  const float mine = pair_max(p, q);
+  const uint32_t mb = f32_bits(fmaxf(mine, ex.other_max(mine)));
+  const uint32_t e = (live && mb) ? (mb >> 23) + 1 : 0;  // as block_header_e
+  const float s = e ? pow2f(30 - ((int)e - 127)) : 0.0f;
+
+  int32_t ip[16], iq[16], got[16], c[32];
+  pair_cast_xy_z1(s, p, q, ip, iq);
+  ex.swap16(H == 0 ? iq : ip, got);
+  pair_z2<H>(ip, iq, got, c);
+
+  uint32_t a[32];
+#pragma unroll
+  for (int r = 0; r < 32; r++) {  // negabinary: the add here, the xor inside the transpose
+    const uint32_t u = (uint32_t)c[r] + kNegabinary;
+    if (PairMap<H>::stays(r)) a[PairMap<H>::row(r)] = u;
+    else ex.seq_put(PairMap<H>::sent_before(r), u);
+  }
+  ex.seq_sync();
+#pragma unroll
+  for (int r = 0; r < 32; r++)
+    if (!PairMap<1 - H>::stays(r)) a[PairMap<1 - H>::row(r)] = ex.seq_get(PairMap<1 - H>::sent_before(r));
+
+  pair_top_planes(a);
+#pragma unroll
+  for (int k = 0; k < 16; k++) ex.plane_put(k, a[16 + k]);
+  ex.plane_sync();
+  uint64_t x[16];
+#pragma unroll
+  for (int k = 0; k < 16; k++) x[k] = ex.plane_get(k);
+
+  BlockEncoder<Mem, false> enc(mem, pos0, maxbits);
+  if (e == 0) {
+    enc.pos = enc.limit;  // an all-zero block (encode.cuh:357-358) or a lane past the end: nothing is written
+  } else if (H == 0) {
+    enc.put(2 * e + 1, 9);
+  } else {
+    enc.pos += 9;
+  }
+  uint64_t acc = 0;
+  pair_code16<H>(x, enc, acc, true);
+  if (ex.more(CSWAP_ANY(enc.active()))) {
+    pair_low_planes(a);
+#pragma unroll
+    for (int k = 0; k < 16; k++) ex.plane_put(k, a[k]);
+    ex.plane_sync();
+#pragma unroll
+    for (int k = 0; k < 16; k++) x[k] = ex.plane_get(k);
+    pair_code16<H>(x, enc, acc, false);
+    ex.done();
+  }
 }
 
 // ---------------------------------------------------------------- decoder

@@ -11,6 +11,7 @@
 // the stream is needed (the reference pre-zeroes the stream and adds every bit
 // with a global atomic, CSWAP+/zfp/encode.cuh:252-299, encode3.cuh:152).
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include "../../include/cswap_hip.h"
 #include "zfp_block.h"
 #include "common.h"
@@ -35,6 +36,14 @@ struct Field3 {
 #define CSWAP_READ_ONCE_BYTES (128ull << 20)
 #endif
 constexpr unsigned long long kReadOnceBytes = CSWAP_READ_ONCE_BYTES;
+
+// Fields below this many bytes are coded by the pair form (two wavefronts per 64 blocks)
+#ifndef CSWAP_PAIR_ENCODE_BYTES
+#define CSWAP_PAIR_ENCODE_BYTES (40ull << 20)
+#endif
+#ifndef CSWAP_PAIR_DECODE_BYTES
+#define CSWAP_PAIR_DECODE_BYTES 0ull
+#endif
 
 // 16 bytes of the field as the compiler's own vector type (what the nontemporal builtins take)
 typedef float stream_f4 __attribute__((ext_vector_type(4)));
@@ -372,6 +381,136 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) 
     const uint32_t b = first + __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));  // lane id again
     __builtin_amdgcn_s_setprio(1);
     finish_and_store_block<INT>(out, fd, first, b, ib, w);
+  }
+}
+
+// ------------------------------------------------------------- the pair form: two wavefronts per 64 blocks
+// For fields that are too small to fill the chip with one lane per block.  A workgroup is two
+// wavefronts; lane l of both works on block first + l, each doing its half of every phase
+// (zfp_block.h: pair_encode_half), so that a field keeps twice as many wavefronts in flight,
+// each with half the serial work.  Fast path only: whole-word rates with an even number of
+// 16-byte pieces per block, full blocks, 16-byte aligned contiguous rows.
+//
+// Dynamic LDS, in dwords: [region: region_dwords(maxbits)] [maxima: 128] [flag: 4]
+// [U0: 1280] [U1: 1280].  U0 and U1 carry all three later exchanges in turn, and the rule
+// that makes this safe without barriers of its own is that a half only ever writes into the
+// one it was the last to read:
+//   z exchange   half h writes U_h (lane * 20 + j, four 16-byte pieces)        barrier  reads U_(1-h)
+//   reorder      writes the 13 coefficients it sends into U_(1-h) (slot * 64 + lane)
+//                                                                               barrier  reads U_h
+//   planes       writes its 32 bits of 16 planes into U_h (k * 64 + lane)      barrier  reads both
+constexpr unsigned kPairMaxima = 128, kPairFlag = 4, kPairU = 1280;
+__host__ __device__ inline unsigned pair_lds_dwords(unsigned maxbits)
+{
+  return region_dwords(maxbits) + kPairMaxima + kPairFlag + 2 * kPairU;
+}
+
+template <int H>
+struct LdsExchange {
+  float* maxima;
+  uint32_t* flag;
+  uint32_t* mine;    // U_H
+  uint32_t* theirs;  // U_(1-H)
+  unsigned lane;
+  __device__ __forceinline__ float other_max(float m)
+  {
+    maxima[H * 64 + lane] = m;
+    __syncthreads();
+    return maxima[(1 - H) * 64 + lane];
+  }
+  __device__ __forceinline__ void swap16(const int32_t (&out)[16], int32_t (&in)[16])
+  {
+    uint4* dst = reinterpret_cast<uint4*>(mine + lane * 20);
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      dst[j] = make_uint4((uint32_t)out[4 * j], (uint32_t)out[4 * j + 1], (uint32_t)out[4 * j + 2], (uint32_t)out[4 * j + 3]);
+    __syncthreads();
+    const uint4* src = reinterpret_cast<const uint4*>(theirs + lane * 20);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const uint4 v = src[j];
+      in[4 * j] = (int32_t)v.x;
+      in[4 * j + 1] = (int32_t)v.y;
+      in[4 * j + 2] = (int32_t)v.z;
+      in[4 * j + 3] = (int32_t)v.w;
+    }
+  }
+  __device__ __forceinline__ void seq_put(int slot, uint32_t v) { theirs[slot * 64 + lane] = v; }
+  __device__ __forceinline__ void seq_sync() { __syncthreads(); }
+  __device__ __forceinline__ uint32_t seq_get(int slot) { return mine[slot * 64 + lane]; }
+  __device__ __forceinline__ void plane_put(int k, uint32_t v) { mine[k * 64 + lane] = v; }
+  __device__ __forceinline__ void plane_sync() { __syncthreads(); }
+  __device__ __forceinline__ uint64_t plane_get(int k)
+  {
+    const uint32_t* u0 = H == 0 ? mine : theirs;
+    const uint32_t* u1 = H == 0 ? theirs : mine;
+    return ((uint64_t)u1[k * 64 + lane] << 32) | u0[k * 64 + lane];
+  }
+  // Half 0 answers for both, so that the two can never disagree about the barriers ahead.
+  __device__ __forceinline__ bool more(bool any)
+  {
+    if (H == 0 && lane == 0) *flag = any ? 1u : 0u;
+    __syncthreads();
+    return __builtin_amdgcn_readfirstlane(*flag) != 0;
+  }
+  __device__ __forceinline__ void done() { __syncthreads(); }
+};
+
+template <int H>
+__device__ __forceinline__ void pair_encode_body(const float* __restrict__ in, const Field3& fd, unsigned maxbits,
+                                                 uint32_t* lds, unsigned lane, uint32_t first)
+{
+  const bool live = first + lane < fd.nblocks;
+  const uint32_t b = live ? first + lane : fd.nblocks - 1;
+  float p[16], q[16];
+  {
+    uint32_t x0, y0, z0;
+    block_origin(fd, b, x0, y0, z0);
+    const WaveBase w = wave_base(fd, first);
+    const char* base = reinterpret_cast<const char*>(in + w.origin);
+    const uint32_t me = lane_bytes(fd, w, x0, y0, z0);
+    const uint32_t sy4 = (uint32_t)fd.sy * 4u, sz4 = (uint32_t)fd.sz * 4u;
+    constexpr int ZP = H == 0 ? 0 : 2, ZQ = H == 0 ? 3 : 1;
+#pragma unroll
+    for (int y = 0; y < 4; y++) {
+      const stream_f4 vp = *reinterpret_cast<const stream_f4*>(base + (size_t)(me + (y * sy4 + ZP * sz4)));
+      const stream_f4 vq = *reinterpret_cast<const stream_f4*>(base + (size_t)(me + (y * sy4 + ZQ * sz4)));
+      p[4 * y] = vp.x; p[4 * y + 1] = vp.y; p[4 * y + 2] = vp.z; p[4 * y + 3] = vp.w;
+      q[4 * y] = vq.x; q[4 * y + 1] = vq.y; q[4 * y + 2] = vq.z; q[4 * y + 3] = vq.w;
+    }
+  }
+  const unsigned region = region_dwords(maxbits);
+  LdsExchange<H> ex;
+  ex.maxima = reinterpret_cast<float*>(lds + region);
+  ex.flag = lds + region + kPairMaxima;
+  ex.mine = lds + region + kPairMaxima + kPairFlag + H * kPairU;
+  ex.theirs = lds + region + kPairMaxima + kPairFlag + (1 - H) * kPairU;
+  ex.lane = lane;
+  LdsBits mem(lds);
+  pair_encode_half<H>(p, q, live, mem.bit0 + lane * slot_bits(maxbits), maxbits, mem, ex);
+}
+
+__global__ __launch_bounds__(128) void zfp_encode3_f32_pair_kernel(const float* __restrict__ in, Field3 fd,
+                                                                   unsigned maxbits, uint64_t* __restrict__ stream)
+{
+  extern __shared__ uint4 lds_raw[];
+  uint32_t* lds = reinterpret_cast<uint32_t*>(lds_raw);
+  const unsigned tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t first = blockIdx.x * 64u;
+  {  // the region starts out zero; the first exchange's barrier orders this before any coder's OR
+    const unsigned n16 = region_dwords(maxbits) / 4;
+    for (unsigned i = tid; i < n16; i += 128) lds_raw[i] = make_uint4(0, 0, 0, 0);
+  }
+  if (__builtin_amdgcn_readfirstlane(tid >> 6) == 0) pair_encode_body<0>(in, fd, maxbits, lds, lane, first);
+  else pair_encode_body<1>(in, fd, maxbits, lds, lane, first);
+  // Both halves are past the barrier of more() or done(): every block is coded.  Thread t
+  // moves half of block t / 2 (W / 2 words, W / 4 16-byte pieces).
+  const uint32_t blk = first + (tid >> 1);
+  if (blk < fd.nblocks) {
+    const unsigned W = maxbits >> 6;
+    const ulonglong2* src = reinterpret_cast<const ulonglong2*>(lds + (tid >> 1) * (slot_bits(maxbits) / 32) + (tid & 1u) * W);
+    ulonglong2* dst = reinterpret_cast<ulonglong2*>(stream + (size_t)blk * W + (tid & 1u) * (W / 2));
+    for (unsigned j = 0; j < W / 4; j++) dst[j] = src[j];
   }
 }
 
@@ -748,6 +887,30 @@ enum Elem { kF32 = 0, kI32 = 1, kF64 = 2, kI64 = 3 };
 constexpr unsigned kFewerWavesFrom = 1024;
 static unsigned elem_bytes(Elem e) { return e == kF32 || e == kI32 ? 4u : 8u; }
 
+// Fields below this many bytes are coded by the pair form where their shape allows
+// (cswap_zfp_set_pair_bytes).
+static std::atomic<unsigned long long> g_pair_encode_bytes{CSWAP_PAIR_ENCODE_BYTES};
+
+// what the pair kernels take: the fast path of the field (aligned contiguous rows, an aligned
+// stream), full blocks only, and a whole-word rate whose blocks split into two halves of
+// whole 16-byte pieces
+static bool pair_shape(const Field3& fd, unsigned maxbits)
+{
+  return fd.rows16 && fd.stream16 && (maxbits & 255u) == 0 && ((fd.nx | fd.ny | fd.nz) & 3u) == 0;
+}
+
+static std::atomic<unsigned long long> g_pair_decode_bytes{CSWAP_PAIR_DECODE_BYTES};
+
+extern "C" void cswap_zfp_set_pair_bytes(size_t encode_below, size_t decode_below, size_t* previous)
+{
+  const size_t e = (size_t)g_pair_encode_bytes.exchange(encode_below, std::memory_order_relaxed);
+  const size_t d = (size_t)g_pair_decode_bytes.exchange(decode_below, std::memory_order_relaxed);
+  if (previous) {
+    previous[0] = e;
+    previous[1] = d;
+  }
+}
+
 #define CSWAP_LAUNCH3(KERNEL_, T_, ARG0_, ARG3_)                                                                   \
   do {                                                                                                              \
     if (whole && !is_int)                                                                                           \
@@ -772,6 +935,12 @@ static int compress3(const void* d_in, Elem elem, size_t nx, size_t ny, size_t n
   hipStream_t st = (hipStream_t)stream;
   const bool whole = (maxbits & 63u) == 0;
   const bool is_int = elem == kI32 || elem == kI64;
+  if (elem == kF32 && pair_shape(fd, maxbits) &&
+      (unsigned long long)nx * ny * nz * 4ull < g_pair_encode_bytes.load(std::memory_order_relaxed)) {
+    hipLaunchKernelGGL(zfp_encode3_f32_pair_kernel, dim3(grid), dim3(128), (size_t)pair_lds_dwords(maxbits) * 4, st,
+                       static_cast<const float*>(d_in), fd, maxbits, d_stream);
+    return check_launch();
+  }
   if (elem_bytes(elem) == 4) {
     const float* in = static_cast<const float*>(d_in);
     const bool once = fd.read_once && fd.rows16;

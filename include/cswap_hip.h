@@ -108,6 +108,17 @@ int cswap_zfp_decompress_i64_nd(const uint64_t* d_stream, int dims, size_t nx, s
                                 ptrdiff_t sx, ptrdiff_t sy, ptrdiff_t sz, unsigned maxbits,
                                 int64_t* d_out, cswap_stream_t stream);
 
+/* No counterpart in the reference (which launches one thread per block whatever the
+ * field's size, encode3.cuh:149-151, decode3.cuh:139-141).  A field of fewer than about
+ * a million blocks does not fill this GPU with one lane per block; below these sizes in
+ * bytes (of the uncompressed fp32 field) the 3-D fp32 kernels run in their pair form
+ * instead -- two wavefronts share 64 blocks, each doing half of every phase -- where the
+ * shape allows it: extents that are multiples of 4, contiguous 16-byte aligned rows, a
+ * 16-byte aligned stream, maxbits a multiple of 256.  Same stream, same values.
+ * 0 = never, SIZE_MAX = whenever the shape allows.  `previous`, if not NULL, receives
+ * the two values that were in force.  Process-wide. */
+void cswap_zfp_set_pair_bytes(size_t encode_below, size_t decode_below, size_t* previous);
+
 /* ------------------------------------------------------------------ ZVC -----
  * Zero-value compaction in the reference's format (zfp/compression.cu).  The
  * tensor of n fp32 elements is cut into `process` chunks of

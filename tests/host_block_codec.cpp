@@ -1,6 +1,7 @@
 // Host build of the product's per-block ZFP codec (cswap_amd/csrc/zfp_block.h),
 // so the exact code each GPU lane runs can be compared with the CPU checker
 // without a GPU.  Field walking here is deliberately naive.
+#include <pthread.h>
 #include <stddef.h>
 #include <string.h>
 #include <vector>
@@ -290,4 +291,113 @@ void host_zfp_decode_w64(const uint64_t* stream, int is_int, int dims, size_t nx
   }
 }
 
+}
+
+// ---- the encoder's pair form (a block shared by two wavefronts): two host threads stand for
+// the two halves, a thread barrier for the workgroup barrier, and the shared words are laid
+// out and reused exactly as the kernel reuses its LDS (a half writes what it sends for the
+// reorder over what it has just read of the z exchange, and its plane words over what it has
+// just read of the reorder), so a step that overwrote something the partner still needs, or a
+// barrier one half takes and the other does not, shows up here: as a wrong stream or as a
+// test that never ends.
+namespace {
+struct AtomicBits {
+  uint32_t* dw;
+  void or32(unsigned d, uint32_t v) const { __atomic_fetch_or(&dw[d / 4], v, __ATOMIC_RELAXED); }
+  uint32_t ld32(unsigned d) const { return dw[d / 4]; }
+};
+struct PairShared {
+  float mx[2];
+  uint32_t u[2][16];
+  int flag;
+  pthread_barrier_t bar;
+};
+template <int H>
+struct HostExchange {
+  PairShared& sh;
+  void wait() { pthread_barrier_wait(&sh.bar); }
+  float other_max(float m) { sh.mx[H] = m; wait(); return sh.mx[1 - H]; }
+  void swap16(const int32_t (&out)[16], int32_t (&in)[16])
+  {
+    for (int i = 0; i < 16; i++) sh.u[H][i] = (uint32_t)out[i];
+    wait();
+    for (int i = 0; i < 16; i++) in[i] = (int32_t)sh.u[1 - H][i];
+  }
+  void seq_put(int slot, uint32_t v) { sh.u[1 - H][slot] = v; }
+  void seq_sync() { wait(); }
+  uint32_t seq_get(int slot) { return sh.u[H][slot]; }
+  void plane_put(int k, uint32_t v) { sh.u[H][k] = v; }
+  void plane_sync() { wait(); }
+  uint64_t plane_get(int k) { return ((uint64_t)sh.u[1][k] << 32) | sh.u[0][k]; }
+  bool more(bool mine) { if (H == 0) sh.flag = mine; wait(); return sh.flag != 0; }
+  void done() { wait(); }
+};
+struct PairJob {
+  const float* in; size_t nx, ny, nz; unsigned maxbits; uint32_t* slots; unsigned slot_dwords; PairShared* sh;
+};
+template <int H>
+void* pair_thread(void* arg)
+{
+  PairJob& j = *static_cast<PairJob*>(arg);
+  const size_t mx = j.nx / 4, my = j.ny / 4, mz = j.nz / 4;
+  HostExchange<H> ex{*j.sh};
+  for (size_t b = 0; b < mx * my * mz; b++) {
+    const size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
+    const int zp = H == 0 ? 0 : 2, zq = H == 0 ? 3 : 1;
+    float p[16], q[16];
+    for (int y = 0; y < 4; y++) for (int x = 0; x < 4; x++) {
+      p[x + 4 * y] = j.in[(x0 + x) + j.nx * ((y0 + y) + j.ny * (z0 + zp))];
+      q[x + 4 * y] = j.in[(x0 + x) + j.nx * ((y0 + y) + j.ny * (z0 + zq))];
+    }
+    AtomicBits mem{j.slots + b * j.slot_dwords};
+    cswap::pair_encode_half<H>(p, q, true, 0u, j.maxbits, mem, ex);
+  }
+  return nullptr;
+}
+}
+
+extern "C" {
+// nx, ny, nz multiples of 4; maxbits a multiple of 64.  Returns the highest dword index
+// (relative to its slot) that any block wrote a non-zero value to, or ~0u on a setup error.
+unsigned host_zfp_encode3_pair(const float* in, size_t nx, size_t ny, size_t nz, unsigned maxbits, uint64_t* stream)
+{
+  if (nx % 4 || ny % 4 || nz % 4 || maxbits % 64) return ~0u;
+  const size_t nb = (nx / 4) * (ny / 4) * (nz / 4);
+  const unsigned W = maxbits / 64, slot_dwords = 2 * W + 4 + 8;
+  std::vector<uint32_t> slots(nb * slot_dwords, 0u);
+  PairShared sh;
+  memset(&sh, 0, sizeof sh);
+  if (pthread_barrier_init(&sh.bar, nullptr, 2)) return ~0u;
+  PairJob job{in, nx, ny, nz, maxbits, slots.data(), slot_dwords, &sh};
+  pthread_t t0, t1;
+  pthread_create(&t0, nullptr, pair_thread<0>, &job);
+  pthread_create(&t1, nullptr, pair_thread<1>, &job);
+  pthread_join(t0, nullptr);
+  pthread_join(t1, nullptr);
+  pthread_barrier_destroy(&sh.bar);
+  unsigned top = 0;
+  for (size_t b = 0; b < nb; b++) {
+    memcpy(stream + b * W, slots.data() + b * slot_dwords, 8 * (size_t)W);
+    for (unsigned d = 0; d < slot_dwords; d++) if (slots[b * slot_dwords + d] && d > top) top = d;
+  }
+  return top;
+}
+
+// BlockEncoder::skip_plane against BlockEncoder::plane on one plane: starting from n known
+// coefficients (acc = their mask) at bit position pos of a zeroed region, returns 1 if both
+// leave the same n and pos.
+int host_skip_plane_agrees(uint64_t x, unsigned n, unsigned pos, unsigned maxbits)
+{
+  uint32_t region[64];
+  memset(region, 0, sizeof region);
+  ArrayBits mem{region};
+  cswap::BlockEncoder<ArrayBits, false> a(mem, 0u, maxbits), b(mem, 0u, maxbits);
+  a.pos = b.pos = pos;
+  a.n = b.n = n;
+  uint64_t acc = n >= 64 ? ~0ull : (n ? ((~0ull) >> (64 - n)) : 0ull);  // any mask whose highest one-bit is n - 1 does
+  if (n) acc = 1ull << (n - 1);
+  a.plane(x);
+  b.skip_plane(x, acc);
+  return a.n == b.n && a.pos == b.pos;
+}
 }

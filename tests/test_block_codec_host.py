@@ -18,7 +18,7 @@ HDR = os.path.join(ROOT, "cswap_amd", "csrc", "zfp_block.h")
 @pytest.fixture(scope="module")
 def host():
     if (not os.path.exists(SO) or os.path.getmtime(SO) < max(os.path.getmtime(SRC), os.path.getmtime(HDR))):
-        subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-o", SO, SRC])
+        subprocess.check_call(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-pthread", "-o", SO, SRC])
     L = C.CDLL(SO)
     L.host_zfp_encode3.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
     L.host_zfp_decode3.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
@@ -254,3 +254,79 @@ def test_fenced_decoder_ignores_what_lies_behind_its_fence(host):
                 top = host.host_zfp_decode3_fenced(a.ctypes.data, nx, ny, nz, maxbits, o.ctypes.data, junk)
                 assert np.array_equal(o.view(np.uint32), plain.view(np.uint32)), (maxbits, scale, junk)
                 assert top < maxbits // 32 + 4, (maxbits, scale, top)
+
+
+# ---- the encoder's pair form: a block shared by two wavefronts (here: two host threads)
+def _pair(host):
+    host.host_zfp_encode3_pair.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
+    host.host_zfp_encode3_pair.restype = C.c_uint
+    host.host_skip_plane_agrees.argtypes = [C.c_uint64, C.c_uint, C.c_uint, C.c_uint]
+    host.host_skip_plane_agrees.restype = C.c_int
+    return host
+
+
+@pytest.mark.timeout(300)
+def test_skipping_a_plane_in_closed_form_leaves_the_coder_where_coding_it_does(host):
+    """BlockEncoder::skip_plane against BlockEncoder::plane (the coder of
+    encode.cuh:331-344) on single planes: every count of known coefficients, planes
+    that are empty, full, sparse, dense, that end in the last coefficient."""
+    L = _pair(host)
+    rng = np.random.default_rng(11)
+    planes = [0, 1, 2**63, 2**64 - 1, 2**63 | 1, 2**62, 0x5555555555555555, 0xAAAAAAAAAAAAAAAA, 2**32, 2**31]
+    for dens in (0.02, 0.1, 0.5, 0.9):
+        for _ in range(60):
+            bits = rng.random(64) < dens
+            planes.append(int(np.packbits(bits, bitorder="little").view(np.uint64)[0]))
+    for k in range(64):
+        planes += [1 << k, (1 << k) - 1 if k else 0, ((1 << 64) - 1) ^ ((1 << k) - 1)]
+    bad = []
+    for x in planes:
+        for n in list(range(0, 65, 3)) + [1, 2, 62, 63, 64]:
+            for pos in (9, 200, 511):
+                if not L.host_skip_plane_agrees(x, n, pos, 2048):
+                    bad.append((hex(x), n, pos))
+    assert not bad, bad[:10]
+
+
+@pytest.mark.timeout(600)
+def test_pair_form_of_the_encoder_matches_golden_vectors_and_the_block_encoder(host, golden):
+    """The pair form (two halves of a workgroup per block; here two threads with the
+    kernel's reuse of its shared words) gives the streams of the golden vectors and of
+    encode_block on random fields, at every whole-word rate incl. the ones that code the
+    low 16 planes, and stays within the slot's 128 bits of slack."""
+    L = _pair(host)
+    n = 0
+    for name, rate, maxbits, f, stream, dec in golden_cases(golden):
+        nz, ny, nx = f.shape
+        if nx % 4 or ny % 4 or nz % 4 or maxbits % 64:
+            continue
+        words = (nx // 4) * (ny // 4) * (nz // 4) * maxbits // 64
+        s = np.zeros(words, dtype=np.uint64)
+        top = L.host_zfp_encode3_pair(f.ctypes.data, nx, ny, nz, maxbits, s.ctypes.data)
+        assert top != 0xFFFFFFFF
+        assert np.array_equal(s.view(np.uint8), stream[:words * 8]), (name, rate)
+        assert top < maxbits // 32 + 4, (name, rate, "wrote past the 128 bits of slack")
+        n += 1
+    assert n >= 20, n
+    rng = np.random.default_rng(5)
+    kinds = {
+        "noise": lambda shape: rng.standard_normal(shape),
+        "smooth": lambda shape: np.cumsum(np.cumsum(rng.standard_normal(shape), axis=2), axis=1) * 1e-3,
+        "sparse": lambda shape: rng.standard_normal(shape) * (rng.random(shape) < 0.05),
+        "wide": lambda shape: rng.standard_normal(shape) * np.exp(8 * rng.standard_normal(shape)),
+        "const": lambda shape: np.full(shape, 1.5),
+        "zero": lambda shape: np.zeros(shape),
+        "tiny": lambda shape: rng.standard_normal(shape) * 1e-30,
+    }
+    for kind, make in kinds.items():
+        for shape in ((4, 4, 4), (8, 12, 16), (12, 8, 20)):
+            f = np.ascontiguousarray(make(shape), dtype=np.float32)
+            nz, ny, nx = shape
+            for maxbits in (64, 128, 256, 512, 1024, 2048, 4096):
+                words = (nx // 4) * (ny // 4) * (nz // 4) * maxbits // 64
+                want = np.zeros(words + 2, dtype=np.uint64)
+                host.host_zfp_encode3(f.ctypes.data, nx, ny, nz, maxbits, want.ctypes.data)
+                s = np.zeros(words, dtype=np.uint64)
+                top = L.host_zfp_encode3_pair(f.ctypes.data, nx, ny, nz, maxbits, s.ctypes.data)
+                assert np.array_equal(s, want[:words]), (kind, shape, maxbits)
+                assert top < maxbits // 32 + 4, (kind, shape, maxbits, top)

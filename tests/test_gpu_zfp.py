@@ -20,6 +20,29 @@ def torch_cuda():
     return torch
 
 
+SIZE_MAX = 2 ** 64 - 1
+FORMS = {"as shipped": None, "one lane per block": (0, 0), "pair form wherever the shape allows": (SIZE_MAX, SIZE_MAX)}
+
+
+@pytest.fixture(params=list(FORMS))
+def zfp_form(request):
+    """Which form of the 3-D fp32 kernels runs: the shipped size thresholds, the form with
+    one lane per block for every field, or the pair form (two wavefronts per 64 blocks)
+    for every field whose shape allows it."""
+    import ctypes as C
+
+    from cswap_amd._lib import lib
+
+    want = FORMS[request.param]
+    if want is None:
+        yield request.param
+        return
+    before = (C.c_size_t * 2)()
+    lib().cswap_zfp_set_pair_bytes(want[0], want[1], before)
+    yield request.param
+    lib().cswap_zfp_set_pair_bytes(before[0], before[1], None)
+
+
 def gpu_encode(torch, f, maxbits):
     from cswap_amd import api
 
@@ -29,7 +52,7 @@ def gpu_encode(torch, f, maxbits):
     return s
 
 
-def test_golden_vectors(torch_cuda, golden):
+def test_golden_vectors(torch_cuda, golden, zfp_form):
     torch = torch_cuda
     from cswap_amd import api
 
@@ -52,7 +75,7 @@ def test_golden_vectors(torch_cuda, golden):
 
 
 @pytest.mark.parametrize("rate", [4, 8, 16])
-def test_config1_bit_exact(torch_cuda, digests, rate):
+def test_config1_bit_exact(torch_cuda, digests, rate, zfp_form):
     torch = torch_cuda
     import oracle
     from cswap_amd import api
@@ -72,7 +95,7 @@ def test_config1_bit_exact(torch_cuda, digests, rate):
 
 
 @pytest.mark.parametrize("rate", [4, 8, 16])
-def test_config3_stack_vs_checker(torch_cuda, rate):
+def test_config3_stack_vs_checker(torch_cuda, rate, zfp_form):
     torch = torch_cuda
     import oracle
     from cswap_amd import api
@@ -138,7 +161,7 @@ def test_strided_field(torch_cuda):
 
 @pytest.mark.parametrize("case", ["padded_rows_and_planes", "one_block_per_slab", "slab_crossing", "planes_before_rows",
                                   "big_offsets"])
-def test_aligned_strided_fields(torch_cuda, case):
+def test_aligned_strided_fields(torch_cuda, case, zfp_form):
     """Fields embedded in larger allocations with 16-byte aligned rows: these take
     the 16-byte row path with a wave-uniform base and 32-bit lane offsets (a
     wavefront's 64 blocks may span many slabs of four planes), except when the
@@ -619,3 +642,58 @@ def test_mid_size_fields_equal_the_zfp_library(torch_cuda, kind, shape, rate):
                                                           o.data_ptr(), None), "decompress")
     torch.cuda.synchronize()
     assert np.array_equal(o.cpu().numpy().view(np.uint8), dec.view(np.uint8)), (kind, shape, maxbits)
+
+
+def test_pair_form_equals_the_form_with_one_lane_per_block(torch_cuda):
+    """The pair form of the kernels (two wavefronts share 64 blocks) against the form with one
+    lane per block, which the tests above pin to the golden vectors and the checker: the same
+    stream bytes and the same decoded bits, on fields whose last workgroup is not full, at every
+    rate the pair form takes (and two it must leave to the other form), on noise, smooth, sparse,
+    constant and all-zero data; and against the checker itself on one field per rate."""
+    torch = torch_cuda
+    import ctypes as C
+
+    import oracle
+    from cswap_amd import api
+    from cswap_amd._lib import lib
+
+    L = lib()
+    before = (C.c_size_t * 2)()
+    L.cswap_zfp_set_pair_bytes(0, 0, before)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(7)
+    try:
+        for shape in ((4, 4, 4), (4, 8, 12), (20, 36, 28), (3, 64, 32, 32), (1, 12, 260, 516), (9, 4, 512, 512)):
+            for kind in ("noise", "smooth", "sparse", "const", "zero"):
+                x = torch.randn(shape, generator=g, device="cuda")
+                if kind == "smooth":
+                    x = torch.cumsum(torch.cumsum(x, -1), -2) * 1e-3
+                elif kind == "sparse":
+                    x = x * (torch.rand(shape, generator=g, device="cuda") < 0.03)
+                elif kind == "const":
+                    x = torch.full(shape, 0.3, device="cuda")
+                elif kind == "zero":
+                    x = torch.zeros(shape, device="cuda")
+                for maxbits in (192, 256, 512, 520, 768, 1024, 2048, 4096):
+                    print("case", shape, kind, maxbits, flush=True)
+                    L.cswap_zfp_set_pair_bytes(0, 0, None)
+                    a = api.cuda_compress(x, maxbits)
+                    da = api.cuda_decompress(a, x.shape, maxbits)
+                    L.cswap_zfp_set_pair_bytes(SIZE_MAX, SIZE_MAX, None)
+                    b = api.cuda_compress(x, maxbits)
+                    db = api.cuda_decompress(a, x.shape, maxbits)
+                    torch.cuda.synchronize()
+                    assert torch.equal(a, b), (shape, kind, maxbits)
+                    assert torch.equal(da.view(torch.int32), db.view(torch.int32)), (shape, kind, maxbits)
+        L.cswap_zfp_set_pair_bytes(SIZE_MAX, SIZE_MAX, None)
+        f = np.random.default_rng(3).standard_normal((24, 20, 36)).astype(np.float32)
+        f[5:9] *= 1e-3
+        for maxbits in (256, 512, 1024, 2048):
+            s = gpu_encode(torch, f, maxbits)
+            want = oracle.zfp_encode3(f, maxbits)
+            assert np.array_equal(s.cpu().numpy().view(np.uint64), want), maxbits
+            d = api.cuda_decompress(s, f.shape, maxbits)
+            torch.cuda.synchronize()
+            assert np.array_equal(d.cpu().numpy().view(np.uint32), oracle.zfp_decode3(want, f.shape, maxbits).view(np.uint32))
+    finally:
+        L.cswap_zfp_set_pair_bytes(before[0], before[1], None)
