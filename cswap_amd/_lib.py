@@ -41,12 +41,17 @@ class Choice(C.Structure):
 
 class EngineConfig(C.Structure):
     _fields_ = [("pinned_pool_bytes", C.c_size_t), ("device_pool_bytes", C.c_size_t), ("process", C.c_int),
-                ("zfp_maxbits", C.c_uint), ("max_tickets", C.c_int), ("costs", Costs)]
+                ("zfp_maxbits", C.c_uint), ("max_tickets", C.c_int), ("costs", Costs), ("timing", C.c_int)]
 
 
 class TicketInfo(C.Structure):
     _fields_ = [("policy", C.c_int), ("n", C.c_size_t), ("nnz", C.c_size_t), ("bytes_in", C.c_size_t),
                 ("bytes_out", C.c_size_t), ("state", C.c_int)]
+
+
+class TicketTiming(C.Structure):
+    _fields_ = [("compress_us", C.c_double), ("copy_out_us", C.c_double), ("copy_in_us", C.c_double),
+                ("decompress_us", C.c_double)]
 
 
 class PlanSummary(C.Structure):
@@ -107,7 +112,8 @@ _SIGNATURES = {
     "cswap_zvc_workspace_bytes": (sz, [i32]),
     "cswap_zvc_compress_fused": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp]),
     "cswap_zvc_workspace_clear": (i32, [vp, i32, vp]),
-    "cswap_zvc_debug_set_lookback": (None, [u, u]),
+    "cswap_zvc_debug_set_lookback": (None, [u, u]),        # include/cswap_test_hooks.h
+    "cswap_test_zvc_stream_groups": (i32, [i32, i32]),      # include/cswap_test_hooks.h
     "cswap_zvc_compress_fused_static": (i32, [vp, i32, i32, vp, vp, vp, vp, vp]),
     "cswap_probe_nnz": (i32, [vp, sz, vp, vp]),
     "cswap_costs_default": (None, [C.POINTER(Costs)]),
@@ -123,6 +129,7 @@ _SIGNATURES = {
     "cswap_swap_prefetch": (i32, [vp, i32]),
     "cswap_swap_release": (i32, [vp, i32]),
     "cswap_swap_info": (i32, [vp, i32, C.POINTER(TicketInfo)]),
+    "cswap_swap_timing": (i32, [vp, i32, C.POINTER(TicketTiming)]),
     "cswap_engine_probe_count": (C.c_ulonglong, [vp]),
     "cswap_engine_calibrate": (i32, [vp, C.POINTER(Costs)]),
     "cswap_engine_copy_stream": (vp, [vp]),

@@ -116,7 +116,12 @@ struct Ticket {
   hipEvent_t ev_ready = nullptr;  // compute stream: compressed data / destination ready
   hipEvent_t ev_copy = nullptr;   // copy stream: transfer finished
   hipEvent_t ev_done = nullptr;   // compute stream: decompression finished
+  // engines with timing only: where each phase starts on its stream (its end is one of the three above)
+  hipEvent_t ev_start[4] = {nullptr, nullptr, nullptr, nullptr};  // compress, copy out, copy in, decompress
+  double us[4] = {-1, -1, -1, -1};  // the four phases, once known (see cswap_ticket_timing)
+  bool in_copied = false;           // the swap-in went over the link (else copy_in_us is 0)
 };
+enum { kPhaseCompress = 0, kPhaseCopyOut = 1, kPhaseCopyIn = 2, kPhaseDecompress = 3 };
 
 }  // namespace
 
@@ -139,7 +144,34 @@ struct cswap_engine {
   hipEvent_t ev_probe = nullptr;
   int device = 0;
   unsigned long long probes = 0;  // counting passes with a host round trip so far
+  bool timing = false;            // events carry timestamps and the phases of every ticket are bracketed
 };
+
+// microseconds between two events that have both fired, else -1
+static double elapsed_us(hipEvent_t a, hipEvent_t b)
+{
+  float ms = 0;
+  if (!a || !b || hipEventElapsedTime(&ms, a, b) != hipSuccess) {
+    (void)hipGetLastError();
+    return -1.0;
+  }
+  return (double)ms * 1e3;
+}
+
+// marks the start of a phase on the stream it is about to run on (engines with timing only)
+static hipError_t phase_start(const cswap_engine* e, Ticket& t, int phase, hipStream_t s)
+{
+  return e->timing ? hipEventRecord(t.ev_start[phase], s) : hipSuccess;
+}
+
+// The outbound side of t has finished: its two phase times are read now, before a swap-in
+// records the same events again.
+static void note_outbound_times(const cswap_engine* e, Ticket& t)
+{
+  if (!e->timing || t.us[kPhaseCopyOut] >= 0) return;
+  t.us[kPhaseCompress] = elapsed_us(t.ev_start[kPhaseCompress], t.ev_ready);
+  t.us[kPhaseCopyOut] = elapsed_us(t.ev_start[kPhaseCopyOut], t.ev_copy);
+}
 
 constexpr int kWsProcess = 65536;  // the engine's single-pass workspace serves chunk counts up to this
 
@@ -162,6 +194,7 @@ extern "C" void cswap_engine_config_default(cswap_engine_config* cfg)
   cfg->zfp_maxbits = 512;
   cfg->max_tickets = 256;
   cswap_costs_default(&cfg->costs);
+  cfg->timing = 0;
 }
 
 extern "C" void cswap_engine_destroy(cswap_engine* e)
@@ -173,6 +206,8 @@ extern "C" void cswap_engine_destroy(cswap_engine* e)
     if (t.ev_ready) (void)hipEventDestroy(t.ev_ready);
     if (t.ev_copy) (void)hipEventDestroy(t.ev_copy);
     if (t.ev_done) (void)hipEventDestroy(t.ev_done);
+    for (hipEvent_t ev : t.ev_start)
+      if (ev) (void)hipEventDestroy(ev);
   }
   if (e->ev_probe) (void)hipEventDestroy(e->ev_probe);
   if (e->h_nnz) (void)hipHostFree(e->h_nnz);
@@ -203,6 +238,8 @@ extern "C" int cswap_engine_create(cswap_engine** out, const cswap_engine_config
   e->costs = cfg.costs;
   e->process = cfg.process;
   e->maxbits = cfg.zfp_maxbits;
+  e->timing = cfg.timing != 0;
+  const unsigned ev_flags = e->timing ? hipEventDefault : hipEventDisableTiming;
   int rc = CSWAP_OK;
   auto fail = [&](hipError_t err) { rc = hip_fail(err); };
   hipError_t err;
@@ -223,9 +260,11 @@ extern "C" int cswap_engine_create(cswap_engine** out, const cswap_engine_config
     e->dpool.reset(cfg.device_pool_bytes);
     e->tickets.resize((size_t)cfg.max_tickets);
     for (auto& t : e->tickets) {
-      if ((err = hipEventCreateWithFlags(&t.ev_ready, hipEventDisableTiming)) != hipSuccess) break;
-      if ((err = hipEventCreateWithFlags(&t.ev_copy, hipEventDisableTiming)) != hipSuccess) break;
-      if ((err = hipEventCreateWithFlags(&t.ev_done, hipEventDisableTiming)) != hipSuccess) break;
+      if ((err = hipEventCreateWithFlags(&t.ev_ready, ev_flags)) != hipSuccess) break;
+      if ((err = hipEventCreateWithFlags(&t.ev_copy, ev_flags)) != hipSuccess) break;
+      if ((err = hipEventCreateWithFlags(&t.ev_done, ev_flags)) != hipSuccess) break;
+      for (int k = 0; k < 4 && e->timing && err == hipSuccess; k++) err = hipEventCreateWithFlags(&t.ev_start[k], ev_flags);
+      if (err != hipSuccess) break;
     }
     if (err != hipSuccess) { fail(err); break; }
   } while (0);
@@ -277,6 +316,7 @@ static bool event_done(hipEvent_t ev)
 static void land_outbound(cswap_engine* e, Ticket& t)
 {
   t.out_pending = false;
+  note_outbound_times(e, t);
   if (t.keep_staged && t.dev_held) {
     if (t.probe_held) {
       e->dpool.free(t.probe_off, t.probe_bytes);
@@ -303,13 +343,18 @@ static void free_ticket(cswap_engine* e, Ticket& t)
 static void reclaim_finished(cswap_engine* e)
 {
   for (auto& t : e->tickets) {
-    if (t.state != kOutInFlight && t.state != kReleasing && !(t.state == kInInFlight && t.out_pending)) continue;
-    if (t.out_pending && event_done(t.ev_copy)) t.out_pending = false;
+    if (t.state != kOutInFlight && t.state != kReleasing && t.state != kInInFlight) continue;
+    if (t.out_pending && event_done(t.ev_copy)) {
+      t.out_pending = false;
+      note_outbound_times(e, t);
+    }
     if (t.done_pending && event_done(t.ev_done)) t.done_pending = false;
     if (t.state == kOutInFlight && !t.out_pending) {
       land_outbound(e, t);
     } else if (t.state == kReleasing && !t.out_pending && !t.done_pending) {
       free_ticket(e, t);
+    } else if (t.state == kInInFlight && !t.out_pending && !t.done_pending) {
+      drop_device(e, t);  // swapped in and decompressed: nobody reads its staging block any more
     }
   }
 }
@@ -323,8 +368,15 @@ static bool reclaim_oldest(cswap_engine* e, bool released_only = false)
     if (((t.state == kOutInFlight && !released_only) || t.state == kReleasing) && (!oldest || t.seq < oldest->seq))
       oldest = &t;
   if (!oldest) return false;
-  if (oldest->out_pending) (void)hipEventSynchronize(oldest->ev_copy);
-  if (oldest->state == kReleasing && oldest->done_pending) (void)hipEventSynchronize(oldest->ev_done);
+  // an event that cannot be waited for (a device error) will not report done either: nothing
+  // comes back, and saying so ends the caller's loop instead of spinning on it
+  hipError_t err = hipSuccess;
+  if (oldest->out_pending) err = hipEventSynchronize(oldest->ev_copy);
+  if (err == hipSuccess && oldest->state == kReleasing && oldest->done_pending) err = hipEventSynchronize(oldest->ev_done);
+  if (err != hipSuccess) {
+    (void)hip_fail(err);
+    return false;
+  }
   reclaim_finished(e);
   return true;
 }
@@ -385,9 +437,12 @@ static int probe_tensor(cswap_engine* e, Ticket& t, const float* d_in, hipStream
 // workspace) or did not finish its job (the bounded wait inside the kernel ran out): the caller
 // then takes the probe path, with nothing held.  On success the ticket holds its staging block
 // and *src is the payload.
-static int single_pass_sparse(cswap_engine* e, Ticket& t, const float* d_in, hipStream_t compute, const void** src)
+static int single_pass_sparse(cswap_engine* e, Ticket& t, const float* d_in, hipStream_t compute, const void** src,
+                              bool small_form_only = false)
 {
-  if (t.process > kWsProcess || !cswap_zvc_takes_single_pass((int)t.n, t.process)) return 1;
+  if (t.process > kWsProcess) return 1;
+  const int form = cswap_zvc_takes_single_pass((int)t.n, t.process);
+  if (form == 0 || (small_form_only && form != 2)) return 1;
   const size_t hdr = zvc_header_bytes((int)t.n, t.process);
   const size_t worst = hdr + 4 * t.n;
   size_t off;
@@ -488,6 +543,7 @@ static int start_outbound_copy(cswap_engine* e, Ticket& t, const void* src, hipS
 {
   hipError_t err = hipEventRecord(t.ev_ready, compute);
   if (err == hipSuccess) err = hipStreamWaitEvent(e->copy, t.ev_ready, 0);
+  if (err == hipSuccess) err = phase_start(e, t, kPhaseCopyOut, e->copy);
   if (err == hipSuccess)
     err = hipMemcpyAsync(e->h_base + t.host_off, src, t.bytes_out, hipMemcpyDeviceToHost, e->copy);
   if (err == hipSuccess) err = hipEventRecord(t.ev_copy, e->copy);
@@ -499,8 +555,10 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
 {
   if (!e || !d_in || !ticket || !nx || !ny || !nz) return CSWAP_E_ARG;
   if (policy != CSWAP_POLICY_AUTO && policy != CSWAP_POLICY_NONE && policy != CSWAP_POLICY_SPARSE &&
-      policy != CSWAP_POLICY_ZFP)
+      policy != CSWAP_POLICY_ZFP && policy != CSWAP_POLICY_AUTO_SPARSE)
     return CSWAP_E_ARG;
+  const bool expect_sparse = policy == CSWAP_POLICY_AUTO_SPARSE;  // the selector, with the compaction as its probe
+  if (expect_sparse) policy = CSWAP_POLICY_AUTO;
   hipStream_t compute = (hipStream_t)compute_;
   std::lock_guard<std::mutex> lock(e->mu);
   const size_t n = nx * ny * nz;
@@ -525,8 +583,11 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   t.dev_held = false;
   t.probe_held = false;
   t.out_pending = t.done_pending = t.keep_staged = false;
+  t.in_copied = false;
+  for (double& u : t.us) u = -1.0;
   t.seq = e->next_seq++;
   t.process = zvc_ok ? process_for(e, n) : 0;
+  if (e->timing) CSWAP_HIP_TRY(hipEventRecord(t.ev_start[kPhaseCompress], compute));
   cswap_costs costs = e->costs;  // the selector prices the ZVC header with this tensor's chunk count
   if (t.process) costs.process = t.process;
 
@@ -543,10 +604,26 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
       want_probe = false;
     }
   }
-  if (policy == CSWAP_POLICY_SPARSE) {
+  // The compaction in its single-kernel form, which counts on the way: for an explicit ZVC
+  // request; for the selector when the caller expects a sparse tensor; and for the selector on
+  // any tensor small enough for the one-kernel form, which costs what the counting pass and the
+  // scan cost there.  The selector then decides with the count in hand and the payload made.
+  if (policy == CSWAP_POLICY_SPARSE || (want_probe && policy == CSWAP_POLICY_AUTO)) {
     const void* payload = nullptr;
-    rc = single_pass_sparse(e, t, d_in, compute, &payload);
+    rc = single_pass_sparse(e, t, d_in, compute, &payload, policy == CSWAP_POLICY_AUTO && !expect_sparse);
     if (rc < 0) return rc;
+    if (rc == 0 && policy == CSWAP_POLICY_AUTO) {
+      cswap_choice ch;
+      if ((rc = cswap_select_field(nx, ny, nz, t.nnz, e->maxbits, &costs, &ch))) { drop_device(e, t); return rc; }
+      t.policy = ch.policy;
+      want_probe = false;  // the count is known
+      if (ch.policy != CSWAP_POLICY_SPARSE) {
+        drop_device(e, t);  // the pass has finished (its count is on the host): the block can go back at once
+        rc = 1;             // on with the selector's choice below
+      } else {
+        rc = 0;
+      }
+    }
     if (rc == 0) {
       size_t hoff;
       if (!alloc_reclaiming(e, e->hpool, t.bytes_out, &hoff)) {
@@ -572,7 +649,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   if (want_probe && (rc = probe_tensor(e, t, d_in, compute, policy == CSWAP_POLICY_SPARSE))) return rc;
   if (t.policy == CSWAP_POLICY_AUTO) {
     cswap_choice ch;
-    if (!t.probe_held) costs.sparse_max_ratio = 0.0;  // not probed: ZVC is not an option
+    if (!t.probe_held) costs.sparse_max_ratio = 0.0;  // no chunk counts to compact with: ZVC is not an option
     if ((rc = cswap_select_field(nx, ny, nz, t.nnz, e->maxbits, &costs, &ch))) { drop_device(e, t); return rc; }
     t.policy = ch.policy;
   }
@@ -609,9 +686,12 @@ extern "C" int cswap_swap_wait(cswap_engine* e, int ticket)
   if (!t) return CSWAP_E_ARG;
   if (t->state == kOnHost) return CSWAP_OK;
   if (t->state == kPrefetched && t->dev_held) return CSWAP_OK;  // landed while a prefetch held its payload
-  if (t->state == kInInFlight && t->out_pending) {  // swapped back in from its staging block before the copy had finished
-    CSWAP_HIP_TRY(hipEventSynchronize(t->ev_copy));
-    t->out_pending = false;
+  if (t->state == kInInFlight) {  // swapped back in already, perhaps from its staging block before the copy had finished
+    if (t->out_pending) {
+      CSWAP_HIP_TRY(hipEventSynchronize(t->ev_copy));
+      t->out_pending = false;
+      note_outbound_times(e, *t);
+    }
     return CSWAP_OK;
   }
   if (t->state != kOutInFlight) return CSWAP_E_STATE;
@@ -659,13 +739,16 @@ extern "C" int cswap_swap_prefetch(cswap_engine* e, int ticket)
   t->dev_off = off; t->dev_bytes = t->bytes_out; t->dev_held = true;
   // the staging region was released only after the events of its last user were seen to have
   // fired, so the copy stream has nothing to order against
-  hipError_t err = hipMemcpyAsync(e->d_base + off, e->h_base + t->host_off, t->bytes_out, hipMemcpyHostToDevice, e->copy_in);
+  hipError_t err = phase_start(e, *t, kPhaseCopyIn, e->copy_in);
+  if (err == hipSuccess)
+    err = hipMemcpyAsync(e->d_base + off, e->h_base + t->host_off, t->bytes_out, hipMemcpyHostToDevice, e->copy_in);
   if (err == hipSuccess) err = hipEventRecord(t->ev_copy, e->copy_in);
   if (err != hipSuccess) {
     (void)hipStreamSynchronize(e->copy_in);
     drop_device(e, *t);
     return hip_fail(err);
   }
+  t->in_copied = true;
   t->state = kPrefetched;
   return CSWAP_OK;
 }
@@ -706,10 +789,13 @@ extern "C" int cswap_swap_in(cswap_engine* e, int ticket, float* d_out, cswap_st
     // the copy may not overtake earlier work of the compute stream on d_out
     err = hipEventRecord(t->ev_ready, compute);
     if (err == hipSuccess) err = hipStreamWaitEvent(e->copy_in, t->ev_ready, 0);
+    if (err == hipSuccess) err = phase_start(e, *t, kPhaseCopyIn, e->copy_in);
     if (err == hipSuccess) err = hipMemcpyAsync(src, e->h_base + t->host_off, t->bytes_out, hipMemcpyHostToDevice, e->copy_in);
     if (err == hipSuccess) err = hipEventRecord(t->ev_copy, e->copy_in);
     if (err == hipSuccess) err = hipStreamWaitEvent(compute, t->ev_copy, 0);
+    t->in_copied = true;
   }
+  if (err == hipSuccess) err = phase_start(e, *t, kPhaseDecompress, compute);
   if (err != hipSuccess) {
     (void)hipStreamSynchronize(e->copy_in);
     (void)hipStreamSynchronize(compute);
@@ -764,6 +850,26 @@ extern "C" int cswap_swap_info(cswap_engine* e, int ticket, cswap_ticket_info* i
   info->bytes_out = t->bytes_out;
   // to the caller a released ticket is free, and a payload that a prefetch found still staged is prefetched
   info->state = t->state == kReleasing ? (int)kFree : (t->state == kOutInFlight && t->keep_staged ? (int)kPrefetched : t->state);
+  return CSWAP_OK;
+}
+
+extern "C" int cswap_swap_timing(cswap_engine* e, int ticket, cswap_ticket_timing* out)
+{
+  if (!e || !out) return CSWAP_E_ARG;
+  std::lock_guard<std::mutex> lock(e->mu);
+  Ticket* t = get_ticket(e, ticket);
+  if (!t || t->state == kFree || t->state == kReleasing) return CSWAP_E_ARG;
+  if (!e->timing) return CSWAP_E_UNSUPPORTED;
+  reclaim_finished(e);  // notes the outbound times of a copy that has finished since anybody last looked
+  if (!t->out_pending) note_outbound_times(e, *t);
+  if (t->state == kInInFlight && t->us[kPhaseDecompress] < 0 && event_done(t->ev_done)) {
+    t->us[kPhaseCopyIn] = t->in_copied ? elapsed_us(t->ev_start[kPhaseCopyIn], t->ev_copy) : 0.0;
+    t->us[kPhaseDecompress] = elapsed_us(t->ev_start[kPhaseDecompress], t->ev_done);
+  }
+  out->compress_us = t->us[kPhaseCompress];
+  out->copy_out_us = t->us[kPhaseCopyOut];
+  out->copy_in_us = t->us[kPhaseCopyIn];
+  out->decompress_us = t->us[kPhaseDecompress];
   return CSWAP_OK;
 }
 

@@ -13,10 +13,12 @@
 // format carries anyway (`begin`) is the device-wide scan; no finer scan is
 // needed.
 #include <hip/hip_runtime.h>
+#include <atomic>
 
 #include <mutex>
 
 #include "../../include/cswap_hip.h"
+#include "../../include/cswap_test_hooks.h"
 #include "common.h"
 
 namespace cswap {
@@ -165,7 +167,7 @@ constexpr int kHalf = 256;  // floats per half of a wave's ring
 #ifndef CSWAP_STAGED_COMPACT_BYTES
 #define CSWAP_STAGED_COMPACT_BYTES (192ull << 20)
 #endif
-static unsigned long long g_staged_compact_bytes = CSWAP_STAGED_COMPACT_BYTES;  // cswap_zvc_set_staged_compact_bytes
+static std::atomic<unsigned long long> g_staged_compact_bytes{CSWAP_STAGED_COMPACT_BYTES};  // cswap_zvc_set_staged_compact_bytes
 
 __device__ __forceinline__ void lds_order()
 {
@@ -541,9 +543,16 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void zvc_expand4_staged_kernel
 // The single-pass kernel below exchanges counts between workgroups through status words
 // in global memory, read and written with relaxed atomics of agent scope (they travel past
 // the per-XCD L2 caches, which are not coherent with each other).
-constexpr unsigned kSpinLimit = 1u << 20;
+// How often a wavefront may ask again for status words it is waiting for, summed over the whole
+// kernel (not per word: once the budget is spent every later wait of that wavefront returns at
+// once, and a wavefront that sees the failure flag up stops waiting as well, so a run that cannot
+// finish -- the grid's workgroups are not all resident at the same time, say -- ends after one
+// budget, not after one per tile).  A turn is a sleep and a trip to memory, 1-2 us: the default
+// is some tens of milliseconds, two orders of magnitude above what the kernel takes for 1 GiB.
+constexpr unsigned kSpinLimit = 1u << 15;
+constexpr unsigned kFlagEvery = 32;  // a waiting wavefront looks at the failure flag every so many turns
 // cswap_zvc_debug_set_lookback: the bound of the waits, and whether tile 0 is never published
-static unsigned g_spin_limit = kSpinLimit, g_skip_first = 0;
+static std::atomic<unsigned> g_spin_limit{kSpinLimit}, g_skip_first{0};
 
 // Head of a workspace.  ws[0]: kWsMagic once cswap_zvc_workspace_clear has prepared it;
 // ws[1]: not 0 after a run whose bounded waits ran out (stays until the next clear, and
@@ -646,13 +655,14 @@ __device__ void zvc_stream_scanner(uint32_t* ws, int tiles, int step, int* nnz, 
   const bool refused = magic != kWsMagic || flag0 != 0u;
   if (refused && lane == 0) *nnz = -1;
   unsigned carry = 0;
+  unsigned spins = 0;    // turns of waiting so far, over all steps
+  bool flagged = false;  // the failure flag is up: no more waiting, the offsets from here on are garbage below n
   // `step` tiles at a time (at most 256): the tiles that the data workgroups count in the same
   // stage, so that a step never waits for a count that is published a stage later than the rest
   for (int t0 = 0; t0 < tiles; t0 += step) {
     // lane l owns tiles t0 + 4l .. t0 + 4l + 3
     const int stop = t0 + step < tiles ? t0 + step : tiles;
     uint32_t v[4] = {kTileReady, kTileReady, kTileReady, kTileReady};
-    unsigned spins = 0;
     while (!refused) {
       bool missing = false;
 #pragma unroll
@@ -661,9 +671,14 @@ __device__ void zvc_stream_scanner(uint32_t* ws, int tiles, int step, int* nnz, 
         v[r] = t < stop ? ld_status(&status[t]) : kTileReady;
         missing |= (v[r] & kTileReady) == 0u;
       }
-      if (__ballot(missing) == 0ull) break;
+      if (__ballot(missing) == 0ull || flagged) break;
       if (++spins > spin_limit) {  // give up: flag it; the offsets that follow are garbage below n
         if (lane == 0) atomicOr(&ws[kWsFlag], 1u);
+        flagged = true;
+        break;
+      }
+      if (spins % kFlagEvery == 0 && ld_status(&ws[kWsFlag]) != 0u) {  // a data workgroup gave up
+        flagged = true;
         break;
       }
       __builtin_amdgcn_s_sleep(4);
@@ -765,14 +780,16 @@ __global__ __launch_bounds__(64 * kSWaves) void zvc_stream_kernel(
   // waits (bounded) until the scanner has published the offset of tile t
   bool gave_up = false;
   uint32_t runs0 = 0;  // ws[kWsRuns] when this wavefront gave up
+  unsigned spins = 0;   // turns of waiting so far, over all tiles
   auto await_offset = [&](int t) {
-    unsigned spins = 0;
-    while ((ov & kTileReady) == 0u) {
-      if (++spins > spin_limit) {
-        // give up: flag it and go on with what is there, so that every workgroup
-        // still reaches its end (offsets are kept inside the tensor, the output is garbage)
-        if (lane == 0) atomicOr(&ws[kWsFlag], 1u);
-        if (!gave_up) runs0 = ld_status(&ws[kWsRuns]);  // the scanner has not finished: it still owes this offset
+    while ((ov & kTileReady) == 0u && !gave_up) {
+      const bool spent = ++spins > spin_limit;
+      if (spent || (spins % kFlagEvery == 0 && ld_status(&ws[kWsFlag]) != 0u)) {
+        // give up (my budget is spent, or somebody else's was): flag it and go on with what is
+        // there, so that every workgroup still reaches its end (offsets are kept inside the
+        // tensor, the output is garbage); no later tile waits again
+        if (spent && lane == 0) atomicOr(&ws[kWsFlag], 1u);
+        runs0 = ld_status(&ws[kWsRuns]);  // the scanner has not finished: it still owes this offset
         gave_up = true;
         break;
       }
@@ -1188,9 +1205,7 @@ extern "C" int cswap_zvc_scan(int* d_count, int k, int* d_nnz, cswap_stream_t st
 
 extern "C" size_t cswap_zvc_set_staged_compact_bytes(size_t bytes)
 {
-  const size_t before = (size_t)g_staged_compact_bytes;
-  g_staged_compact_bytes = bytes;
-  return before;
+  return (size_t)g_staged_compact_bytes.exchange(bytes);
 }
 
 extern "C" int cswap_zvc_compact(const float* d_in, int n, int process, const int* d_begin, float* d_values,
@@ -1270,8 +1285,8 @@ extern "C" size_t cswap_zvc_workspace_bytes(int process)
 
 extern "C" void cswap_zvc_debug_set_lookback(unsigned spin_limit, unsigned skip_first)
 {
-  g_spin_limit = spin_limit ? spin_limit : kSpinLimit;
-  g_skip_first = skip_first;
+  g_spin_limit.store(spin_limit ? spin_limit : kSpinLimit);
+  g_skip_first.store(skip_first);
 }
 
 // compute units of the current device (0 if the query fails), looked up once per device
@@ -1291,14 +1306,25 @@ static int device_compute_units()
 static int status_words(int process);
 // Tensors of at least this many bytes take the single pass in cswap_zvc_compress_fused; smaller ones
 // finish sooner with the three kernels (a few rounds of the grid do not fill the pipeline).
-static unsigned long long g_single_pass_bytes = 64ull << 20;  // cswap_zvc_set_single_pass_bytes
+static std::atomic<unsigned long long> g_single_pass_bytes{64ull << 20};  // cswap_zvc_set_single_pass_bytes
 
 extern "C" size_t cswap_zvc_set_single_pass_bytes(size_t bytes)
 {
-  const size_t before = (size_t)g_single_pass_bytes;
-  g_single_pass_bytes = bytes;
-  return before;
+  return (size_t)g_single_pass_bytes.exchange(bytes);
 }
+
+// Data workgroups of the pipeline kernel: one per compute unit but one (the scanner's), no more
+// than there are tiles, and no more than the 256 tiles whose counts the scanner's one wavefront
+// turns into offsets per step (four per lane) -- on a part with more compute units than that the
+// tiles past the 256th of every step would never get an offset.
+static int stream_data_groups(int tiles, int compute_units)
+{
+  int g = compute_units - 1;
+  if (g > tiles) g = tiles;
+  if (g > 4 * 64) g = 4 * 64;
+  return g < 0 ? 0 : g;
+}
+extern "C" int cswap_test_zvc_stream_groups(int tiles, int compute_units) { return stream_data_groups(tiles, compute_units); }
 
 // whether the single pass takes a tensor of this shape; fills its geometry
 static bool single_pass_shape(const Geometry& g, int n, int process, StreamGeometry& sg)
@@ -1326,7 +1352,8 @@ static bool small_pass_shape(const Geometry& g, int n, int process, StreamGeomet
   sg.tiles = 0;
   const int cus = device_compute_units();
   const int G = cus < kQGroupsMax ? cus : kQGroupsMax;
-  if (G < 1 || g.E % 32 != 0 || g_single_pass_bytes == ~0ull || 4ull * (unsigned long long)n >= g_single_pass_bytes) return false;
+  const unsigned long long single_from = g_single_pass_bytes.load();
+  if (G < 1 || g.E % 32 != 0 || single_from == ~0ull || 4ull * (unsigned long long)n >= single_from) return false;
   // every row of the mask layout has an owner, also the rows of chunks that hold no data (their words are zero)
   int R = 8;  // 8, 16 or 32 rows per wavefront (64 would need more registers than a wavefront of sixteen has)
   while (R <= 32 && (long long)G * kQWaves * R < (long long)sg.rows) R *= 2;
@@ -1363,7 +1390,7 @@ extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, v
     uint32_t* counts = ws + 16 + status_words(process) - kSmallWords;
 #define CSWAP_SMALL(R)                                                                                              \
   hipLaunchKernelGGL(zvc_small_kernel<R>, dim3(groups), dim3(64 * kQWaves), 0, (hipStream_t)stream, d_in, sg, ws, \
-                     counts, d_begin, d_nnz, d_values, d_mask, g_spin_limit, g_skip_first)
+                     counts, d_begin, d_nnz, d_values, d_mask, g_spin_limit.load(), g_skip_first.load())
     if (rows == 8) CSWAP_SMALL(8);
     else if (rows == 16) CSWAP_SMALL(16);
     else CSWAP_SMALL(32);
@@ -1372,13 +1399,13 @@ extern "C" int cswap_zvc_compress_fused(const float* d_in, int n, int process, v
   }
   if (!single_pass) return cswap_zvc_compress(d_in, n, process, d_begin, d_nnz, d_values, d_mask, stream);
   // one workgroup per compute unit, the last of them the scanner
-  const int data_groups = sg.tiles < cus - 1 ? sg.tiles : cus - 1;
+  const int data_groups = stream_data_groups(sg.tiles, cus);
   if (4ull * (unsigned long long)n >= g_staged_compact_bytes)
     hipLaunchKernelGGL(zvc_stream_kernel<true>, dim3(data_groups + 1), dim3(64 * kSWaves), 0, (hipStream_t)stream,
-                       d_in, sg, ws, d_begin, d_nnz, d_values, d_mask, g_spin_limit, g_skip_first);
+                       d_in, sg, ws, d_begin, d_nnz, d_values, d_mask, g_spin_limit.load(), g_skip_first.load());
   else
     hipLaunchKernelGGL(zvc_stream_kernel<false>, dim3(data_groups + 1), dim3(64 * kSWaves), 0, (hipStream_t)stream,
-                       d_in, sg, ws, d_begin, d_nnz, d_values, d_mask, g_spin_limit, g_skip_first);
+                       d_in, sg, ws, d_begin, d_nnz, d_values, d_mask, g_spin_limit.load(), g_skip_first.load());
   return check_launch();
 }
 

@@ -90,6 +90,8 @@ class Execution:
                     self.memo_hits += 1
                 else:
                     remember = True
+                    if m and m[0] == t.numel() and m[1] == swap.SPARSE:
+                        act = swap.AUTO_SPARSE   # the selector, with the compaction itself as its probe
             ticket = self.engine.pre(t, act)
             if remember:
                 self._memo[tid] = [t.numel(), self.engine.info(ticket).policy, 0]

@@ -139,6 +139,11 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
                 policy = known[0]
                 self.memo[slot] = (known[0], known[1] + 1)
                 self.stats["memo_hits"] = self.stats.get("memo_hits", 0) + 1
+            elif known is not None and known[0] == swap.SPARSE:
+                # still the selector's call, but with the compaction itself as its probe: the payload
+                # is made by the time the count is known, and the count confirms the choice every time
+                policy = swap.AUTO_SPARSE
+                self.stats["memo_sparse"] = self.stats.get("memo_sparse", 0) + 1
         try:
             try:
                 ticket = self.engine.pre(t.detach(), policy)
@@ -153,7 +158,7 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
             self.stats["kept_no_room"] = self.stats.get("kept_no_room", 0) + 1
             return t                     # pinned pool, staging pool or tickets exhausted: the tensor stays on the device
         info = self.engine.info(ticket)
-        if self.memo is not None and policy == swap.AUTO:
+        if self.memo is not None and policy in (swap.AUTO, swap.AUTO_SPARSE):
             self.memo[slot] = (info.policy, 0)
         self.stats["swapped"] += 1
         self.stats["bytes_in"] += info.bytes_in

@@ -13,10 +13,11 @@ import time
 
 import torch
 
-from ._lib import Choice, Costs, EngineConfig, TicketInfo, check, lib
+from ._lib import Choice, Costs, EngineConfig, TicketInfo, TicketTiming, check, lib
 from .workloads import field_dims
 
 AUTO, NONE, SPARSE, ZFP = -1, 2, 3, 6
+AUTO_SPARSE = -3   # the selector for a tensor expected to be sparse: the compaction itself is its probe
 POLICY_NAME = {NONE: "none", SPARSE: "sparse", ZFP: "zfp"}
 
 
@@ -42,7 +43,7 @@ def select_field(nx: int, ny: int, nz: int, nnz: int, maxbits: int = 512, costs:
 
 class SwapEngine:
     def __init__(self, pinned_bytes: int = 1 << 30, device_bytes: int = 1 << 30, maxbits: int = 512,
-                 process: int = 0, max_tickets: int = 256, costs: Costs | None = None):
+                 process: int = 0, max_tickets: int = 256, costs: Costs | None = None, timing: bool = False):
         cfg = EngineConfig()
         lib().cswap_engine_config_default(C.byref(cfg))
         cfg.pinned_pool_bytes = pinned_bytes
@@ -52,6 +53,7 @@ class SwapEngine:
         cfg.max_tickets = max_tickets
         if costs is not None:
             cfg.costs = costs
+        cfg.timing = 1 if timing else 0
         self._h = C.c_void_p()
         check(lib().cswap_engine_create(C.byref(self._h), C.byref(cfg)), "cswap_engine_create")
 
@@ -110,6 +112,13 @@ class SwapEngine:
 
     def release(self, ticket: int) -> None:
         check(lib().cswap_swap_release(self._h, ticket), "cswap_swap_release")
+
+    def timing(self, ticket: int) -> TicketTiming:
+        """Phase times of the ticket in microseconds, from the engine's own events
+        (engines created with ``timing=True``); -1 = not finished yet."""
+        t = TicketTiming()
+        check(lib().cswap_swap_timing(self._h, ticket, C.byref(t)), "cswap_swap_timing")
+        return t
 
     def info(self, ticket: int) -> TicketInfo:
         i = TicketInfo()

@@ -100,6 +100,11 @@ class Execution {
           memo->uses++;
           memo_hits++;
           memo = nullptr;
+        } else if (memo->n == n && memo->policy == CSWAP_POLICY_SPARSE) {
+          // remembered as sparse: still the selector's call, with the compaction itself as its
+          // probe (the payload is made by the time the count is known; the count confirms or
+          // overturns the choice every time, so this memory never goes stale)
+          act = CSWAP_POLICY_AUTO_SPARSE;
         }
       }
       int ticket = -1;

@@ -214,12 +214,6 @@ int cswap_zvc_takes_single_pass(int n, int process);
  * the three kernels for every tensor).
  * Returns the previous value.  Process-wide. */
 size_t cswap_zvc_set_single_pass_bytes(size_t bytes);
-/* For tests of that failure path only.  spin_limit: how many times a wavefront
- * asks again for a status word it waits for before it gives up (0 = the default,
- * about a million); skip_first: if not 0 the count of the first tile is never
- * published, so that everything after it waits in vain.  Process-wide; (0, 0)
- * restores normal operation. */
-void cswap_zvc_debug_set_lookback(unsigned spin_limit, unsigned skip_first);
 /* No counterpart in the reference.  cswap_zvc_compress_fused for callers that
  * cannot allocate a workspace (code under HIP graph capture, serving loops and
  * harnesses that forbid hipMalloc): the status words live in a static device
@@ -256,7 +250,16 @@ int cswap_probe_nnz(const float* d_in, size_t n, unsigned long long* d_nnz, cswa
  * 393-397).
  */
 typedef enum { CSWAP_POLICY_AUTO = -1, CSWAP_POLICY_NONE = 2, CSWAP_POLICY_SPARSE = 3,
-               CSWAP_POLICY_ZFP = 6 } cswap_policy; /* codes as in Execution.h:70,86,107 */
+               CSWAP_POLICY_ZFP = 6, /* codes as in Execution.h:70,86,107 */
+               /* The selector again, for a tensor that is expected to be sparse (the caller
+                * remembers that the selector chose ZVC for it the last time): the engine runs the
+                * ZVC compaction right away, in its single-kernel form, which produces the count on
+                * the way -- the reference's one probe is likewise the count pass of its compactor
+                * (Execution.h:89-95) -- and asks the selector with that count.  If the answer is
+                * still ZVC the payload is there already; if not, the selector's choice runs as
+                * it would have after a probe.  Never a wrong result, one wasted pass when the
+                * expectation was wrong. */
+               CSWAP_POLICY_AUTO_SPARSE = -3 } cswap_policy;
 
 typedef struct {
   double bw_d2h_gbs, bw_h2d_gbs;         /* pinned host link, GB/s */
@@ -322,6 +325,9 @@ typedef struct {
   unsigned zfp_maxbits;       /* bits per 4x4x4 block for policy ZFP; 0 = 512 (8 bits/value) */
   int    max_tickets;         /* tensors that may be swapped out at once; 0 = 256 */
   cswap_costs costs;          /* used by CSWAP_POLICY_AUTO; zero bw fields = defaults */
+  int    timing;              /* not 0: every phase of a ticket is bracketed by timing events on the stream it
+                                 runs on and cswap_swap_timing reports them (the reference's profiler slots,
+                                 Execution.h:109-126,285-295).  0 (default): events carry no timestamps. */
 } cswap_engine_config;
 
 typedef struct {
@@ -331,6 +337,23 @@ typedef struct {
   int    state;               /* 0 free, 1 out in flight, 2 resident on host, 3 in in flight, 4 prefetched */
 } cswap_ticket_info;
 
+/* What a ticket's phases took on the GPU, in microseconds, from events recorded on the stream
+ * each phase runs on (engines created with config.timing only).  -1: that phase has not
+ * finished yet (or never started); 0: it did not take place (a raw swap has no kernels; a
+ * tensor that came back from its staging block crossed the link only once).
+ *   compress_us    from the call of cswap_swap_out on the compute stream to the end of the
+ *                  compression kernel: probe or single-pass count, the host round trip for
+ *                  the count, the selector, the compression (the reference's slot 2,
+ *                  Execution.h:109-116, which also starts before `compress` and ends after it)
+ *   copy_out_us    the device-to-host copy on the copy stream (what the reference splits into
+ *                  the part under the consumer's kernel, slot 0, and the wait after it,
+ *                  slot 1: Execution.h:285-295)
+ *   copy_in_us     the host-to-device copy on the inbound copy stream
+ *   decompress_us  the decompression kernel on the compute stream */
+typedef struct {
+  double compress_us, copy_out_us, copy_in_us, decompress_us;
+} cswap_ticket_timing;
+
 void cswap_engine_config_default(cswap_engine_config* cfg);
 int  cswap_engine_create(cswap_engine** out, const cswap_engine_config* cfg);
 void cswap_engine_destroy(cswap_engine* e);
@@ -338,7 +361,14 @@ void cswap_engine_destroy(cswap_engine* e);
 /* Execution::pre: compress d_in on `compute` (policy AUTO probes and selects
  * first, which costs one small host round trip like Execution.h:92) and start
  * the device-to-host copy on the engine's copy stream, ordered after the
- * compression by an event.  The tensor is the field a[nz][ny][nx]. */
+ * compression by an event.  The tensor is the field a[nz][ny][nx].
+ * The probe of an AUTO request is the counting pass of the compactor, whose per-chunk
+ * counts the compaction then reuses (Execution.h:89-95); for tensors small enough for the
+ * one-kernel form of the compactor (cswap_zvc_takes_single_pass == 2, up to 32 MiB) it is
+ * that kernel itself, into a staging block of the worst-case size when the pool has one
+ * to spare: a tensor that turns out sparse is compacted by the time its count is known.
+ * Calls that probe hold the engine's lock over the host round trip (about 20 us): two
+ * threads' swap-outs through one engine take turns. */
 int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, size_t ny, size_t nz, int policy,
                    cswap_stream_t compute, int* ticket);
 /* Execution::post: block the host until the copy of `ticket` has finished;
@@ -370,6 +400,9 @@ int cswap_swap_prefetch(cswap_engine* e, int ticket);
  * and the ticket number is not handed out again before that. */
 int cswap_swap_release(cswap_engine* e, int ticket);
 int cswap_swap_info(cswap_engine* e, int ticket, cswap_ticket_info* info);
+/* Phase times of a ticket so far (see cswap_ticket_timing); does not wait for anything.
+ * CSWAP_E_UNSUPPORTED on an engine created without config.timing. */
+int cswap_swap_timing(cswap_engine* e, int ticket, cswap_ticket_timing* out);
 /* Number of probes so far: counting passes followed by the host round trip for
  * the non-zero count (the one at Execution.h:92), which a selector-driven or ZVC
  * swap-out pays and an explicit raw or ZFP request does not. */

@@ -60,3 +60,20 @@ def test_argument_errors_do_not_launch():
     assert L.cswap_zfp_decompress_f32(None, 4, 4, 4, 0, 0, 0, 512, None, None) == -1
     assert L.cswap_zvc_count(None, 10, 16384, None, None) == -1
     assert L.cswap_probe_nnz(None, 0, None, None) == -1
+
+
+def test_pipeline_kernel_grid_fits_its_scanner_on_any_part():
+    """The ZVC pipeline kernel runs one data workgroup per compute unit but one, never more than
+    there are tiles, and never more than the 256 tiles its one scanner wavefront serves per step:
+    on a part with more compute units than that, the tiles beyond would wait for an offset that
+    never comes.  The grid is computed on the host, so parts this build never runs on can be
+    asked about."""
+    from cswap_amd import _lib
+
+    f = _lib.lib().cswap_test_zvc_stream_groups
+    assert f(10000, 256) == 255          # MI355X
+    assert f(10000, 304) == 256          # more compute units than the scanner serves per step
+    assert f(10000, 1024) == 256
+    assert f(100, 256) == 100            # fewer tiles than compute units
+    assert f(5, 304) == 5
+    assert f(10000, 2) == 1 and f(10000, 1) == 0

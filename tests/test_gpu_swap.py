@@ -791,3 +791,166 @@ def test_a_full_staging_pool_makes_requests_wait_not_fail(torch_cuda):
             eng.release(tk)
     finally:
         eng.close()
+
+
+def test_selector_with_the_compaction_as_its_probe(torch_cuda):
+    """CSWAP_POLICY_AUTO_SPARSE: the selector for a tensor its caller expects to be sparse.  The
+    single-kernel compaction runs first and yields the count; a sparse tensor ends up as ZVC with
+    one host round trip and the payload the three kernels make; a dense one is handed on to the
+    selector's choice (ZFP here) and still comes back as that codec would give it; plain AUTO on a
+    tensor small enough for the one-kernel form takes the same route.  Sizes on both sides of the
+    pipeline kernel's threshold."""
+    torch = torch_cuda
+    import oracle
+    from cswap_amd import swap
+    from cswap_amd._lib import lib
+
+    eng = swap.SwapEngine(pinned_bytes=384 << 20, device_bytes=640 << 20)
+    try:
+        for shape, zeros in (((32, 64, 32, 32), 0.7), ((64, 64, 64, 64), 0.6), ((128, 64, 64, 64), 0.5)):
+            x = relu_tensor(torch, shape, zeros, 31)
+            n = x.numel()
+            nnz = int((x != 0).sum().item())
+            form = lib().cswap_zvc_takes_single_pass(n, eng.process_for(n))
+            assert form in (1, 2)
+            for pol in (swap.AUTO_SPARSE, swap.AUTO, swap.SPARSE):
+                print("sparse", shape, pol, "form", form, flush=True)
+                before = eng.probe_count()
+                tk = eng.pre(x, pol)
+                assert eng.probe_count() == before + 1          # one host round trip, whichever way
+                info = eng.info(tk)
+                assert info.policy == swap.SPARSE and info.nnz == nnz
+                assert info.bytes_out == 4 * nnz + n // 8 + 4 * eng.process_for(n)
+                out = torch.full_like(x, -1.0)
+                eng.swap_in(tk, out)
+                torch.cuda.synchronize()
+                eng.release(tk)
+                assert torch.equal(out, x)
+        g = torch.Generator(device="cuda"); g.manual_seed(5)
+        for shape in ((32, 64, 32, 32), (128, 64, 64, 64)):
+            x = torch.randn(shape, generator=g, device="cuda")
+            for pol in (swap.AUTO_SPARSE, swap.AUTO):
+                print("dense", shape, pol, flush=True)
+                tk = eng.pre(x, pol)
+                info = eng.info(tk)
+                assert info.policy == swap.ZFP and info.nnz == int((x != 0).sum().item())
+                out = torch.full_like(x, -1.0)
+                eng.swap_in(tk, out)
+                torch.cuda.synchronize()
+                eng.release(tk)
+                f = x.cpu().numpy().reshape(-1, shape[-2], shape[-1])
+                want = oracle.zfp_decode3(oracle.zfp_encode3(f, 512, omp=True), f.shape, 512, omp=True)
+                assert np.array_equal(out.cpu().numpy().reshape(f.shape).view(np.uint32), want.view(np.uint32))
+    finally:
+        eng.close()
+
+
+@pytest.mark.parametrize("policy_name", ["none", "sparse", "zfp", "auto"])
+def test_phase_times_of_a_ticket_come_from_the_engine(torch_cuda, policy_name):
+    """An engine created with timing brackets every phase of a ticket with events on the stream
+    it runs on (the reference's profiler slots, Execution.h:109-126,285-295): after a swap-out,
+    a wait, a swap-in and a synchronize the four figures are there, the copies take the time
+    the link needs for the payload, and together they fit inside the wall clock around the
+    calls.  Before a phase has finished its figure is -1; an engine without timing refuses."""
+    torch = torch_cuda
+    import time
+
+    from cswap_amd import swap
+    from cswap_amd._lib import CswapError
+
+    pol = {"none": swap.NONE, "sparse": swap.SPARSE, "zfp": swap.ZFP, "auto": swap.AUTO}[policy_name]
+    x = relu_tensor(torch, (64, 64, 64, 64), 0.6, 9)          # 64 MiB
+    out = torch.empty_like(x)
+    eng = swap.SwapEngine(pinned_bytes=256 << 20, device_bytes=256 << 20, timing=True)
+    try:
+        for rep in range(3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            tk = eng.pre(x, pol)
+            first = eng.timing(tk)
+            eng.post(tk)
+            mid = eng.timing(tk)
+            eng.swap_in(tk, out)
+            torch.cuda.synchronize()
+            wall_us = (time.perf_counter() - t0) * 1e6
+            t = eng.timing(tk)
+            info = eng.info(tk)
+            eng.release(tk)
+            print(policy_name, rep, "compress %.1f copy out %.1f copy in %.1f decompress %.1f us; wall %.1f us; %d bytes"
+                  % (t.compress_us, t.copy_out_us, t.copy_in_us, t.decompress_us, wall_us, info.bytes_out), flush=True)
+            assert first.copy_in_us == -1 and first.decompress_us == -1
+            assert mid.compress_us >= 0 and mid.copy_out_us > 0 and mid.copy_in_us == -1
+            assert t.compress_us == mid.compress_us and t.copy_out_us == mid.copy_out_us
+            assert t.copy_in_us > 0 and t.decompress_us >= 0
+            if info.policy != swap.NONE:
+                assert t.compress_us > 1 and t.decompress_us > 1
+            # a link of 20 to 100 GB/s
+            for c in (t.copy_out_us, t.copy_in_us):
+                assert info.bytes_out / 100e3 <= c <= info.bytes_out / 20e3 + 50, (c, info.bytes_out)
+            assert t.compress_us + t.copy_out_us + t.copy_in_us + t.decompress_us <= wall_us
+        assert torch.equal(out, x) or pol in (swap.ZFP,)
+    finally:
+        eng.close()
+    plain = swap.SwapEngine(pinned_bytes=64 << 20, device_bytes=64 << 20)
+    try:
+        tk = plain.pre(x[:4], swap.NONE)
+        with pytest.raises(CswapError):
+            plain.timing(tk)
+        plain.post(tk)
+        plain.release(tk)
+    finally:
+        plain.close()
+
+
+def test_pipeline_kernel_of_the_compaction_runs_beside_payload_copies(torch_cuda):
+    """The pipeline form of the single-pass compaction needs every one of its workgroups
+    resident at once, and on this GPU the engine's transfers are themselves kernels on the copy
+    streams.  A 256 MiB raw swap-out keeps the outbound copy stream busy for milliseconds; an
+    explicit ZVC request for a 192 MiB tensor issued right behind it must still finish its
+    single pass (a count of -1 would send the engine to the three kernels, which would show as
+    a second probe) with the payload the three kernels make, and in about the time it takes
+    alone."""
+    torch = torch_cuda
+    import time
+
+    from cswap_amd import swap
+    from cswap_amd._lib import lib
+
+    g = torch.Generator(device="cuda"); g.manual_seed(77)
+    big = torch.randn(64 << 20, generator=g, device="cuda").reshape(64, 64, 128, 128)        # 256 MiB, goes out raw
+    n = 48 << 20
+    x = torch.relu(torch.randn(n, generator=g, device="cuda")).reshape(48, 64, 128, 128)     # 192 MiB
+    nnz = int((x != 0).sum().item())
+    eng = swap.SwapEngine(pinned_bytes=640 << 20, device_bytes=320 << 20, timing=True)
+    try:
+        assert lib().cswap_zvc_takes_single_pass(n, eng.process_for(n)) == 1
+        alone = []
+        for _ in range(3):
+            tk = eng.pre(x, swap.SPARSE)
+            eng.post(tk)
+            alone.append(eng.timing(tk).compress_us)
+            eng.release(tk)
+        beside = []
+        for rep in range(3):
+            print("rep", rep, flush=True)
+            torch.cuda.synchronize()
+            tb = eng.pre(big, swap.NONE)                     # its copy is now running on the copy stream
+            before = eng.probe_count()
+            tk = eng.pre(x, swap.SPARSE)
+            assert eng.probe_count() == before + 1, "the single pass gave up and the three kernels ran"
+            info = eng.info(tk)
+            assert info.policy == swap.SPARSE and info.nnz == nnz
+            out = torch.full_like(x, -1.0)
+            eng.swap_in(tk, out)                             # from its staging block: its own copy waits behind the big one
+            torch.cuda.synchronize()
+            assert torch.equal(out, x)
+            eng.post(tb)
+            eng.post(tk)
+            beside.append(eng.timing(tk).compress_us)
+            eng.release(tk)
+            eng.release(tb)
+        print("single pass + count round trip, 192 MiB: alone %s us, beside a 256 MiB copy %s us"
+              % (["%.0f" % v for v in alone], ["%.0f" % v for v in beside]), flush=True)
+        assert min(beside) < 3 * min(alone) + 200
+    finally:
+        eng.close()
