@@ -111,8 +111,8 @@ def main():
         print(json.dumps(extras(torch, api, dev, zvc_only=args.zvc_mib)))
         return
     if args.swap_only:
-        from cswap_amd import swap
-        print(json.dumps({"swap": swap.bench_schedule(dev), "swap_backward": swap.bench_backward(dev)}))
+        import bench_parts
+        print(json.dumps({"swap": bench_parts.bench_schedule(dev), "swap_backward": bench_parts.bench_backward(dev)}))
         return
 
     rate = 8
@@ -184,7 +184,7 @@ def main():
         "vs_baseline": None, "dtype": "fp32", "data": "synthetic",
         "config": {"workload": "config5 attention probabilities fp32 [32,12,512,512] = softmax(N(0,1)), "
                                "zfp field nx=512 ny=512 nz=384, rate 8, compress then decompress",
-                   "bytes_in": 4 * n, "rate_bits_per_value": rate},
+                   "bytes_in": 4 * n},
         "roofline": roofline,
     }
     detail = {"clock_settle_s": CLOCK_SETTLE_S, "kernel_event_samples": len(evs),
@@ -209,23 +209,60 @@ def main():
     print(json.dumps(result))
 
 
+def zfp_cold_pair(torch, api, t, rate, copies, reps):
+    """[compress, decompress] in ms with nothing of a launch's operands left in the memory-side
+    cache (256 MB) from the launches before it: the loop rotates over `copies` separate fields,
+    streams and outputs, so that between two uses of a buffer more than the cache's size in
+    other traffic has gone by.  A timing loop over one tensor re-reads what the previous launch
+    left behind; in a swap the encoder's field was written by the producing layer a while ago
+    and the decoder's stream has just come over the link."""
+    from cswap_amd.workloads import field_dims
+
+    nx, ny, nz = field_dims(t.shape)
+    mb = 64 * rate
+    fields = [t] + [t.clone() for _ in range(copies - 1)]
+    streams = [torch.empty(api.zfp_stream_capacity(nx, ny, nz, mb), dtype=torch.uint8, device=t.device)
+               for _ in range(copies)]
+    outs = [torch.empty_like(t) for _ in range(copies)]
+    for f, s_ in zip(fields, streams):
+        api.cuda_compress(f, mb, out=s_)
+    state = {"i": 0}
+
+    def enc():
+        k = state["i"] % copies
+        state["i"] += 1
+        api.cuda_compress(fields[k], mb, out=streams[k])
+
+    def dec():
+        k = state["i"] % copies
+        state["i"] += 1
+        api.cuda_decompress(streams[k], t.shape, mb, out=outs[k])
+
+    return ev_ms(torch, enc, reps), ev_ms(torch, dec, reps)
+
+
 def headline_fractions(ex):
     """A few fractions of the 8 TB/s HBM roofline (algorithmic bytes) picked from
     the extra figures, short enough for the one-line record:
     [compress, decompress] for ZFP, [count+scan+compact, expand] for ZVC."""
     def pick(key, a, b):
         row = ex.get(key)
-        return [row[a], row[b]] if row else None
+        return [round(row[a], 3), round(row[b], 3)] if row and a in row else None
 
     also = {
         "zfp_r16_attn402MB": pick("zfp_attn_402MB_r16", "compress_hbm_frac", "decompress_hbm_frac"),
         "zfp_r8_ffn201MB": pick("zfp_config5_ffn_gelu_r8", "compress_hbm_frac", "decompress_hbm_frac"),
         "zfp_r8_hidden50MB": pick("zfp_config5_hidden_gelu_r8", "compress_hbm_frac", "decompress_hbm_frac"),
-        "zfp_r8_config3_34MB": pick("zfp_config3_64x32x32_r8", "compress_hbm_frac", "decompress_hbm_frac"),
-        "zfp_r8_config1_16MB": pick("zfp_config1_16MB_r8", "compress_hbm_frac", "decompress_hbm_frac"),
+        "zfp_r8_c3_34MB": pick("zfp_config3_64x32x32_r8", "compress_hbm_frac", "decompress_hbm_frac"),
+        "zfp_r8_c1_16MB": pick("zfp_config1_16MB_r8", "compress_hbm_frac", "decompress_hbm_frac"),
+        # the same three tensors with every launch's operands cold in the memory-side cache
+        "cold": {k: v for k, v in (("attn402MB", pick("zfp_attn_402MB_r8", "compress_hbm_frac_cold", "decompress_hbm_frac_cold")),
+                                   ("ffn201MB", pick("zfp_config5_ffn_gelu_r8", "compress_hbm_frac_cold", "decompress_hbm_frac_cold")),
+                                   ("hidden50MB", pick("zfp_config5_hidden_gelu_r8", "compress_hbm_frac_cold", "decompress_hbm_frac_cold")))
+                 if v is not None} or None,
         "zvc_256MiB": pick("zvc_relu_256MiB", "compress_total_hbm_frac", "expand_hbm_frac"),
         "zvc_512MiB": pick("zvc_relu_512MiB", "compress_total_hbm_frac", "expand_hbm_frac"),
-        "zvc_config2_50pct": pick("zvc_config2_s50", "compress_total_hbm_frac", "expand_hbm_frac"),
+        "zvc_c2_50pct": pick("zvc_config2_s50", "compress_total_hbm_frac", "expand_hbm_frac"),
     }
     zc = (ex.get("zvc_relu_256MiB") or {}).get("cpu_baseline")
     if zc:     # the CPU sparse path on the 256 MiB tensor, one core: [compress, expand] GB/s of fp32
@@ -234,7 +271,10 @@ def headline_fractions(ex):
         also["box_copy_GBs"] = ex["box_memory_GBs"]["copy_read_plus_write"]
     sw = ex.get("swap")
     if sw and "total_none_ms" in sw:
-        also["swap_config4_ms"] = {"raw": sw["total_none_ms"], "selector": sw["total_auto_ms"]}
+        # sums over the 44 tensors: raw, selector on first sight, selector with remembered decisions; and the
+        # largest compressed / raw latency ratio among the tensors the selector compressed (target: below 1)
+        also["swap_c4_ms"] = {"raw": sw["total_none_ms"], "auto": sw["total_auto_ms"],
+                              "memo": sw["total_remembered_ms"], "worst_vs_raw": sw["worst_compressed_over_raw"]}
     return {k: v for k, v in also.items() if v is not None}
 
 
@@ -477,6 +517,12 @@ def extras(torch, api, dev, zvc_only=0, cpu=False):
                 "compress_GBs_fp32": round(4 * n / e / 1e6, 1), "decompress_GBs_fp32": round(4 * n / d / 1e6, 1),
                 "compress_hbm_frac": round(bpv * n / e / 1e6 / HBM_PEAK_GBS, 4),
                 "decompress_hbm_frac": round(bpv * n / d / 1e6 / HBM_PEAK_GBS, 4)}
+            if label == "attn_402MB" and rate == 8:
+                ce, cd = zfp_cold_pair(torch, api, t, rate, 3, 30)     # 3 x (403 + 101) MB between two uses of a buffer
+                ex[f"zfp_{label}_r{rate}"].update({
+                    "compress_ms_cold": round(ce, 4), "decompress_ms_cold": round(cd, 4),
+                    "compress_hbm_frac_cold": round(bpv * n / ce / 1e6 / HBM_PEAK_GBS, 4),
+                    "decompress_hbm_frac_cold": round(bpv * n / cd / 1e6 / HBM_PEAK_GBS, 4)})
     # ---- what this box's memory gives plain kernels on the same 402.7 MB buffer (bytes moved per second):
     # torch's device copy (reads and writes it), fill (writes it), and this library's read-only counting pass
     other = torch.empty_like(big)
@@ -491,7 +537,7 @@ def extras(torch, api, dev, zvc_only=0, cpu=False):
     # ---- configuration 5's other tensors (rates 8 and 16) and configuration 3's stack (rates 4/8/16)
     from cswap_amd.workloads import config3_fields, config5_tensor_torch
 
-    def zfp_case(key, t, rate):
+    def zfp_case(key, t, rate, cold=0):
         n = t.numel()
         nx, ny, nz = field_dims(t.shape)
         mb = 64 * rate
@@ -507,11 +553,17 @@ def extras(torch, api, dev, zvc_only=0, cpu=False):
                    "compress_hbm_frac": round(bpv * n / e / 1e6 / HBM_PEAK_GBS, 4),
                    "decompress_hbm_frac": round(bpv * n / d / 1e6 / HBM_PEAK_GBS, 4),
                    "stream_over_input": round(s.numel() / (4 * n), 4)}
+        if cold:
+            ce, cd = zfp_cold_pair(torch, api, t, rate, cold, reps)
+            ex[key].update({"compress_ms_cold": round(ce, 4), "decompress_ms_cold": round(cd, 4),
+                            "compress_hbm_frac_cold": round(bpv * n / ce / 1e6 / HBM_PEAK_GBS, 4),
+                            "decompress_hbm_frac_cold": round(bpv * n / cd / 1e6 / HBM_PEAK_GBS, 4)})
 
     for name in ("hidden_gelu", "ffn_gelu"):
         t = config5_tensor_torch(name, dev, seed=0)
         for rate in (8, 16):
-            zfp_case(f"zfp_config5_{name}_r{rate}", t, rate)
+            # cold figures at 8 bits per value: 8 rotating copies (8 x 63 MB and 8 x 252 MB between two uses)
+            zfp_case(f"zfp_config5_{name}_r{rate}", t, rate, cold=8 if rate == 8 else 0)
         del t
     for name, f in config3_fields(batch=128).items():
         t = torch.from_numpy(f).to(dev)
@@ -541,17 +593,12 @@ def extras(torch, api, dev, zvc_only=0, cpu=False):
 
     zvc_extras(torch, api, dev, ex, config2_tensor, cpu=cpu)
 
-    try:
-        from cswap_amd import swap
-        ex["swap"] = swap.bench_schedule(dev)
-        ex["swap_backward"] = swap.bench_backward(dev)
-        from cswap_amd import planner
-        ex["planner"] = planner.bench_planner(dev)
-        from cswap_amd import hooks
-        ex["train_step"] = hooks.bench_training_step(dev)
-        ex["train_step_transformer"] = hooks.bench_transformer_step(dev)
-    except ImportError:
-        pass
+    import bench_parts
+    ex["swap"] = bench_parts.bench_schedule(dev)
+    ex["swap_backward"] = bench_parts.bench_backward(dev)
+    ex["planner"] = bench_parts.bench_planner(dev)
+    ex["train_step"] = bench_parts.bench_training_step(dev)
+    ex["train_step_transformer"] = bench_parts.bench_transformer_step(dev)
     return ex
 
 

@@ -239,141 +239,3 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
                 self.engine.release(h.ticket)
                 self._released.add(h.ticket)
         self._order.clear()
-
-
-def _measure_step(step, params, make_ctx, reps=5):
-    """Median and best wall time of ``step(ctx)`` over ``reps`` runs after two warm-up
-    runs (a step whose copies overlap compute differently from run to run has a
-    spread worth showing), the step's peak in torch's allocator above what is
-    allocated before it, and the hook statistics of the last run."""
-    import time
-
-    for _ in range(2):
-        step(make_ctx())
-    for p in params:
-        p.grad = None
-    torch.cuda.synchronize()
-    base = torch.cuda.memory_allocated()     # weights, input and whatever else the process holds
-    torch.cuda.reset_peak_memory_stats()
-    times = []
-    stats = None
-    for _ in range(reps):
-        ctx = make_ctx()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        step(ctx)
-        torch.cuda.synchronize()
-        times.append((time.perf_counter() - t0) * 1e3)
-        stats = ctx.stats if ctx is not None else None
-    times.sort()
-    return (times[len(times) // 2], times[0]), (torch.cuda.max_memory_allocated() - base) / 1e6, stats
-
-
-def _swap_rows(res, eng, step, params, min_bytes, reps):
-    memo = {}        # the selector's decisions, kept across the iterations of the last row
-    for label, pol, kw in (("raw_swap", swap.NONE, {}), ("selector", swap.AUTO, {}),
-                           ("selector_remembered", swap.AUTO, {"memo": memo})):
-        ms, mb, st = _measure_step(step, params,
-                                   lambda: swap_saved_tensors(eng, policy=pol, min_bytes=min_bytes, **kw), reps)
-        res[label] = {"step_ms": round(ms[0], 2), "step_ms_best": round(ms[1], 2), "step_peak_MB": round(mb, 1),
-                      "swapped_tensors": st["swapped"],
-                      "swapped_MB": round(st["bytes_in"] / 1e6, 1), "link_MB": round(st["bytes_out"] / 1e6, 1),
-                      "shared": st["shared"], "by_policy": dict(st.get("by_policy", {})),
-                      "prefetched": st.get("prefetched", 0), "resident": st.get("resident", 0),
-                      "kept_no_room": st.get("kept_no_room", 0), "memo_hits": st.get("memo_hits", 0)}
-
-
-def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int = 8 << 20) -> dict:
-    """Forward + backward of a VGG-16 (conv/BN/ReLU x13, 5 pools, linear head) on
-    random data with and without activation swapping through the saved-tensor
-    hooks: step time and peak device memory of the step (torch's allocator, above
-    what is allocated before the step).  Stock autograd, nothing patched."""
-
-    from .planner import _vgg_modules
-
-    torch.manual_seed(0)
-    feats = torch.nn.Sequential(*_vgg_modules(torch, dev))
-    head = torch.nn.Linear(512 * (image // 32) ** 2, 10).to(dev)
-    x = torch.randn(batch, 3, image, image, device=dev)
-    params = list(feats.parameters()) + list(head.parameters())
-
-    def step(ctx):
-        for p in params:
-            p.grad = None
-        if ctx is None:
-            loss = head(feats(x).flatten(1)).square().mean()
-        else:
-            with ctx:
-                loss = head(feats(x).flatten(1)).square().mean()
-        loss.backward()
-        if ctx is not None:
-            ctx.close()
-        return loss
-
-    res = {"model": f"VGG-16 BN, batch {batch}, 3x{image}x{image}", "min_bytes": min_bytes}
-    base_ms, base_mb, _ = _measure_step(step, params, lambda: None)
-    res["no_swap"] = {"step_ms": round(base_ms[0], 2), "step_peak_MB": round(base_mb, 1)}
-    staging = 192 << 20
-    eng = swap.SwapEngine(pinned_bytes=4 << 30, device_bytes=staging)
-    eng.calibrate()
-    res["staging_pool_MB"] = round(staging / 1e6, 1)    # device memory the engine holds besides torch's allocator
-    _swap_rows(res, eng, step, params, min_bytes, 9)
-    eng.close()
-    return res
-
-
-def bench_transformer_step(dev, layers: int = 4, batch: int = 32, seq: int = 512, hidden: int = 768, heads: int = 12,
-                           min_bytes: int = 8 << 20) -> dict:
-    """Forward + backward of a BERT-base-shaped encoder stack (attention written
-    out, so the [batch, heads, seq, seq] probabilities are saved as in
-    configuration 5; GELU feed-forward of 4 x hidden) with and without swapping
-    through the saved-tensor hooks.  No ReLU anywhere: the selector has only ZFP
-    and raw to choose from."""
-    import math
-
-    torch.manual_seed(0)
-
-    class Block(torch.nn.Module):
-        def __init__(self):
-            super().__init__()
-            self.qkv = torch.nn.Linear(hidden, 3 * hidden)
-            self.proj = torch.nn.Linear(hidden, hidden)
-            self.ln1 = torch.nn.LayerNorm(hidden)
-            self.ln2 = torch.nn.LayerNorm(hidden)
-            self.fc1 = torch.nn.Linear(hidden, 4 * hidden)
-            self.fc2 = torch.nn.Linear(4 * hidden, hidden)
-
-        def forward(self, x):
-            b, s, h = x.shape
-            q, k, v = self.qkv(self.ln1(x)).view(b, s, 3, heads, h // heads).permute(2, 0, 3, 1, 4)
-            p = torch.softmax(q @ k.transpose(-1, -2) / math.sqrt(h // heads), dim=-1)
-            x = x + self.proj((p @ v).transpose(1, 2).reshape(b, s, h))
-            return x + self.fc2(torch.nn.functional.gelu(self.fc1(self.ln2(x))))
-
-    net = torch.nn.Sequential(*[Block() for _ in range(layers)]).to(dev)
-    x = torch.randn(batch, seq, hidden, device=dev)
-    params = list(net.parameters())
-
-    def step(ctx):
-        for p in params:
-            p.grad = None
-        if ctx is None:
-            loss = net(x).square().mean()
-        else:
-            with ctx:
-                loss = net(x).square().mean()
-        loss.backward()
-        if ctx is not None:
-            ctx.close()
-
-    res = {"model": f"{layers} encoder blocks, batch {batch}, seq {seq}, hidden {hidden}, {heads} heads",
-           "min_bytes": min_bytes}
-    ms, mb, _ = _measure_step(step, params, lambda: None, 5)
-    res["no_swap"] = {"step_ms": round(ms[0], 2), "step_peak_MB": round(mb, 1)}
-    staging = 768 << 20
-    eng = swap.SwapEngine(pinned_bytes=12 << 30, device_bytes=staging)
-    eng.calibrate()
-    res["staging_pool_MB"] = round(staging / 1e6, 1)
-    _swap_rows(res, eng, step, params, min_bytes, 9)
-    eng.close()
-    return res

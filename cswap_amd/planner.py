@@ -77,19 +77,7 @@ class PolicyMaker:
         return self._plan(lib().cswap_planner_capuchin, n)
 
 
-# ------------------------------------------------------------------ measurement
-def _vgg_modules(torch, dev):
-    """VGG-16 feature extractor (conv/bn/relu x13, 5 pools; CSWAP+/vgg16-cifar10.cpp:77-97)."""
-    mods = []
-    cin = 3
-    for c, reps in [(64, 2), (128, 2), (256, 3), (512, 3), (512, 3)]:
-        for _ in range(reps):
-            mods += [torch.nn.Conv2d(cin, c, 3, padding=1), torch.nn.BatchNorm2d(c), torch.nn.ReLU()]
-            cin = c
-        mods.append(torch.nn.MaxPool2d(2))
-    return [m.to(dev) for m in mods]
-
-
+# ------------------------------------------------------------------ the walk of the reference's drivers
 def run_planned_iteration(engine, mods, x, policy, begin_stage, backward_factor: int = 2, check=None,
                           keep=None):
     """One iteration of the walk the reference's drivers do: forward with
@@ -147,58 +135,3 @@ def run_planned_iteration(engine, mods, x, policy, begin_stage, backward_factor:
                 mods[i](inp)
     torch.cuda.synchronize()
     return time.perf_counter() - t0
-
-
-def bench_planner(dev, batch: int = 128, ratio: float = 0.5) -> dict:
-    """Profile a VGG-16 forward at 3x64x64, plan with the calibrated cost model,
-    run the planned iteration and compare predicted with measured overhead, for
-    make_policy and for the raw-swap baseline."""
-    import time
-
-    import torch
-
-    from . import api, swap
-
-    torch.manual_seed(0)
-    mods = _vgg_modules(torch, dev)
-    for m in mods:
-        m.eval()
-    x = torch.randn(batch, 3, 64, 64, device=dev)
-    n = len(mods)
-    eng = swap.SwapEngine(pinned_bytes=3 << 30, device_bytes=1 << 30)
-    costs = eng.calibrate()
-    pm = PolicyMaker(costs)
-    with torch.no_grad():
-        for _ in range(2):                      # warm up kernels and allocator
-            t = x
-            for m in mods:
-                t = m(t)
-        t, tid = x, -1
-        for i, m in enumerate(mods):
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            out = m(t)
-            torch.cuda.synchronize()
-            pm.add_comptime((time.perf_counter() - t0) * 1e6)
-            pm.add_tensor(i, out.numel() * 4)
-            pm.add_stepdep([tid, i])
-            nx, ny, nz = swap.field_dims(out.shape)
-            pm.set_field(i, nx, ny, nz)
-            pm.set_nnz(i, int(api.probe_nnz(out).item()))
-            t, tid = out, i
-    pm.init(ratio)
-    res = {"ratio": ratio, "ops": n}
-    none_s = min(run_planned_iteration(eng, mods, x, [0] * n, list(range(1, n + 1))) for _ in range(3))
-    res["measured_none_ms"] = round(none_s * 1e3, 2)
-    for label, fn in (("make_policy", pm.make_policy), ("capuchin", pm.capuchin)):
-        pol, t_us = fn(n)
-        s = pm.summary
-        best = min(run_planned_iteration(eng, mods, x, pol, pm.begin_stage) for _ in range(3))
-        res[label] = {"policy": pol, "predicted_overhead_ms": round((t_us - s.base_time_us) / 1e3, 2),
-                      "measured_overhead_ms": round((best - none_s) * 1e3, 2),
-                      "moved_MB": round(s.bytes_moved / 1e6, 1), "link_MB": round(s.bytes_on_link / 1e6, 1),
-                      "selected": s.n_selected}
-    res["base_predicted_ms"] = round(pm.summary.base_time_us / 1e3, 2)
-    eng.close()
-    pm.close()
-    return res

@@ -173,3 +173,23 @@ def config5_tensor_numpy(name: str, batch: int, seed: int = 0) -> np.ndarray:
     xd = x.astype(np.float64)
     erf = np.vectorize(math.erf)
     return (0.5 * xd * (1.0 + erf(xd / math.sqrt(2.0)))).astype(np.float32)
+
+
+def dummy_layer_compute(a, b, reps: int) -> None:
+    """Stand-in for a layer's kernels that run on the compute stream while a copy is in flight."""
+    import torch
+
+    for _ in range(reps):
+        torch.mm(a, b)
+
+
+def vgg16_modules(torch, dev):
+    """VGG-16 feature extractor (conv/bn/relu x13, 5 pools; CSWAP+/vgg16-cifar10.cpp:77-97)."""
+    mods = []
+    cin = 3
+    for c, reps in [(64, 2), (128, 2), (256, 3), (512, 3), (512, 3)]:
+        for _ in range(reps):
+            mods += [torch.nn.Conv2d(cin, c, 3, padding=1), torch.nn.BatchNorm2d(c), torch.nn.ReLU()]
+            cin = c
+        mods.append(torch.nn.MaxPool2d(2))
+    return [m.to(dev) for m in mods]

@@ -36,7 +36,7 @@ typedef struct {
 } cswap_zfp_stream;
 
 typedef struct {
-  int type;                 /* 3 = float (zfp_type_float); other types are not supported */
+  int type;                 /* zfp_type: 1 = int32, 2 = int64, 3 = float, 4 = double (cuZFP.cu:389-423) */
   size_t nx, ny, nz, nw;
   ptrdiff_t sx, sy, sz, sw; /* 0 = contiguous */
   void* data;               /* DEVICE or host memory */

@@ -69,7 +69,7 @@ def test_config4_schedule_through_the_selector(torch_cuda):
     torch = torch_cuda
     import oracle
     from cswap_amd import swap
-    from cswap_amd.workloads import config4_schedule, config4_tensor, field_dims
+    from cswap_amd.workloads import config4_schedule, config4_tensor, dummy_layer_compute, field_dims
 
     sched = config4_schedule(128)
     assert len(sched) == 44
@@ -91,7 +91,7 @@ def test_config4_schedule_through_the_selector(torch_cuda):
                     torch.cuda.synchronize()
                     t0 = time.perf_counter()
                     tk = eng.pre(x, pol)
-                    swap._dummy_compute(a, b, 2)      # the layer's kernels, while the copy is in flight
+                    dummy_layer_compute(a, b, 2)      # the layer's kernels, while the copy is in flight
                     eng.post(tk)
                     eng.swap_in(tk, out)
                     torch.cuda.synchronize()

@@ -127,11 +127,12 @@ def test_planned_iteration_restores_every_swapped_tensor():
     import torch
 
     from cswap_amd import api, swap
-    from cswap_amd.planner import PolicyMaker, _vgg_modules, run_planned_iteration
+    from cswap_amd.planner import PolicyMaker, run_planned_iteration
+    from cswap_amd.workloads import vgg16_modules
 
     torch.manual_seed(0)
     dev = torch.device("cuda")
-    mods = [m.eval() for m in _vgg_modules(torch, dev)][:17]
+    mods = [m.eval() for m in vgg16_modules(torch, dev)][:17]
     x = torch.randn(16, 3, 64, 64, device=dev)
     costs = swap.default_costs()
     costs.allow_lossy = 0
