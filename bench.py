@@ -92,6 +92,12 @@ def main():
     ap.add_argument("--zvc-only", action="store_true",
                     help="run only one ReLU zero-value-compaction case (for profiling); prints its figures")
     ap.add_argument("--zvc-mib", type=int, default=256, help="size of the --zvc-only tensor in MiB")
+    ap.add_argument("--zfp-only", choices=sorted(ZFP_ONLY_CASES),
+                    help="run only the ZFP kernels on one of the smaller workloads, each in a loop of its own "
+                         "(for profiling); prints its figures")
+    ap.add_argument("--zfp-form", choices=["shipped", "lane", "pair"], default="shipped",
+                    help="with --zfp-only: the kernel form, as shipped (by field size), one lane per block, "
+                         "or the pair form wherever the shape allows")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; run with --gpus 1 "
@@ -109,6 +115,9 @@ def main():
     torch.cuda.set_device(dev)
     if args.zvc_only:
         print(json.dumps(extras(torch, api, dev, zvc_only=args.zvc_mib)))
+        return
+    if args.zfp_only:
+        print(json.dumps(zfp_only(torch, api, dev, args.zfp_only, args.zfp_form)))
         return
     if args.swap_only:
         import bench_parts
@@ -239,6 +248,44 @@ def zfp_cold_pair(torch, api, t, rate, copies, reps):
         api.cuda_decompress(streams[k], t.shape, mb, out=outs[k])
 
     return ev_ms(torch, enc, reps), ev_ms(torch, dec, reps)
+
+
+# --zfp-only: name -> (what it is, rate)
+ZFP_ONLY_CASES = {"config1": ("config 1, PReLU(N(0,1)) fp32 [64,64,32,32], 16.8 MB", 8),
+                  "config3_34MB": ("config 3, fp32 [128,64,32,32], 33.6 MB", 8),
+                  "hidden50MB": ("config 5, GELU(N(0,1)) fp32 [32,512,768], 50.3 MB", 8),
+                  "ffn201MB_r16": ("config 5, GELU(N(0,1)) fp32 [32,512,3072], 201.3 MB, 16 bits per value", 16)}
+
+
+def zfp_only(torch, api, dev, name, form):
+    """One of the smaller ZFP workloads, compress and decompress each in a loop of its own."""
+    import ctypes as C
+
+    from cswap_amd._lib import lib
+    from cswap_amd.workloads import config1_field, config3_fields, config5_tensor_torch, field_dims
+
+    if form != "shipped":
+        big = C.c_size_t(-1).value
+        lib().cswap_zfp_set_pair_bytes(big if form == "pair" else 0, big if form == "pair" else 0, None)
+    what, rate = ZFP_ONLY_CASES[name]
+    if name == "config1":
+        t = torch.from_numpy(config1_field()).to(dev)
+    elif name == "config3_34MB":
+        t = torch.from_numpy(config3_fields(batch=128)["64x32x32"]).to(dev)
+    else:
+        t = config5_tensor_torch("hidden_gelu" if name == "hidden50MB" else "ffn_gelu", dev, seed=0)
+    n = t.numel()
+    nx, ny, nz = field_dims(t.shape)
+    mb = 64 * rate
+    s = torch.empty(api.zfp_stream_capacity(nx, ny, nz, mb), dtype=torch.uint8, device=dev)
+    o = torch.empty_like(t)
+    api.cuda_compress(t, mb, out=s); api.cuda_decompress(s, t.shape, mb, out=o)
+    e = ev_ms(torch, lambda: api.cuda_compress(t, mb, out=s), 2000, settle_s=0.1)
+    d = ev_ms(torch, lambda: api.cuda_decompress(s, t.shape, mb, out=o), 2000, settle_s=0.1)
+    bpv = 4 + rate / 8
+    return {"workload": what, "form": form, "rate": rate, "compress_us": round(e * 1e3, 2), "decompress_us": round(d * 1e3, 2),
+            "compress_hbm_frac": round(bpv * n / e / 1e6 / HBM_PEAK_GBS, 4),
+            "decompress_hbm_frac": round(bpv * n / d / 1e6 / HBM_PEAK_GBS, 4)}
 
 
 def headline_fractions(ex):
