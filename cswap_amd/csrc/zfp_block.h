@@ -1268,6 +1268,140 @@ CSWAP_HD void decode_block(Mem& mem, unsigned pos0, unsigned maxbits, float (&f)
   }
 }
 
+// ---------------------------------------------------------------- one block, two wavefronts: decoding
+// The pair form of the decoder.  Where a bit plane starts in a block's stream is only known once
+// the planes before it are decoded, so the planes stay one chain per block: half 0 decodes them
+// for all 64 blocks (lane per block, as the one-wavefront kernel does) while half 1 waits; what
+// comes after -- the bit transposes, the reorder, the inverse lifting, the cast and the stores --
+// is split as in pair_encode_half, mirrored:
+//   planes    half 0 hands over the plane words; each half takes its 32 bits of every plane: the
+//             coefficients 32 H .. 32 H + 31 in coding order after the transposes   (exchange 1;
+//             once more for the low 16 planes, when some block of the 64 has budget left for them)
+//   reorder   half 0 needs the coefficients of z-index 0 and 2, half 1 those of 1 and 3: 19 of a
+//             half's 32 are among its own, 13 come from the partner                    (exchange 2)
+//   lifting along z (inv_lift4 on (x, y, z, w) = z-index 0, 1, 2, 3): its first lines pair y with
+//             w and z with x -- what each half holds --, the last two pair y with z and w with x:
+//             half 0 sends z and gets w, half 1 the reverse                            (exchange 3)
+//             half 0 ends with the slices z = 0 and 3, half 1 with 2 and 1, as the encoder's halves
+//             start
+//   lifting along y and x of both slices, cast: no exchange
+// Results are those of decode_block.
+//
+// Exchange (every call is made by both halves, in this order):
+//   void     plane_put(int k, uint64_t), scale_put(float)        half 0 only, before planes_sync
+//   bool     planes_sync(bool)              half 0's answer (do the low planes follow) for both
+//   uint32_t plane_get(int k)               my 32 bits of plane word k;  float scale_get()
+//   void     consumed(), low_sync()         around half 0's decoding of the low planes, if they follow
+//   void     seq_put(int slot, uint32_t), seq_sync(), uint32_t seq_get(int slot)
+//   void     swap16(const int32_t(&)[16], int32_t(&)[16])
+template <class Dec>
+CSWAP_HD void pair_decode16(Dec& dec, uint64_t (&x)[16], bool top)
+{
+#pragma unroll
+  for (int k = 15; k >= 0; k--) {
+    x[k] = 0;  // planes that no block of the wavefront can reach are zero without a read
+    if (CSWAP_ANY(dec.active())) x[k] = (top && k >= 12) ? dec.leading_plane() : dec.plane();
+  }
+}
+
+// p, q receive the half's two z-slices ([x + 4y]; half 0: z = 0 and 3, half 1: z = 2 and 1).
+// The block owns [pos0, pos0 + maxbits) of the bit region behind mem, followed by a fence of
+// one-bits (only half 0 reads it).
+template <int H, class Ex, class Mem>
+CSWAP_HD void pair_decode_half(Mem& mem, unsigned pos0, unsigned maxbits, Ex& ex, float (&p)[16], float (&q)[16])
+{
+  BlockDecoder<Mem, 64, true> dec(mem, pos0, maxbits);
+  uint64_t x[16];
+  bool any = false;
+  if (H == 0) {
+    const uint32_t h = (uint32_t)dec.window(pos0);
+    const bool coded = (h & 1) != 0;  // an empty block: its budget counts as spent, every plane reads as zero
+    dec.pos = coded ? pos0 + 9 : dec.limit;
+    pair_decode16(dec, x, true);
+#pragma unroll
+    for (int k = 0; k < 16; k++) ex.plane_put(k, x[k]);
+    ex.scale_put(coded ? decode_scale((h >> 1) & 0xffu) : 0.0f);
+    any = CSWAP_ANY(dec.active());
+  }
+  const bool low = ex.planes_sync(any);
+  uint32_t a[32];
+#pragma unroll
+  for (int k = 0; k < 16; k++) a[16 + k] = ex.plane_get(k);
+  const float w = ex.scale_get();
+  tr_half<16, kNotIn>(a);
+  uint32_t c = kNegabinary;
+  if (low) {
+    ex.consumed();
+    if (H == 0) {
+      pair_decode16(dec, x, false);
+#pragma unroll
+      for (int k = 0; k < 16; k++) ex.plane_put(k, x[k]);
+    }
+    ex.low_sync();
+#pragma unroll
+    for (int k = 0; k < 16; k++) a[k] = ex.plane_get(k);
+    tr_half<0, kNotIn>(a);
+  } else {  // no low planes: their complemented odd planes are missing from the minuend as well
+#pragma unroll
+    for (int k = 0; k < 16; k++) a[k] = 0;
+    c = kNegabinary & 0xffff0000u;
+  }
+  tr_stage<16, 0, 32>(a);
+
+  // a[i] is coefficient 32 H + i of the coding order with the negabinary constant still added
+#pragma unroll
+  for (int r = 0; r < 32; r++)  // what the partner needs of mine
+    if (!PairMap<1 - H>::stays(r)) ex.seq_put(PairMap<1 - H>::sent_before(r), a[PairMap<1 - H>::row(r)] - c);
+  ex.seq_sync();
+  int32_t v[32];
+#pragma unroll
+  for (int r = 0; r < 32; r++)
+    v[r] = (int32_t)(PairMap<H>::stays(r) ? a[PairMap<H>::row(r)] - c : ex.seq_get(PairMap<H>::sent_before(r)));
+
+  // lifting along z.  Half 0 holds x = v[i], z = v[16 + i]; half 1 holds y = v[i], w = v[16 + i].
+  int32_t keep[16], send[16], got[16];
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    if (H == 0) {  // z += x; x -= z_before
+      const int32_t z0 = v[16 + i];
+      send[i] = wadd(z0, v[i]);
+      keep[i] = wsub(v[i], z0);
+    } else {       // y += w >> 1; w -= y >> 1; y += w; w -= y_before
+      int32_t y = wadd(v[i], v[16 + i] >> 1);
+      int32_t ww = wsub(v[16 + i], y >> 1);
+      keep[i] = wadd(y, ww);
+      send[i] = wsub(ww, y);
+    }
+  }
+  ex.swap16(send, got);
+  int32_t ip[16], iq[16];
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    if (H == 0) {  // keep = x, got = w:  w += x; x -= w_before   -> slices 0 (x) and 3 (w)
+      iq[i] = wadd(got[i], keep[i]);
+      ip[i] = wsub(keep[i], got[i]);
+    } else {       // keep = y, got = z:  y += z; z -= y_before   -> slices 2 (z) and 1 (y)
+      iq[i] = wadd(keep[i], got[i]);
+      ip[i] = wsub(got[i], keep[i]);
+    }
+  }
+#pragma unroll
+  for (int xx = 0; xx < 4; xx++) {
+    inv_lift4(ip[xx], ip[xx + 4], ip[xx + 8], ip[xx + 12]);
+    inv_lift4(iq[xx], iq[xx + 4], iq[xx + 8], iq[xx + 12]);
+  }
+#pragma unroll
+  for (int y = 0; y < 4; y++) {
+    inv_lift4(ip[4 * y], ip[4 * y + 1], ip[4 * y + 2], ip[4 * y + 3]);
+    inv_lift4(iq[4 * y], iq[4 * y + 1], iq[4 * y + 2], iq[4 * y + 3]);
+  }
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    p[i] = w * (float)ip[i];
+    q[i] = w * (float)iq[i];
+  }
+}
+
 // ---------------------------------------------------------------- 2-D and 1-D blocks
 // Blocks of 4x4 = 16 and 4 values (CSWAP+/zfp/encode2.cuh, encode1.cuh,
 // decode2.cuh, decode1.cuh): same cast and coder with 16 / 4 coefficients, lifting

@@ -514,6 +514,120 @@ __global__ __launch_bounds__(128) void zfp_encode3_f32_pair_kernel(const float* 
   }
 }
 
+// The pair form of the decoder (zfp_block.h: pair_decode_half).  Dynamic LDS, in dwords:
+// [region: dec_region_dwords(maxbits)] [scales: 64] [flag: 4] [U0: 1024] [U1: 1024].
+//   planes     half 0 writes the low words of 16 plane words into U0 and the high words into U1
+//              (k * 64 + lane)                                                barrier  half h reads U_h
+//              (the same again for the low 16 planes, between two more barriers, when they follow)
+//   reorder    half h writes the 13 coefficients it sends into U_h (slot * 64 + lane)
+//                                                                              barrier  reads U_(1-h)
+//   z exchange half h writes into U_(1-h) (j * 64 + lane)                     barrier  reads U_h
+// again a half only ever writes into the one it was the last to read.
+constexpr unsigned kPairScales = 64, kPairDecU = 1024;
+__host__ __device__ inline unsigned pair_dec_lds_dwords(unsigned maxbits)
+{
+  return dec_region_dwords(maxbits) + kPairScales + kPairFlag + 2 * kPairDecU;
+}
+
+template <int H>
+struct LdsDecExchange {
+  float* scales;
+  uint32_t* flag;
+  uint32_t* u0;
+  uint32_t* u1;
+  unsigned lane;
+  __device__ __forceinline__ uint32_t* mine() const { return H == 0 ? u0 : u1; }
+  __device__ __forceinline__ uint32_t* theirs() const { return H == 0 ? u1 : u0; }
+  __device__ __forceinline__ void plane_put(int k, uint64_t x)
+  {
+    u0[k * 64 + lane] = (uint32_t)x;
+    u1[k * 64 + lane] = (uint32_t)(x >> 32);
+  }
+  __device__ __forceinline__ void scale_put(float w) { scales[lane] = w; }
+  __device__ __forceinline__ bool planes_sync(bool any)
+  {
+    if (H == 0 && lane == 0) *flag = any ? 1u : 0u;
+    __syncthreads();
+    return __builtin_amdgcn_readfirstlane(*flag) != 0;
+  }
+  __device__ __forceinline__ uint32_t plane_get(int k) { return mine()[k * 64 + lane]; }
+  __device__ __forceinline__ float scale_get() { return scales[lane]; }
+  __device__ __forceinline__ void consumed() { __syncthreads(); }
+  __device__ __forceinline__ void low_sync() { __syncthreads(); }
+  __device__ __forceinline__ void seq_put(int slot, uint32_t v) { mine()[slot * 64 + lane] = v; }
+  __device__ __forceinline__ void seq_sync() { __syncthreads(); }
+  __device__ __forceinline__ uint32_t seq_get(int slot) { return theirs()[slot * 64 + lane]; }
+  __device__ __forceinline__ void swap16(const int32_t (&out)[16], int32_t (&in)[16])
+  {
+#pragma unroll
+    for (int j = 0; j < 16; j++) theirs()[j * 64 + lane] = (uint32_t)out[j];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 16; j++) in[j] = (int32_t)mine()[j * 64 + lane];
+  }
+};
+
+template <int H>
+__device__ __forceinline__ void pair_decode_body(const Field3& fd, unsigned maxbits, uint32_t* lds, unsigned lane,
+                                                 uint32_t first, float* __restrict__ out)
+{
+  const unsigned region = dec_region_dwords(maxbits);
+  LdsDecExchange<H> ex;
+  ex.scales = reinterpret_cast<float*>(lds + region);
+  ex.flag = lds + region + kPairScales;
+  ex.u0 = lds + region + kPairScales + kPairFlag;
+  ex.u1 = ex.u0 + kPairDecU;
+  ex.lane = lane;
+  LdsBits mem(lds);
+  float p[16], q[16];
+  pair_decode_half<H>(mem, mem.bit0 + lane * dec_slot_bits(maxbits), maxbits, ex, p, q);
+  if (first + lane < fd.nblocks) {
+    uint32_t x0, y0, z0;
+    block_origin(fd, first + lane, x0, y0, z0);
+    const WaveBase w = wave_base(fd, first);
+    char* base = reinterpret_cast<char*>(out + w.origin);
+    const uint32_t me = lane_bytes(fd, w, x0, y0, z0);
+    const uint32_t sy4 = (uint32_t)fd.sy * 4u, sz4 = (uint32_t)fd.sz * 4u;
+    constexpr int ZP = H == 0 ? 0 : 2, ZQ = H == 0 ? 3 : 1;
+#pragma unroll
+    for (int y = 0; y < 4; y++) {
+      const stream_f4 vp = {p[4 * y], p[4 * y + 1], p[4 * y + 2], p[4 * y + 3]};
+      const stream_f4 vq = {q[4 * y], q[4 * y + 1], q[4 * y + 2], q[4 * y + 3]};
+      __builtin_nontemporal_store(vp, reinterpret_cast<stream_f4*>(base + (size_t)(me + (y * sy4 + ZP * sz4))));
+      __builtin_nontemporal_store(vq, reinterpret_cast<stream_f4*>(base + (size_t)(me + (y * sy4 + ZQ * sz4))));
+    }
+  }
+}
+
+__global__ __launch_bounds__(128) void zfp_decode3_f32_pair_kernel(const uint64_t* __restrict__ stream, Field3 fd,
+                                                                   unsigned maxbits, float* __restrict__ out)
+{
+  extern __shared__ uint4 lds_raw[];
+  uint32_t* lds = reinterpret_cast<uint32_t*>(lds_raw);
+  const unsigned tid = threadIdx.x, lane = tid & 63u;
+  const uint32_t first = blockIdx.x * 64u;
+  {  // thread t brings in half of block t / 2; the fence of ones behind every block comes with the second half.
+     // The slots of blocks past the end of the field read as empty blocks.
+    const unsigned W = maxbits >> 6;
+    const uint32_t blk = first + (tid >> 1);
+    uint64_t* dst = reinterpret_cast<uint64_t*>(lds + (tid >> 1) * (dec_slot_bits(maxbits) / 32)) + (tid & 1u) * (W / 2);
+    if (blk < fd.nblocks) {
+      const ulonglong2* src = reinterpret_cast<const ulonglong2*>(stream + (size_t)blk * W + (tid & 1u) * (W / 2));
+      for (unsigned j = 0; j < W / 4; j++) {
+        const ulonglong2 v = src[j];
+        dst[2 * j] = v.x;
+        dst[2 * j + 1] = v.y;
+      }
+    } else {
+      for (unsigned j = 0; j < W / 2; j++) dst[j] = 0;
+    }
+    if (tid & 1u) dst[W / 2] = ~0ull;
+  }
+  __syncthreads();
+  if (__builtin_amdgcn_readfirstlane(tid >> 6) == 0) pair_decode_body<0>(fd, maxbits, lds, lane, first, out);
+  else pair_decode_body<1>(fd, maxbits, lds, lane, first, out);
+}
+
 // ------------------------------------------------------------- 64-bit elements
 // Fields of doubles or int64 (zfp_type_double, zfp_type_int64): the same
 // decomposition, values moved as 64-bit patterns.  Fast path: full block whose
@@ -984,6 +1098,12 @@ static int decompress3(const uint64_t* d_stream, Elem elem, size_t nx, size_t ny
   hipStream_t st = (hipStream_t)stream;
   const bool whole = (maxbits & 63u) == 0;
   const bool is_int = elem == kI32 || elem == kI64;
+  if (elem == kF32 && pair_shape(fd, maxbits) &&
+      (unsigned long long)nx * ny * nz * 4ull < g_pair_decode_bytes.load(std::memory_order_relaxed)) {
+    hipLaunchKernelGGL(zfp_decode3_f32_pair_kernel, dim3(grid), dim3(128), (size_t)pair_dec_lds_dwords(maxbits) * 4, st,
+                       d_stream, fd, maxbits, static_cast<float*>(d_out));
+    return check_launch();
+  }
   if (elem_bytes(elem) == 4) {
     float* out = static_cast<float*>(d_out);
     lds_bytes = (size_t)dec_region_dwords(maxbits) * 4;

@@ -401,3 +401,83 @@ int host_skip_plane_agrees(uint64_t x, unsigned n, unsigned pos, unsigned maxbit
   return a.n == b.n && a.pos == b.pos;
 }
 }
+
+// ---- the decoder's pair form, the same way: two threads, the kernel's reuse of its shared words
+namespace {
+struct PairDecShared {
+  float scale;
+  uint32_t u[2][16];
+  int flag;
+  pthread_barrier_t bar;
+};
+template <int H>
+struct HostDecExchange {
+  PairDecShared& sh;
+  void wait() { pthread_barrier_wait(&sh.bar); }
+  void plane_put(int k, uint64_t x) { sh.u[0][k] = (uint32_t)x; sh.u[1][k] = (uint32_t)(x >> 32); }
+  void scale_put(float w) { sh.scale = w; }
+  bool planes_sync(bool any) { if (H == 0) sh.flag = any; wait(); return sh.flag != 0; }
+  uint32_t plane_get(int k) { return sh.u[H][k]; }
+  float scale_get() { return sh.scale; }
+  void consumed() { wait(); }
+  void low_sync() { wait(); }
+  void seq_put(int slot, uint32_t v) { sh.u[H][slot] = v; }
+  void seq_sync() { wait(); }
+  uint32_t seq_get(int slot) { return sh.u[1 - H][slot]; }
+  void swap16(const int32_t (&out)[16], int32_t (&in)[16])
+  {
+    for (int j = 0; j < 16; j++) sh.u[1 - H][j] = (uint32_t)out[j];
+    wait();
+    for (int j = 0; j < 16; j++) in[j] = (int32_t)sh.u[H][j];
+  }
+};
+struct PairDecJob {
+  const uint32_t* slots; unsigned slot_dwords; size_t nx, ny, nz; unsigned maxbits; float* out; PairDecShared* sh;
+};
+template <int H>
+void* pair_dec_thread(void* arg)
+{
+  PairDecJob& j = *static_cast<PairDecJob*>(arg);
+  const size_t mx = j.nx / 4, my = j.ny / 4, mz = j.nz / 4;
+  HostDecExchange<H> ex{*j.sh};
+  for (size_t b = 0; b < mx * my * mz; b++) {
+    const size_t x0 = (b % mx) * 4, y0 = ((b / mx) % my) * 4, z0 = (b / (mx * my)) * 4;
+    const int zp = H == 0 ? 0 : 2, zq = H == 0 ? 3 : 1;
+    ArrayBits mem{const_cast<uint32_t*>(j.slots + b * j.slot_dwords)};
+    float p[16], q[16];
+    cswap::pair_decode_half<H>(mem, 0u, j.maxbits, ex, p, q);
+    for (int y = 0; y < 4; y++) for (int x = 0; x < 4; x++) {
+      j.out[(x0 + x) + j.nx * ((y0 + y) + j.ny * (z0 + zp))] = p[x + 4 * y];
+      j.out[(x0 + x) + j.nx * ((y0 + y) + j.ny * (z0 + zq))] = q[x + 4 * y];
+    }
+    ex.wait();  // the shared words are reused by the next block
+  }
+  return nullptr;
+}
+}
+
+extern "C" int host_zfp_decode3_pair(const uint64_t* stream, size_t nx, size_t ny, size_t nz, unsigned maxbits, float* out)
+{
+  if (nx % 4 || ny % 4 || nz % 4 || maxbits % 64) return -1;
+  const size_t nb = (nx / 4) * (ny / 4) * (nz / 4);
+  const unsigned W = maxbits / 64, slot_dwords = 2 * W + 16;
+  std::vector<uint32_t> slots(nb * slot_dwords);
+  uint32_t junk = 12345u;
+  for (size_t b = 0; b < nb; b++) {  // the block, its fence of 64 ones, then whatever
+    uint32_t* s = slots.data() + b * slot_dwords;
+    memcpy(s, stream + b * W, 8 * (size_t)W);
+    s[2 * W] = s[2 * W + 1] = 0xffffffffu;
+    for (unsigned d = 2 * W + 2; d < slot_dwords; d++) s[d] = junk = junk * 1664525u + 1013904223u;
+  }
+  PairDecShared sh;
+  memset(&sh, 0, sizeof sh);
+  if (pthread_barrier_init(&sh.bar, nullptr, 2)) return -1;
+  PairDecJob job{slots.data(), slot_dwords, nx, ny, nz, maxbits, out, &sh};
+  pthread_t t0, t1;
+  pthread_create(&t0, nullptr, pair_dec_thread<0>, &job);
+  pthread_create(&t1, nullptr, pair_dec_thread<1>, &job);
+  pthread_join(t0, nullptr);
+  pthread_join(t1, nullptr);
+  pthread_barrier_destroy(&sh.bar);
+  return 0;
+}

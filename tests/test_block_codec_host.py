@@ -262,6 +262,8 @@ def _pair(host):
     host.host_zfp_encode3_pair.restype = C.c_uint
     host.host_skip_plane_agrees.argtypes = [C.c_uint64, C.c_uint, C.c_uint, C.c_uint]
     host.host_skip_plane_agrees.restype = C.c_int
+    host.host_zfp_decode3_pair.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_void_p]
+    host.host_zfp_decode3_pair.restype = C.c_int
     return host
 
 
@@ -330,3 +332,46 @@ def test_pair_form_of_the_encoder_matches_golden_vectors_and_the_block_encoder(h
                 top = L.host_zfp_encode3_pair(f.ctypes.data, nx, ny, nz, maxbits, s.ctypes.data)
                 assert np.array_equal(s, want[:words]), (kind, shape, maxbits)
                 assert top < maxbits // 32 + 4, (kind, shape, maxbits, top)
+
+
+@pytest.mark.timeout(600)
+def test_pair_form_of_the_decoder_matches_golden_vectors_and_the_block_decoder(host, golden):
+    """The decoder's pair form (half 0 decodes the bit planes, both halves share what follows; here
+    two threads with the kernel's reuse of its shared words) gives the decoded values of the golden
+    vectors and of decode_block on the streams of random fields, at every whole-word rate."""
+    L = _pair(host)
+    n = 0
+    for name, rate, maxbits, f, stream, dec in golden_cases(golden):
+        nz, ny, nx = f.shape
+        if nx % 4 or ny % 4 or nz % 4 or maxbits % 64:
+            continue
+        words = (nx // 4) * (ny // 4) * (nz // 4) * maxbits // 64
+        g = np.zeros(words * 8, dtype=np.uint8)
+        g[:] = stream[:words * 8]
+        o = np.full(f.shape, -7.0, dtype=np.float32)
+        assert L.host_zfp_decode3_pair(g.ctypes.data, nx, ny, nz, maxbits, o.ctypes.data) == 0
+        assert np.array_equal(o.view(np.uint32), dec.view(np.uint32)), (name, rate)
+        n += 1
+    assert n >= 20, n
+    rng = np.random.default_rng(6)
+    kinds = {
+        "noise": lambda shape: rng.standard_normal(shape),
+        "smooth": lambda shape: np.cumsum(np.cumsum(rng.standard_normal(shape), axis=2), axis=1) * 1e-3,
+        "sparse": lambda shape: rng.standard_normal(shape) * (rng.random(shape) < 0.05),
+        "wide": lambda shape: rng.standard_normal(shape) * np.exp(8 * rng.standard_normal(shape)),
+        "const": lambda shape: np.full(shape, 1.5),
+        "zero": lambda shape: np.zeros(shape),
+    }
+    for kind, make in kinds.items():
+        for shape in ((4, 4, 4), (8, 12, 16)):
+            f = np.ascontiguousarray(make(shape), dtype=np.float32)
+            nz, ny, nx = shape
+            for maxbits in (64, 128, 256, 512, 1024, 2048, 4096):
+                words = (nx // 4) * (ny // 4) * (nz // 4) * maxbits // 64
+                s = np.zeros(words + 2, dtype=np.uint64)
+                host.host_zfp_encode3(f.ctypes.data, nx, ny, nz, maxbits, s.ctypes.data)
+                want = np.zeros_like(f)
+                host.host_zfp_decode3(s.ctypes.data, nx, ny, nz, maxbits, want.ctypes.data)
+                o = np.full(f.shape, -7.0, dtype=np.float32)
+                assert L.host_zfp_decode3_pair(s.ctypes.data, nx, ny, nz, maxbits, o.ctypes.data) == 0
+                assert np.array_equal(o.view(np.uint32), want.view(np.uint32)), (kind, shape, maxbits)

@@ -55,5 +55,11 @@ def test_zfp_fp32_kernels_fit_five_waves_without_scratch():
         else:
             assert v["VGPRs"] <= 96 and v["Occupancy"] >= 5, (k, v)
     assert fewer == {"Li3E": 4, "Li4E": 2}, fewer
+    # the pair forms for small fields (two wavefronts per 64 blocks): small enough in registers that
+    # the LDS of their workgroups, not the register file, bounds how many are resident
+    pair = {k: v for k, v in kernels.items() if "pair_kernel" in k}
+    assert len(pair) == 2, sorted(kernels)
+    for k, v in pair.items():
+        assert v["ScratchSize"] == 0 and v["VGPRs"] <= 72 and v["Occupancy"] >= 7, (k, v)
     for k, v in kernels.items():                       # the other kernels: no scratch either
         assert v["ScratchSize"] == 0, (k, v)
