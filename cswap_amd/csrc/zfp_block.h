@@ -871,6 +871,7 @@ CSWAP_HD void pair_code16(const uint64_t (&x)[16], Enc& enc, uint64_t& acc, bool
 {
 #pragma unroll
   for (int k = 15; k >= 0; k--) {
+    if (!CSWAP_ANY(enc.active())) continue;  // every block of the wavefront is out of budget: nothing more is written
     if ((k & 1) == (H == 0 ? 1 : 0)) {
       if (top && k >= 12) enc.leading_plane(x[k]);
       else enc.plane(x[k]);
