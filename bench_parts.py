@@ -247,7 +247,8 @@ def _swap_rows(res, eng, step, params, min_bytes, reps):
                       "swapped_MB": round(st["bytes_in"] / 1e6, 1), "link_MB": round(st["bytes_out"] / 1e6, 1),
                       "shared": st["shared"], "by_policy": dict(st.get("by_policy", {})),
                       "prefetched": st.get("prefetched", 0), "resident": st.get("resident", 0),
-                      "kept_no_room": st.get("kept_no_room", 0), "memo_hits": st.get("memo_hits", 0)}
+                      "kept_no_room": st.get("kept_no_room", 0), "memo_hits": st.get("memo_hits", 0),
+                      "memo_sparse": st.get("memo_sparse", 0)}
 
 
 def bench_training_step(dev, batch: int = 128, image: int = 64, min_bytes: int = 8 << 20) -> dict:
