@@ -14,7 +14,7 @@ Before the W warm-up steps the same step runs, untimed, for CLOCK_SETTLE_S
 seconds: after an idle gap the GPU needs about 25 ms of continuous work to
 return to its steady clocks, and a training loop never leaves it idle.
 
-The last line of stdout is ONE short JSON object (under 1500 characters) that
+The last line of stdout is ONE short JSON object (cut to 1480 characters if need be: fit_line) that
 also carries
   roofline      HBM-roofline figures of the dominant (slower) ZFP kernel, from
                 HIP-event timing of that kernel inside the timed region (events
@@ -191,8 +191,8 @@ def main():
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "fp32", "data": "synthetic",
-        "config": {"workload": "config5 attention probabilities fp32 [32,12,512,512] = softmax(N(0,1)), "
-                               "zfp field nx=512 ny=512 nz=384, rate 8, compress then decompress",
+        "config": {"workload": "config5 attention probabilities fp32 [32,12,512,512]=softmax(N(0,1)), "
+                               "field 512x512x384, rate 8, compress then decompress",
                    "bytes_in": 4 * n},
         "roofline": roofline,
     }
@@ -215,7 +215,30 @@ def main():
             result["extra_file"] = os.path.relpath(args.extra_file, ROOT)
         except OSError as err:      # a read-only tree: the figures above are still printed
             print(f"bench.py: could not write {args.extra_file}: {err}", file=sys.stderr)
-    print(json.dumps(result))
+    print(fit_line(result))
+
+
+LINE_LIMIT = 1480   # characters; the driver keeps a 2000-character tail of stdout
+
+
+def fit_line(result, limit=LINE_LIMIT):
+    """The result as one JSON line of at most `limit` characters.  What does not fit goes,
+    least important first: the name of the file with the rest of the figures when it is a
+    long path, then the entries of `also` from its end; the contract's own keys always stay.
+    (Everything dropped here is still in that file.)"""
+    line = json.dumps(result)
+    if len(line) <= limit:
+        return line
+    result = dict(result)
+    if len(str(result.get("extra_file", ""))) > 40:
+        result["extra_file"] = os.path.basename(result["extra_file"])
+    also = dict(result.get("also") or {})
+    while len(json.dumps(result)) > limit and also:
+        also.popitem()
+        result["also"] = also
+    if not also:
+        result.pop("also", None)
+    return json.dumps(result)
 
 
 def zfp_cold_pair(torch, api, t, rate, copies, reps):
@@ -322,7 +345,10 @@ def headline_fractions(ex):
         # largest compressed / raw latency ratio among the tensors the selector compressed (target: below 1)
         also["swap_c4_ms"] = {"raw": sw["total_none_ms"], "auto": sw["total_auto_ms"],
                               "memo": sw["total_remembered_ms"], "worst_vs_raw": sw["worst_compressed_over_raw"]}
-    return {k: v for k, v in also.items() if v is not None}
+    # most important first: fit_line() drops from the end when the line would get too long
+    order = ["zfp_r8_c1_16MB", "zfp_r8_c3_34MB", "zfp_r8_hidden50MB", "zfp_r8_ffn201MB", "cold", "swap_c4_ms",
+             "zvc_256MiB", "zvc_512MiB", "zvc_c2_50pct", "zfp_r16_attn402MB", "box_copy_GBs", "zvc_256MiB_cpu_GBs"]
+    return {k: also[k] for k in order if also.get(k) is not None}
 
 
 def median(xs):

@@ -30,6 +30,27 @@ def test_defaults_are_one_gpu_and_a_run_of_minutes_at_most():
         assert flag in out.stdout
 
 
+def test_the_line_is_cut_to_its_limit_by_dropping_the_least_important_figures():
+    sys.path.insert(0, ROOT)
+    try:
+        import bench
+    finally:
+        sys.path.remove(ROOT)
+    contract = {"metric": "m" * 70, "value": 1.0, "config": {"workload": "w" * 150}, "roofline": {"frac": 0.5},
+                "cpu_baseline": {"value": 0.2}}
+    also = {f"figure_{i}": [0.123, 0.456] for i in range(60)}
+    full = dict(contract, also=also, extra_file="../" * 20 + "extra.json")
+    line = bench.fit_line(full)
+    assert len(line) <= bench.LINE_LIMIT < 1500
+    r = json.loads(line)
+    assert all(r[k] == v for k, v in contract.items())          # the contract's keys are untouched
+    kept = list(r["also"])
+    assert kept and kept == list(also)[:len(kept)]               # dropped from the end only
+    assert r["extra_file"] == "extra.json"
+    short = dict(contract, also={"a": 1}, extra_file="gpurun_out/bench_extra.json")
+    assert json.loads(bench.fit_line(short)) == short            # a line that fits is left alone
+
+
 def _check_line(r, steps, warmup):
     assert r["n_gpus"] == 1 and r["steps"] == steps and r["warmup"] == warmup
     assert r["unit"] == "GB/s" and r["higher_is_better"] is True and r["vs_baseline"] is None
