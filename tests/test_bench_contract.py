@@ -92,11 +92,18 @@ def test_the_drivers_command_prints_a_short_last_line(tmp_path):
     r = json.loads(last)
     _check_line(r, 20, 5)
     assert "extra" not in r and r["also"]
-    assert r["also"]["box_copy_GBs"] > 1000                  # what a plain device copy reaches on this box
-    assert len(r["also"]["zvc_256MiB_cpu_GBs"]) == 2         # the CPU sparse path beside the ZVC figures
-    for pair in r["also"].values():
-        vals = pair.values() if isinstance(pair, dict) else (pair if isinstance(pair, list) else [pair])
-        assert all(v > 0 for v in vals)
+    def numbers(v):
+        if isinstance(v, dict):
+            v = list(v.values())
+        return [x for item in v for x in numbers(item)] if isinstance(v, list) else [v]
+
+    assert all(x > 0 for x in numbers(r["also"]))
+    # the small-field, cold-cache and swap figures are the first to be kept when the line is cut
+    assert {"zfp_r8_c1_16MB", "cold", "swap_c4_ms"} <= set(r["also"])
+    assert len(r["also"]["cold"]["attn402MB"]) == 2 and r["also"]["swap_c4_ms"]["worst_vs_raw"] > 0
     full = json.loads(extra.read_text())
+    assert full["also"]["box_copy_GBs"] > 1000               # what a plain device copy reaches on this box
+    assert len(full["also"]["zvc_256MiB_cpu_GBs"]) == 2      # the CPU sparse path beside the ZVC figures
+    assert set(r["also"]) <= set(full["also"])               # what the line dropped is still in the file
     assert full["value"] == r["value"] and "zvc_relu_512MiB" in full["extra"] and "swap" in full["extra"]
     assert full["extra"]["zvc_relu_256MiB"]["cpu_baseline"]["all_cores"]["cores"] >= 1
