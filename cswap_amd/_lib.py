@@ -130,6 +130,7 @@ _SIGNATURES = {
     "cswap_swap_release": (i32, [vp, i32]),
     "cswap_swap_info": (i32, [vp, i32, C.POINTER(TicketInfo)]),
     "cswap_swap_timing": (i32, [vp, i32, C.POINTER(TicketTiming)]),
+    "cswap_engine_set_zfp_maxbits": (i32, [vp, C.c_uint]),
     "cswap_engine_probe_count": (C.c_ulonglong, [vp]),
     "cswap_engine_calibrate": (i32, [vp, C.POINTER(Costs)]),
     "cswap_engine_copy_stream": (vp, [vp]),

@@ -102,6 +102,7 @@ struct Ticket {
   int state = kFree;
   int policy = CSWAP_POLICY_NONE;
   int process = 0;  // ZVC chunk count this tensor was compacted with
+  unsigned maxbits = 0;  // ZFP bits per block this tensor was (or would be) coded with: the engine's rate at its swap-out
   size_t n = 0, nnz = 0, nx = 0, ny = 0, nz = 0;
   size_t bytes_out = 0;
   size_t host_off = 0, host_bytes = 0;
@@ -487,7 +488,7 @@ static int reserve_blocks(cswap_engine* e, Ticket& t, int requested)
   }
   if (t.policy == CSWAP_POLICY_SPARSE || t.policy == CSWAP_POLICY_ZFP) {
     t.bytes_out = t.policy == CSWAP_POLICY_SPARSE ? zvc_header_bytes((int)t.n, t.process) + 4 * t.nnz
-                                                  : cswap_zfp_stream_capacity(t.nx, t.ny, t.nz, e->maxbits);
+                                                  : cswap_zfp_stream_capacity(t.nx, t.ny, t.nz, t.maxbits);
     size_t off;
     if (alloc_reclaiming(e, e->dpool, t.bytes_out, &off)) {
       t.dev_off = off; t.dev_bytes = t.bytes_out; t.dev_held = true;
@@ -530,7 +531,7 @@ static int compress_tensor(cswap_engine* e, Ticket& t, const float* d_in, hipStr
     *src = base;
   } else if (t.policy == CSWAP_POLICY_ZFP) {
     uint64_t* d_stream = (uint64_t*)(e->d_base + t.dev_off);
-    rc = cswap_zfp_compress_f32(d_in, t.nx, t.ny, t.nz, 0, 0, 0, e->maxbits, d_stream, compute);
+    rc = cswap_zfp_compress_f32(d_in, t.nx, t.ny, t.nz, 0, 0, 0, t.maxbits, d_stream, compute);
     *src = d_stream;
   } else {
     *src = d_in;
@@ -587,6 +588,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   for (double& u : t.us) u = -1.0;
   t.seq = e->next_seq++;
   t.process = zvc_ok ? process_for(e, n) : 0;
+  t.maxbits = e->maxbits;
   if (e->timing) CSWAP_HIP_TRY(hipEventRecord(t.ev_start[kPhaseCompress], compute));
   cswap_costs costs = e->costs;  // the selector prices the ZVC header with this tensor's chunk count
   if (t.process) costs.process = t.process;
@@ -598,7 +600,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     // best conceivable ZVC outcome (all zeros) is modelled to beat the raw swap,
     // the raw swap it is.
     cswap_choice best_case;
-    if ((rc = cswap_select_field(nx, ny, nz, 0, e->maxbits, &costs, &best_case))) return rc;
+    if ((rc = cswap_select_field(nx, ny, nz, 0, t.maxbits, &costs, &best_case))) return rc;
     if (best_case.policy == CSWAP_POLICY_NONE) {
       t.policy = CSWAP_POLICY_NONE;
       want_probe = false;
@@ -614,7 +616,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
     if (rc < 0) return rc;
     if (rc == 0 && policy == CSWAP_POLICY_AUTO) {
       cswap_choice ch;
-      if ((rc = cswap_select_field(nx, ny, nz, t.nnz, e->maxbits, &costs, &ch))) { drop_device(e, t); return rc; }
+      if ((rc = cswap_select_field(nx, ny, nz, t.nnz, t.maxbits, &costs, &ch))) { drop_device(e, t); return rc; }
       t.policy = ch.policy;
       want_probe = false;  // the count is known
       if (ch.policy != CSWAP_POLICY_SPARSE) {
@@ -650,7 +652,7 @@ extern "C" int cswap_swap_out(cswap_engine* e, const float* d_in, size_t nx, siz
   if (t.policy == CSWAP_POLICY_AUTO) {
     cswap_choice ch;
     if (!t.probe_held) costs.sparse_max_ratio = 0.0;  // no chunk counts to compact with: ZVC is not an option
-    if ((rc = cswap_select_field(nx, ny, nz, t.nnz, e->maxbits, &costs, &ch))) { drop_device(e, t); return rc; }
+    if ((rc = cswap_select_field(nx, ny, nz, t.nnz, t.maxbits, &costs, &ch))) { drop_device(e, t); return rc; }
     t.policy = ch.policy;
   }
 
@@ -811,7 +813,7 @@ extern "C" int cswap_swap_in(cswap_engine* e, int ticket, float* d_out, cswap_st
     rc = cswap_zvc_expand((const float*)(base + hdr), (const uint32_t*)(base + 4 * (size_t)t->process),
                           (const int*)base, (int)t->n, t->process, d_out, compute);
   } else if (t->policy == CSWAP_POLICY_ZFP) {
-    rc = cswap_zfp_decompress_f32((const uint64_t*)src, t->nx, t->ny, t->nz, 0, 0, 0, e->maxbits, d_out, compute);
+    rc = cswap_zfp_decompress_f32((const uint64_t*)src, t->nx, t->ny, t->nz, 0, 0, 0, t->maxbits, d_out, compute);
   }
   err = hipEventRecord(t->ev_done, compute);
   t->state = kInInFlight;  // (from the staging block: out_pending stays up, the outbound copy may still run)
@@ -850,6 +852,14 @@ extern "C" int cswap_swap_info(cswap_engine* e, int ticket, cswap_ticket_info* i
   info->bytes_out = t->bytes_out;
   // to the caller a released ticket is free, and a payload that a prefetch found still staged is prefetched
   info->state = t->state == kReleasing ? (int)kFree : (t->state == kOutInFlight && t->keep_staged ? (int)kPrefetched : t->state);
+  return CSWAP_OK;
+}
+
+extern "C" int cswap_engine_set_zfp_maxbits(cswap_engine* e, unsigned maxbits)
+{
+  if (!e || maxbits < 16 || maxbits > 4096) return CSWAP_E_ARG;
+  std::lock_guard<std::mutex> lock(e->mu);
+  e->maxbits = maxbits;  // tickets in flight keep the rate they went out with
   return CSWAP_OK;
 }
 

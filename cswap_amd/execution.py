@@ -42,6 +42,10 @@ class Execution:
     def init(self) -> None:
         self.index = -1
 
+    def setRatio(self, ratio: int) -> None:  # noqa: N802 (the reference's name, CSWAP+/Execution.h:63)
+        """4 * ratio bits per 4x4x4 block for the ZFP swap-outs from now on (128: a quarter of fp32)."""
+        self.engine.set_maxbits(4 * int(ratio))
+
     def preforward(self) -> None:
         self.init()
         self._dropped.clear()

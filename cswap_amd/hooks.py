@@ -20,6 +20,7 @@ from . import swap
 from ._lib import CswapError
 
 E_NOMEM = -4   # CSWAP_E_NOMEM
+KEEP = 0       # the reference's policy code for "stays on the device" (only with ``only``)
 
 
 class _Handle:
@@ -83,14 +84,26 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
     round trip, CSWAP+/Execution.h:92 has the same one); the k-th swapped tensor of
     an iteration is the same activation every time, so its decision is remembered
     under (k, element count).  A remembered "ZFP" or "raw" is passed to the engine
-    as an explicit policy and costs no probe; "ZVC" needs the non-zero count anyway
-    and is probed as before.  After ``recheck`` uses an entry is probed again, so a
-    layer whose sparsity drifts is noticed."""
+    as an explicit policy and costs no probe; a remembered "ZVC" goes in as
+    ``AUTO_SPARSE``: the one-kernel compaction runs first and its count is the
+    selector's probe, so the choice is confirmed every time.  After ``recheck`` uses
+    a ZFP or raw entry is probed again, so a layer whose sparsity drifts is noticed.
+
+    ``only``: when set to a tensor, nothing but that tensor (the same contiguous
+    bytes) is swapped while the hooks are active.  Other eligible tensors saved in
+    the meantime (a ReLU saves its output, which is the next layer's input) are
+    held as they are and remembered: ``swap_named`` swaps such a tensor out later,
+    for every node that saved it, once the caller says how.  ``policy`` and
+    ``only`` may be changed between two activations of the same context, which is
+    how the per-layer calls of ``cswap_amd.torch_names`` drive one context per
+    iteration."""
 
     def __init__(self, engine: "swap.SwapEngine", policy: int = swap.AUTO, min_bytes: int = 1 << 20,
-                 prefetch: int = 2, depth: int = 2, memo: dict | None = None, recheck: int = 16):
+                 prefetch: int = 2, depth: int = 2, memo: dict | None = None, recheck: int = 16,
+                 only: torch.Tensor | None = None):
         self.engine = engine
         self.policy = policy
+        self.only = only
         self.min_bytes = min_bytes
         self.prefetch = prefetch
         self.depth = max(1, depth)
@@ -116,19 +129,47 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
             h.keep = None
             self._live.pop(h.key, None)
 
+    @staticmethod
+    def _key(t: torch.Tensor):
+        return (t.data_ptr(), t.numel(), t._version)
+
+    def _eligible(self, t: torch.Tensor) -> bool:
+        return (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.dim() >= 1
+                and t.numel() * 4 >= self.min_bytes and not isinstance(t, torch.nn.Parameter)
+                and not t.is_leaf)
+
     def _pack(self, t: torch.Tensor):
-        eligible = (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.dim() >= 1
-                    and t.numel() * 4 >= self.min_bytes and not isinstance(t, torch.nn.Parameter)
-                    and not t.is_leaf)
-        if not eligible:
+        if not self._eligible(t):
             self.stats["kept"] += 1
             return t
-        key = (t.data_ptr(), t.numel(), t._version)
+        key = self._key(t)
         h = self._live.get(key)
         if h is not None:                # same tensor saved by another node: one swap serves both
             h.refs += 1
             self.stats["shared"] += 1
             return _Ref(h, tuple(t.shape))
+        if self.only is not None and (self.policy == KEEP or not (t.data_ptr() == self.only.data_ptr()
+                                                                  and t.numel() == self.only.numel())):
+            # not the tensor this activation is for (or that one is to stay): held as it is, until
+            # swap_named says otherwise
+            h = _Handle(None, tuple(t.shape), t, key, False)
+            self._live[key] = h
+            self.stats["held"] = self.stats.get("held", 0) + 1
+            return _Ref(h, tuple(t.shape))
+        h = _Handle(None, tuple(t.shape), t, key, False)
+        return _Ref(h, tuple(t.shape)) if self._swap_out(t, h) else t
+
+    def swap_named(self, t: torch.Tensor) -> bool:
+        """Swaps out, with the current ``policy``, a tensor that was saved and held while the hooks
+        were active for another one.  False if ``t`` is not such a tensor (nobody has saved it yet:
+        the pack hook will see it) or could not go out."""
+        h = self._live.get(self._key(t)) if self._eligible(t) else None
+        if h is None or h.ticket is not None or self.policy == KEEP:
+            return False
+        return self._swap_out(t, h)
+
+    def _swap_out(self, t: torch.Tensor, h) -> bool:
+        """Starts the swap-out of t for handle h (which holds t); False if it has to stay on the device."""
         self._settle(self.depth - 1)
         self._drain()
         policy, slot = self.policy, (self._position, t.numel())
@@ -156,7 +197,7 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
             if err.code != E_NOMEM:
                 raise
             self.stats["kept_no_room"] = self.stats.get("kept_no_room", 0) + 1
-            return t                     # pinned pool, staging pool or tickets exhausted: the tensor stays on the device
+            return False                 # pinned pool, staging pool or tickets exhausted: the tensor stays on the device
         info = self.engine.info(ticket)
         if self.memo is not None and policy in (swap.AUTO, swap.AUTO_SPARSE):
             self.memo[slot] = (info.policy, 0)
@@ -166,11 +207,12 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
         by = self.stats.setdefault("by_policy", {})
         name = {swap.NONE: "raw", swap.SPARSE: "zvc", swap.ZFP: "zfp"}.get(info.policy, str(info.policy))
         by[name] = by.get(name, 0) + 1
-        h = _Handle(ticket, tuple(t.shape), t, key, info.policy == swap.NONE)   # keeps the device copy alive for now
+        h.ticket = ticket
+        h.raw = info.policy == swap.NONE     # h.keep holds the device copy alive for now
         self._pending.append(h)
-        self._live[key] = h
+        self._live[h.key] = h
         self._order.append(h)
-        return _Ref(h, tuple(t.shape))
+        return True
 
     # -- backward side
     def _drain(self):
@@ -188,6 +230,13 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
             h.refs -= 1
             if h.refs <= 0:
                 h.out = None
+            return out.view(ref.shape)
+        if h.ticket is None:             # held, and never named for a swap: it is where it was
+            out = h.keep.detach()
+            h.refs -= 1
+            if h.refs <= 0:
+                h.keep = None
+                self._live.pop(h.key, None)
             return out.view(ref.shape)
         self._drain()
         if h.keep is not None:           # still on the device: its outbound copy was one of the last in flight
@@ -239,3 +288,6 @@ class swap_saved_tensors(torch.autograd.graph.saved_tensors_hooks):
                 self.engine.release(h.ticket)
                 self._released.add(h.ticket)
         self._order.clear()
+        for h in self._live.values():      # held and never swapped
+            h.keep = None
+        self._live.clear()

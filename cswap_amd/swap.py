@@ -72,6 +72,11 @@ class SwapEngine:
         check(lib().cswap_engine_calibrate(self._h, C.byref(c)), "cswap_engine_calibrate")
         return c
 
+    def set_maxbits(self, maxbits: int) -> None:
+        """ZFP bits per 4x4x4 block for the swap-outs from now on (setRatio: CSWAP+/Execution.h:63;
+        tensors already out come back with the rate they went out with)."""
+        check(lib().cswap_engine_set_zfp_maxbits(self._h, maxbits), "cswap_engine_set_zfp_maxbits")
+
     # Execution::pre
     def pre(self, t: torch.Tensor, policy: int = AUTO) -> int:
         if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()):

@@ -46,6 +46,9 @@ class Execution {
     for (int i = 0; i < n; i++) begin_stage[(size_t)i] = i + 1;
   }
   void init() { index = -1; }
+  // setRatio (Execution.h:63, called again from the training loop): 4 * ratio bits per 4x4x4
+  // block for the ZFP swap-outs from now on; 128 = a quarter of the fp32 size.
+  int setRatio(int ratio) { return ratio > 0 ? cswap_engine_set_zfp_maxbits(engine_, 4u * (unsigned)ratio) : CSWAP_E_ARG; }
   // also forgets what the previous iteration dropped (the caller recomputed it)
   void preforward()
   {

@@ -403,6 +403,14 @@ int cswap_swap_info(cswap_engine* e, int ticket, cswap_ticket_info* info);
 /* Phase times of a ticket so far (see cswap_ticket_timing); does not wait for anything.
  * CSWAP_E_UNSUPPORTED on an engine created without config.timing. */
 int cswap_swap_timing(cswap_engine* e, int ticket, cswap_ticket_timing* out);
+/* The ZFP rate (bits per 4x4x4 block, 16..4096) of the swap-outs from now on;
+ * config.zfp_maxbits until it is called.  Replaces setRatio(int) called from the
+ * training loop (CSWAP+/Execution.h:63; CIFAR10/cifar10.py:106 sets it every
+ * epoch): maxbits = 4 * ratio.  A ticket keeps the rate it was swapped out with,
+ * so tensors that are on the host or in flight come back correctly whatever is
+ * set in between.  (The cost model's ZFP throughput figures stay those of the
+ * rate the engine was calibrated with.) */
+int cswap_engine_set_zfp_maxbits(cswap_engine* e, unsigned maxbits);
 /* Number of probes so far: counting passes followed by the host round trip for
  * the non-zero count (the one at Execution.h:92), which a selector-driven or ZVC
  * swap-out pays and an explicit raw or ZFP request does not. */

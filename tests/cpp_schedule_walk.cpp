@@ -60,6 +60,7 @@ int main()
   int time_ = 0;
   cswap::Execution exe(eng);
   exe.init_(n_ops);
+  CS_OK(exe.setRatio(128));  // as Execution::init_ does (Execution.h:63): 8 bits per value
   exe.policy = pm.make_policy(time_, n_ops);
   if (exe.policy.size() != (size_t)n_ops || !pm.summary().target_met) { printf("no plan\n"); return 4; }
   exe.begin_stage = pm.begin_stage();
