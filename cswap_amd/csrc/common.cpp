@@ -1,7 +1,22 @@
 // common.cpp -- error strings and ABI version
 #include "common.h"
 
+#include <atomic>
+
 namespace cswap {
+int device_compute_units()
+{
+  static std::atomic<int> cus[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  int v = cus[dev].load(std::memory_order_relaxed);
+  if (!v) {
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cus[dev].store(v, std::memory_order_relaxed);
+  }
+  return v;
+}
+
 int& last_hip_error()
 {
   static thread_local int e = 0;

@@ -14,6 +14,9 @@ inline int hip_fail(hipError_t e)
   return CSWAP_E_HIP;
 }
 
+// compute units of the current device (0 if the query fails), looked up once per device
+int device_compute_units();
+
 // to be called right after a kernel launch: picks up launch-configuration errors
 inline int check_launch()
 {

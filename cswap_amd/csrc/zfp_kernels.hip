@@ -42,7 +42,7 @@ constexpr unsigned long long kReadOnceBytes = CSWAP_READ_ONCE_BYTES;
 #define CSWAP_PAIR_ENCODE_BYTES (40ull << 20)
 #endif
 #ifndef CSWAP_PAIR_DECODE_BYTES
-#define CSWAP_PAIR_DECODE_BYTES 0ull
+#define CSWAP_PAIR_DECODE_BYTES (40ull << 20)   // and only from 16 bits per value on (kPairDecodeFromBits)
 #endif
 
 // 16 bytes of the field as the compiler's own vector type (what the nontemporal builtins take)
@@ -1015,6 +1015,22 @@ static bool pair_shape(const Field3& fd, unsigned maxbits)
 
 static std::atomic<unsigned long long> g_pair_decode_bytes{CSWAP_PAIR_DECODE_BYTES};
 
+// The pair form pays while all of a field's workgroups are on the chip at once (twice the
+// wavefronts, each with half the serial work); a field that needs a second round of them is
+// faster with one lane per block.  How many workgroups a compute unit holds is set by their
+// LDS: measured, 88 % of what its 160 KB divided by the workgroup's bytes allows.  A limit of
+// SIZE_MAX takes the form for every field it can code (tests, measurements).
+static bool pair_fits(unsigned grid, size_t lds_bytes, unsigned long long limit)
+{
+  if (limit == ~0ull) return true;
+  const double per_cu = 0.88 * 160.0 * 1024.0 / (double)lds_bytes;
+  return (double)grid <= per_cu * (double)device_compute_units();
+}
+// The decoder's pair form gains nothing at 8 bits per value (the plane loop, which one half
+// runs alone, is 60 % of its time) and 3-7 % from 16 bits per value on, where the shared back
+// end weighs more.
+constexpr unsigned kPairDecodeFromBits = 1024;
+
 extern "C" void cswap_zfp_set_pair_bytes(size_t encode_below, size_t decode_below, size_t* previous)
 {
   const size_t e = (size_t)g_pair_encode_bytes.exchange(encode_below, std::memory_order_relaxed);
@@ -1049,8 +1065,9 @@ static int compress3(const void* d_in, Elem elem, size_t nx, size_t ny, size_t n
   hipStream_t st = (hipStream_t)stream;
   const bool whole = (maxbits & 63u) == 0;
   const bool is_int = elem == kI32 || elem == kI64;
-  if (elem == kF32 && pair_shape(fd, maxbits) &&
-      (unsigned long long)nx * ny * nz * 4ull < g_pair_encode_bytes.load(std::memory_order_relaxed)) {
+  const unsigned long long pair_below = g_pair_encode_bytes.load(std::memory_order_relaxed);
+  if (elem == kF32 && pair_shape(fd, maxbits) && (unsigned long long)nx * ny * nz * 4ull < pair_below &&
+      pair_fits(grid, (size_t)pair_lds_dwords(maxbits) * 4, pair_below)) {
     hipLaunchKernelGGL(zfp_encode3_f32_pair_kernel, dim3(grid), dim3(128), (size_t)pair_lds_dwords(maxbits) * 4, st,
                        static_cast<const float*>(d_in), fd, maxbits, d_stream);
     return check_launch();
@@ -1098,8 +1115,10 @@ static int decompress3(const uint64_t* d_stream, Elem elem, size_t nx, size_t ny
   hipStream_t st = (hipStream_t)stream;
   const bool whole = (maxbits & 63u) == 0;
   const bool is_int = elem == kI32 || elem == kI64;
-  if (elem == kF32 && pair_shape(fd, maxbits) &&
-      (unsigned long long)nx * ny * nz * 4ull < g_pair_decode_bytes.load(std::memory_order_relaxed)) {
+  const unsigned long long pair_below = g_pair_decode_bytes.load(std::memory_order_relaxed);
+  if (elem == kF32 && pair_shape(fd, maxbits) && (unsigned long long)nx * ny * nz * 4ull < pair_below &&
+      (maxbits >= kPairDecodeFromBits || pair_below == ~0ull) &&
+      pair_fits(grid, (size_t)pair_dec_lds_dwords(maxbits) * 4, pair_below)) {
     hipLaunchKernelGGL(zfp_decode3_f32_pair_kernel, dim3(grid), dim3(128), (size_t)pair_dec_lds_dwords(maxbits) * 4, st,
                        d_stream, fd, maxbits, static_cast<float*>(d_out));
     return check_launch();

@@ -1289,20 +1289,6 @@ extern "C" void cswap_zvc_debug_set_lookback(unsigned spin_limit, unsigned skip_
   g_skip_first.store(skip_first);
 }
 
-// compute units of the current device (0 if the query fails), looked up once per device
-static int device_compute_units()
-{
-  static int cus[64];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-  if (!cus[dev]) {
-    int v = 0;
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-    cus[dev] = v;
-  }
-  return cus[dev];
-}
-
 static int status_words(int process);
 // Tensors of at least this many bytes take the single pass in cswap_zvc_compress_fused; smaller ones
 // finish sooner with the three kernels (a few rounds of the grid do not fill the pipeline).

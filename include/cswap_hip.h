@@ -115,7 +115,11 @@ int cswap_zfp_decompress_i64_nd(const uint64_t* d_stream, int dims, size_t nx, s
  * instead -- two wavefronts share 64 blocks, each doing half of every phase -- where the
  * shape allows it: extents that are multiples of 4, contiguous 16-byte aligned rows, a
  * 16-byte aligned stream, maxbits a multiple of 256.  Same stream, same values.
- * 0 = never, SIZE_MAX = whenever the shape allows.  `previous`, if not NULL, receives
+ * Below the limit the form is taken while all of the field's workgroups fit on the chip
+ * at once (their LDS decides how many do: about 37 MB at 8 bits per value, 30 MB at 16,
+ * 21 MB at 32), and by the decoder only from 16 bits per value on (at 8 it measured no
+ * gain).  0 = never; SIZE_MAX = whenever the shape allows, whatever the size and rate
+ * (tests and measurements).  Defaults: 40 MiB both.  `previous`, if not NULL, receives
  * the two values that were in force.  Process-wide. */
 void cswap_zfp_set_pair_bytes(size_t encode_below, size_t decode_below, size_t* previous);
 
